@@ -1,0 +1,151 @@
+/*
+ * libmustafar_hip.so -- C ABI of the MI355X (gfx950) sparse-KV decode-attention kernels.
+ *
+ * Conventions for every entry point
+ *   - all data pointers are DEVICE pointers; `stream` is a hipStream_t passed as void*
+ *     (NULL = the default stream); launches are asynchronous, nothing here synchronises;
+ *   - fp16 buffers are IEEE binary16 (`mstf_half` = raw 16-bit pattern);
+ *   - inputs are borrowed and never modified; outputs are caller-allocated;
+ *   - nothing allocates: scratch memory comes in through `workspace` (size from the
+ *     matching *_workspace_bytes query, 256-byte aligned);
+ *   - the return value is MSTF_OK or a negative MSTF_E* code (never an exception);
+ *     mstf_strerror() names it; a failed launch also records the HIP error, readable
+ *     with mstf_last_hip_error().
+ *
+ * Compressed fp16 format ("bitmap format"), per KV head b (D = head_dim, tiles of 64 elements):
+ *   key   tile t = tokblk*D + ch            : 64 consecutive tokens of channel ch
+ *   value tile t = tokblk*D + half*64 + tok : 64 consecutive channels of one token
+ *   bmp[b][t]  bit (63-i) set  <=>  element i of the tile is non-zero
+ *   idx[b][t]  start of the tile's packed values, in 4-byte units, relative to the head's base;
+ *              idx[b][T] = total; every tile is padded with +0.0 to a multiple of 8 values
+ *   nz_off[b]  base of head b inside the flat nz buffer, in 16-byte units
+ * This is the layout defined by the reference producer kernel/compression.py:8-435 and
+ * consumed by kernel/csrc/SpMM_Kernel.cuh:49-211.
+ */
+#ifndef MUSTAFAR_HIP_H
+#define MUSTAFAR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t mstf_half;
+
+enum {
+    MSTF_OK = 0,
+    MSTF_EINVAL = -1,       /* null pointer, non-positive size, inconsistent arguments */
+    MSTF_EALIGN = -2,       /* a pointer is not aligned as required */
+    MSTF_EUNSUPPORTED = -3, /* shape outside what the kernels cover (e.g. head_dim != 128) */
+    MSTF_EWORKSPACE = -4,   /* workspace missing or too small */
+    MSTF_ELAUNCH = -5       /* HIP reported an error at launch; see mstf_last_hip_error() */
+};
+
+const char* mstf_strerror(int code);
+int mstf_last_hip_error(void);
+/* library version: major*10000 + minor*100 + patch */
+int mstf_version(void);
+
+/* ------------------------------------------------------------------ pruning (A1)
+ * Replaces dh_prune_key / dh_prune_value (models/llama_mustafar_kernel.py:194-274):
+ * per row of D values, thr = kth-th smallest |x|, keep |x| >= thr, pruned entries become
+ * +0/-0 by sign (the result of x * mask).  x, y: [rows, D]; y may alias x.  D must be 128. */
+int mstf_prune_rows_f16(void* stream, const mstf_half* x, mstf_half* y, int64_t rows, int D, int kth);
+
+/* ------------------------------------------------------------------ compression (C1, C2)
+ * Replace convert_key_batched / convert_value_batched (kernel/compression.py:249-342, 344-435)
+ * fused with the pruning above.
+ *   x [B, M, N] fp16, M % 64 == 0, N == 128.
+ *   kth > 0: prune each row first (as mstf_prune_rows_f16) without writing the dense result;
+ *   kth == 0: x is already pruned, zeros are the holes (exactly what the reference converts).
+ * Phase 1 ("count") writes bmp [B,T], idx [B,T+1], nz_off [B] and *total_halfs (device uint64:
+ * number of fp16 values the flat nz buffer must hold).  Phase 2 ("scatter") fills nz.
+ * mstf_compress_*_f16 runs both; with nz == NULL it runs phase 1 only.  Tiles whose values
+ * would not fit in nz_capacity_halfs are not written (compare *total_halfs afterwards). */
+size_t mstf_compress_workspace_bytes(int B, int M, int N);
+int mstf_compress_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
+                          uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz,
+                          uint64_t nz_capacity_halfs, void* workspace, size_t workspace_bytes);
+int mstf_compress_value_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
+                            uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz,
+                            uint64_t nz_capacity_halfs, void* workspace, size_t workspace_bytes);
+/* Phase 2 alone, on the outputs of a finished phase 1 (same x, B, M, N). */
+int mstf_scatter_key_f16(void* stream, const mstf_half* x, int B, int M, int N, const uint64_t* bmp,
+                         const uint32_t* idx, const uint32_t* nz_off, mstf_half* nz, uint64_t nz_capacity_halfs);
+int mstf_scatter_value_f16(void* stream, const mstf_half* x, int B, int M, int N, const uint64_t* bmp,
+                           const uint32_t* idx, const uint32_t* nz_off, mstf_half* nz, uint64_t nz_capacity_halfs);
+
+/* ------------------------------------------------------------------ key SpMV (K1)
+ * Replaces mustafar_key_formulation (kernel/kernel_wrapper/mustafar_wrapper.cu:19-133 ->
+ * Key_SplitK_API, kernel/csrc/SpMM_API.cu:179 -> Key_Kernel, kernel/csrc/SpMM_Kernel.cuh:240-520):
+ *   C[bq, n, m] = sum_d Ktilde[bq / groups][m, d] * Bm[bq, n, d]      (fp32 accumulate, fp16 result)
+ * Bm [Bq, n_rows, K] fp16, C [Bq, n_rows, M] fp16.  M = compressed tokens (M % 64 == 0),
+ * K = head_dim (128), Bq = query heads x batch, groups = query heads per KV head.
+ * n_rows = 8 reproduces the reference operator (its N is hard-wired to 8, mustafar_wrapper.cu:125);
+ * n_rows = 1 is the decode fast path without the 7 padding rows.
+ * Every compressed byte is read once per KV head, not once per query head. */
+int mstf_key_spmv_f16(void* stream, const uint64_t* bmp, const mstf_half* nz, const uint32_t* idx,
+                      const uint32_t* nz_off, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq, int groups,
+                      int n_rows);
+
+/* ------------------------------------------------------------------ value SpMV (V1)
+ * Replaces mustafar_value_formulation (mustafar_wrapper.cu:139-263 -> Value_SplitK_API,
+ * SpMM_API.cu:331 -> Value_Kernel, SpMM_Kernel.cuh:535-796 + SplitK_Reduction, Reduction_Kernel.cuh:26-48):
+ *   C[bq, n, d] = sum_t Vtilde[bq / groups][t, d] * P[bq, n, t]
+ * P [Bq, n_rows, K] fp16, C [Bq, n_rows, M] fp16.  M = head_dim (128), K = compressed tokens.
+ * Tokens are split over workgroups; fp32 partial sums go through `workspace`. */
+size_t mstf_value_spmv_workspace_bytes(int M, int K, int Bq, int groups, int n_rows);
+int mstf_value_spmv_f16(void* stream, const uint64_t* bmp, const mstf_half* nz, const uint32_t* idx,
+                        const uint32_t* nz_off, const mstf_half* P, mstf_half* C, int M, int K, int Bq, int groups,
+                        int n_rows, void* workspace, size_t workspace_bytes);
+
+/* ------------------------------------------------------------------ scale + softmax (S1)
+ * The glue between the two products (models/llama_mustafar_kernel.py:405,425):
+ *   w = fp16(s / sqrt(head_dim));  p = fp16(softmax_fp32(w))   over each row of length L.
+ * s, p: [rows, L] fp16 with row strides (in elements) s_stride / p_stride; p may alias s. */
+int mstf_scale_softmax_f16(void* stream, const mstf_half* s, mstf_half* p, int64_t rows, int L, int64_t s_stride,
+                           int64_t p_stride, int head_dim);
+
+/* ------------------------------------------------------------------ quantised format (Q1-Q4)
+ * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),
+ * with the bit width a parameter (the reference hard-codes 2).  Same tiles and bitmaps as above;
+ *   counts[B,T] raw non-zeros; units[B,T] = ceil(count / capacity), capacity = 32 / bit;
+ *   tile_off[B,T] GLOBAL 4-byte-word offset of the tile inside `packed`;
+ *   scales/zeros[B,T] fp16: scale = (max - min) / (2^bit - 1) (1 when 0 or empty),
+ *   zero = floor(-min / scale + 0.5); code = clamp(floor(v / scale + 0.5) + zero, 0, 2^bit - 1);
+ *   code j of a tile sits at bits bit*(j % capacity) of word j / capacity.
+ * kth as in mstf_compress_*_f16.  packed == NULL runs the sizing phase only. */
+size_t mstf_compress_quant_workspace_bytes(int B, int M, int N);
+int mstf_compress_key_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit, uint64_t* bmp,
+                            uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,
+                            mstf_half* zeros, uint64_t* total_words, uint32_t* packed, uint64_t packed_capacity_words,
+                            void* workspace, size_t workspace_bytes);
+int mstf_compress_value_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit, uint64_t* bmp,
+                              uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,
+                              mstf_half* zeros, uint64_t* total_words, uint32_t* packed,
+                              uint64_t packed_capacity_words, void* workspace, size_t workspace_bytes);
+
+/* Consumers: mustafar_key_formulation_quant[_meta] (kernel_quant/kernel_wrapper/mustafar_wrapper_quant.cu:14-214
+ * -> Key_Kernel_Quant, kernel_quant/csrc/SpMM_Kernel_Quant.cuh:273-503) and
+ * mustafar_value_formulation_quant[_decode_n1] (mustafar_wrapper_quant.cu:216-457 -> Value_Kernel_Quant,
+ * SpMM_Kernel_Quant.cuh:510-735).  Same products as the fp16 entry points on the dequantised
+ * matrix (q - zero) * scale; dequant_mode 0 = fp32 arithmetic rounded once to fp16, 1 = fp16
+ * arithmetic (SpMM_Kernel_Quant.cuh:190-191,238-240).  counts/units may be NULL (derived from the
+ * bitmaps, as the non-_meta key entry point does).  bit in {2, 4}; capacity must equal 32 / bit. */
+int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                        const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
+                        const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq, int groups,
+                        int n_rows, int bit, int capacity, int dequant_mode);
+size_t mstf_value_spmv_quant_workspace_bytes(int M, int K, int Bq, int groups, int n_rows);
+int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                          const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
+                          const mstf_half* zeros, const mstf_half* P, mstf_half* C, int M, int K, int Bq, int groups,
+                          int n_rows, int bit, int capacity, int dequant_mode, void* workspace,
+                          size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MUSTAFAR_HIP_H */

@@ -1,0 +1,182 @@
+// Device helpers shared by the fp16 and the quantised compressors: the padded LDS slab of one
+// (KV head, 64-token block) unit, the per-row radix select and the tile bitmaps.
+#pragma once
+#include "common.hpp"
+
+namespace mstf {
+
+constexpr int kD = 128;                  // head_dim the slab layout is built for
+constexpr int kRowDw = kD / 2 + 1;       // dwords per LDS row: 64 of data + 1 of padding
+constexpr int kSlabDw = 64 * kRowDw;     // 16640 bytes
+
+typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ us2_t as_us2(uint32_t x) { return __builtin_bit_cast(us2_t, x); }
+__device__ __forceinline__ uint32_t us2_u32(us2_t x) { return __builtin_bit_cast(uint32_t, x); }
+
+// Streams rows [row0, row0+64) of a [rows, 128] fp16 matrix into the padded LDS slab.
+// Rows >= rows_valid are filled with zeros.
+__device__ __forceinline__ void slab_load(const _Float16* x, int64_t row0, int64_t rows_valid, uint32_t* slab,
+                                          int lane)
+{
+    const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD);
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const int e = j * 64 + lane;  // 16-byte piece index inside the slab
+        const int row = e >> 4, c16 = e & 15;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + row < rows_valid) v = src[e];
+        uint32_t* d = slab + row * kRowDw + c16 * 4;
+        d[0] = v.x;
+        d[1] = v.y;
+        d[2] = v.z;
+        d[3] = v.w;
+    }
+}
+
+// kth-th smallest (1-based) of the 128 fp16 magnitudes of this lane's row.
+// mag[j] holds two 15-bit magnitudes.  Greedy MSB-first: the answer is the largest c with
+// #(mag < c) < kth.  (mag - c) wraps above 0x7FFF exactly when mag < c, so bit 15 of the packed
+// 16-bit difference is the comparison result.
+__device__ __forceinline__ uint32_t select_kth(const uint32_t (&mag)[64], int kth)
+{
+    uint32_t thr = 0;
+#pragma unroll 1
+    for (int bit = 14; bit >= 0; bit--) {
+        const uint32_t cand = thr | (1u << bit);
+        const us2_t c2 = as_us2(cand | (cand << 16));
+        us2_t cnt = as_us2(0u);
+#pragma unroll
+        for (int j = 0; j < 64; j++) cnt += (as_us2(mag[j]) - c2) >> (unsigned short)15;
+        const uint32_t below = (uint32_t)cnt.x + (uint32_t)cnt.y;
+        if (below < (uint32_t)kth) thr = cand;
+    }
+    return thr;
+}
+
+__device__ __forceinline__ uint32_t wave_excl_scan(uint32_t v, int lane, uint32_t& total)
+{
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        uint32_t t = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += t;
+    }
+    total = __shfl(inc, 63, 64);
+    return inc - v;
+}
+
+__device__ __forceinline__ uint32_t padded_units(uint64_t bm)
+{
+    return (uint32_t)((__popcll(bm) + 7) & ~7) >> 1;  // 4-byte units: nnz padded to 8 halfs
+}
+
+
+// Keep decision of one unit, as tile bitmaps (MSB-first).  Lane l returns the bitmaps of tiles
+// l (bmA) and 64+l (bmB) of the unit:
+//   key   : tile c = channel c over the 64 tokens        (ballot across lane = token)
+//   value : tile (half, token) with lane = token         (packed inside the lane)
+// mag[j] = magnitudes of channels 2j (low half) and 2j+1 (high half) of this lane's token;
+// an element is kept when its magnitude is >= thr (thr >= 1, so zeros never are).
+template <bool IS_VALUE>
+__device__ __forceinline__ void unit_bitmaps(const uint32_t (&mag)[64], uint32_t thr, int lane, uint64_t& bmA,
+                                             uint64_t& bmB)
+{
+    const us2_t t2 = as_us2(thr | (thr << 16));
+    if (!IS_VALUE) {
+        bmA = 0;
+        bmB = 0;
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            const uint32_t d = us2_u32(as_us2(mag[j]) - t2);  // bit 15 / 31 set <=> pruned
+            const uint64_t k0 = __builtin_bitreverse64(__ballot((d & 0x8000u) == 0u));
+            const uint64_t k1 = __builtin_bitreverse64(__ballot((d & 0x80000000u) == 0u));
+            const int c0 = 2 * j, c1 = 2 * j + 1;
+            if (c0 < 64) {
+                bmA = (lane == c0) ? k0 : bmA;
+                bmA = (lane == c1) ? k1 : bmA;
+            } else {
+                bmB = (lane == c0 - 64) ? k0 : bmB;
+                bmB = (lane == c1 - 64) ? k1 : bmB;
+            }
+        }
+    } else {
+        uint32_t w[4] = {0u, 0u, 0u, 0u};  // [half0 hi, half0 lo, half1 hi, half1 lo]
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            const uint32_t d = us2_u32(as_us2(mag[j]) - t2);
+            const uint32_t two = (((d >> 15) & 1u) << 1 | (d >> 31)) ^ 3u;  // [kept(2j), kept(2j+1)] MSB-first
+            const int jj = j & 15;                                        // pair index inside a 32-channel word
+            w[j >> 4] |= two << (30 - 2 * jj);
+        }
+        bmA = u64_of(w[1], w[0]);
+        bmB = u64_of(w[3], w[2]);
+    }
+}
+
+// Loads this lane's row magnitudes from the slab and returns the keep threshold
+// (kth == 0: input already pruned, keep the non-zeros).
+__device__ __forceinline__ uint32_t row_threshold(const uint32_t* slab, int lane, int kth, uint32_t (&mag)[64])
+{
+#pragma unroll
+    for (int j = 0; j < 64; j++) mag[j] = slab[lane * kRowDw + j] & 0x7FFF7FFFu;
+    uint32_t thr = 1u;
+    if (kth > 0) {
+        thr = select_kth(mag, kth);
+        if (thr == 0u) thr = 1u;  // zeros are never stored
+    }
+    return thr;
+}
+
+// Exclusive scan of per-head totals over one workgroup of 1024 threads; out[b] = sum of earlier
+// totals >> shift, *total = (sum of all) * total_mul.
+__device__ __forceinline__ void heads_scan(const uint32_t* head_tot, uint32_t* out, uint64_t* total, int B, int shift,
+                                           uint64_t total_mul)
+{
+    __shared__ uint64_t wsum[16];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per = (B + 1023) / 1024;
+    const int i0 = tid * per;
+    uint64_t mine = 0;
+    for (int i = i0; i < i0 + per && i < B; i++) mine += head_tot[i];
+    uint64_t inc = mine;
+    for (int o = 1; o < 64; o <<= 1) {
+        uint64_t t = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += t;
+    }
+    if (lane == 63) wsum[wave] = inc;
+    __syncthreads();
+    uint64_t pre = 0;
+    for (int w = 0; w < wave; w++) pre += wsum[w];
+    uint64_t run = pre + inc - mine;
+    for (int i = i0; i < i0 + per && i < B; i++) {
+        out[i] = (uint32_t)(run >> shift);
+        run += head_tot[i];
+    }
+    if (tid == 1023) *total = total_mul * run;
+}
+
+// Exclusive scan of one head's unit totals (grid.x = head, 256 threads) into LDS `base`
+// (nblk entries); returns the head total to every thread.
+__device__ __forceinline__ uint32_t units_scan(const uint32_t* ut, uint32_t* base, int nblk)
+{
+    __shared__ uint32_t carry_sh[4];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t carry = 0;
+    for (int s = 0; s < nblk; s += 256) {
+        const int i = s + tid;
+        const uint32_t v = i < nblk ? ut[i] : 0u;
+        uint32_t wtot;
+        const uint32_t e = wave_excl_scan(v, lane, wtot);
+        __syncthreads();
+        if (lane == 0) carry_sh[wave] = wtot;
+        __syncthreads();
+        uint32_t pre = carry;
+        for (int w = 0; w < wave; w++) pre += carry_sh[w];
+        if (i < nblk) base[i] = pre + e;
+        carry += carry_sh[0] + carry_sh[1] + carry_sh[2] + carry_sh[3];
+    }
+    __syncthreads();
+    return carry;
+}
+
+}  // namespace mstf

@@ -1,0 +1,141 @@
+"""Zero-copy device path: fused prune+compress into a flat cache, SpMVs with one row per head.
+
+Everything stays on the device; the only host synchronisation is the optional read-back of the
+packed size when the caller did not provide a capacity.
+"""
+import math
+
+import torch
+
+from ._lib import check, lib
+
+_WS = {}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def workspace(device, nbytes):
+    """A per-device scratch tensor that only grows (256-byte aligned by the caching allocator)."""
+    key = (device.type, device.index)
+    t = _WS.get(key)
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _WS[key] = t
+    return t
+
+
+def kth_from_sparsity(sparsity, head_dim):
+    """Rank of the pruning threshold: max(1, int(target_sparsity * D)) as in dh_prune_key."""
+    return max(1, int(sparsity * head_dim))
+
+
+class CompressedKV:
+    """One side (K or V) of the compressed cache, flat on the device.
+
+    bmp int64 [B, T], idx int32 [B, T+1], nz fp16 flat, nz_off int32 [B] (16-byte units)."""
+
+    def __init__(self, bmp, idx, nz, nz_off, tokens, head_dim, is_value, total_halfs=None):
+        self.bmp, self.idx, self.nz, self.nz_off = bmp, idx, nz, nz_off
+        self.tokens, self.head_dim, self.is_value = tokens, head_dim, is_value
+        self.total_halfs = total_halfs
+
+    @property
+    def heads(self):
+        return self.bmp.shape[0]
+
+    def packed(self):
+        """The used part of the flat value buffer (needs the host-side size)."""
+        return self.nz[:int(self.total_halfs)]
+
+    def nbytes(self):
+        """Algorithmic size: bitmaps + offsets + packed values actually used."""
+        used = self.nz.numel() if self.total_halfs is None else int(self.total_halfs)
+        return self.bmp.numel() * 8 + self.idx.numel() * 4 + used * 2
+
+
+def prune_rows(x, kth, out=None):
+    """dh_prune_key / dh_prune_value on the last axis (D = 128)."""
+    assert x.is_cuda and x.dtype == torch.float16 and x.is_contiguous()
+    D = x.shape[-1]
+    y = torch.empty_like(x) if out is None else out
+    check(lib().mstf_prune_rows_f16(_stream(), x.data_ptr(), y.data_ptr(), x.numel() // D, D, int(kth)),
+          "mstf_prune_rows_f16")
+    return y
+
+
+def compress(x, is_value, kth=0, capacity_halfs=None):
+    """Prune (kth > 0) and compress x [B, M, N] into the bitmap format.
+
+    With capacity_halfs=None the packed size is read back once (like the reference's .item());
+    with a capacity the call is fully asynchronous and `total_halfs` stays on the device."""
+    assert x.is_cuda and x.dtype == torch.float16 and x.dim() == 3
+    x = x.contiguous()
+    B, M, N = x.shape
+    T = M * N // 64
+    dev = x.device
+    L = lib()
+    bmp = torch.empty((B, T), dtype=torch.int64, device=dev)
+    idx = torch.empty((B, T + 1), dtype=torch.int32, device=dev)
+    nz_off = torch.empty((B,), dtype=torch.int32, device=dev)
+    total = torch.empty((1,), dtype=torch.int64, device=dev)
+    wsb = L.mstf_compress_workspace_bytes(B, M, N)
+    ws = workspace(dev, wsb)
+    fn = L.mstf_compress_value_f16 if is_value else L.mstf_compress_key_f16
+    name = "mstf_compress_value_f16" if is_value else "mstf_compress_key_f16"
+    if capacity_halfs is None:
+        check(fn(_stream(), x.data_ptr(), B, M, N, int(kth), bmp.data_ptr(), idx.data_ptr(), nz_off.data_ptr(),
+                 total.data_ptr(), None, 0, ws.data_ptr(), ws.numel()), name)
+        n = int(total.item())
+        nz = torch.empty((max(n, 8),), dtype=torch.float16, device=dev)
+        sc = L.mstf_scatter_value_f16 if is_value else L.mstf_scatter_key_f16
+        check(sc(_stream(), x.data_ptr(), B, M, N, bmp.data_ptr(), idx.data_ptr(), nz_off.data_ptr(), nz.data_ptr(),
+                 n), name.replace("compress", "scatter"))
+        if n == 0:
+            nz.zero_()
+        return CompressedKV(bmp, idx, nz if n == 0 else nz[:n], nz_off, M, N, is_value, n)
+    nz = torch.empty((int(capacity_halfs),), dtype=torch.float16, device=dev)
+    check(fn(_stream(), x.data_ptr(), B, M, N, int(kth), bmp.data_ptr(), idx.data_ptr(), nz_off.data_ptr(),
+             total.data_ptr(), nz.data_ptr(), int(capacity_halfs), ws.data_ptr(), ws.numel()), name)
+    return CompressedKV(bmp, idx, nz, nz_off, M, N, is_value, total)
+
+
+def key_spmv(ck, q, groups, n_rows=1, out=None):
+    """scores[bq, n, t] = sum_d K[bq // groups][t, d] * q[bq, n, d]   (unscaled).  q: [Bq, n_rows, D]."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    Bq = q.numel() // (n_rows * ck.head_dim)
+    C = torch.empty((Bq, n_rows, ck.tokens), dtype=torch.float16, device=q.device) if out is None else out
+    check(lib().mstf_key_spmv_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
+                                  ck.nz_off.data_ptr(), q.data_ptr(), C.data_ptr(), ck.tokens, ck.head_dim, Bq,
+                                  groups, n_rows), "mstf_key_spmv_f16")
+    return C
+
+
+def value_spmv(cv, p, groups, n_rows=1, out=None):
+    """out[bq, n, d] = sum_t V[bq // groups][t, d] * p[bq, n, t].  p: [Bq, n_rows, Lc]."""
+    assert p.dtype == torch.float16 and p.is_contiguous()
+    Bq = p.numel() // (n_rows * cv.tokens)
+    L = lib()
+    C = torch.empty((Bq, n_rows, cv.head_dim), dtype=torch.float16, device=p.device) if out is None else out
+    wsb = L.mstf_value_spmv_workspace_bytes(cv.head_dim, cv.tokens, Bq, groups, n_rows)
+    ws = workspace(p.device, wsb)
+    check(L.mstf_value_spmv_f16(_stream(), cv.bmp.data_ptr(), cv.nz.data_ptr(), cv.idx.data_ptr(),
+                                cv.nz_off.data_ptr(), p.data_ptr(), C.data_ptr(), cv.head_dim, cv.tokens, Bq, groups,
+                                n_rows, ws.data_ptr(), ws.numel()), "mstf_value_spmv_f16")
+    return C
+
+
+def scale_softmax(s, head_dim, out=None):
+    """softmax(s / sqrt(head_dim), dtype=float32).to(float16) over the last axis."""
+    assert s.dtype == torch.float16 and s.stride(-1) == 1
+    L = s.shape[-1]
+    s2 = s.reshape(-1, L)
+    p = torch.empty_like(s2) if out is None else out.reshape(-1, L)
+    check(lib().mstf_scale_softmax_f16(_stream(), s2.data_ptr(), p.data_ptr(), s2.shape[0], L, s2.stride(0),
+                                       p.stride(0), int(head_dim)), "mstf_scale_softmax_f16")
+    return p.reshape(s.shape)
+
+
+def sqrt_head_dim(head_dim):
+    return math.sqrt(head_dim)
