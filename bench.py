@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Headline benchmark: sparse decode attention of one Llama-3-8B layer on one MI355X.
+
+Workload (BASELINE.json configs[1]): batch 8, 32 query / 8 KV heads, head_dim 128, 4096 cached
+tokens, per-token magnitude pruning at 70 % on K and V, fp16.  A step is one decode-attention
+pass for one new token: key SpMV -> scale+softmax -> value SpMV over the compressed cache.
+Several distinct caches are rotated between steps so that reads come from HBM, not from the
+256 MB Infinity Cache.  Prints exactly one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def make_kv(torch, dev, Bkv, L, D, gen):
+    """fp16 N(0,1) K and V; K gets 4 outlier channels per head scaled x10."""
+    K = torch.randn((Bkv, L, D), generator=gen, device=dev, dtype=torch.float32)
+    V = torch.randn((Bkv, L, D), generator=gen, device=dev, dtype=torch.float32)
+    ch = torch.stack([torch.randperm(D, generator=gen, device=dev)[:4] for _ in range(Bkv)])
+    scale = torch.ones((Bkv, 1, D), device=dev)
+    scale.scatter_(2, ch.view(Bkv, 1, 4), 10.0)
+    return (K * scale).half(), V.half()
+
+
+def event_time_us(torch, fn, iters):
+    """Average duration of fn() over `iters` back-to-back launches, HIP events on the launch stream."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters
+
+
+def cpu_baseline(args, bs, nkv, groups, L, D, kth):
+    """The oracle's dense masked attention (prune -> q.K^T -> /sqrt(d) -> fp32 softmax -> P.V) on the
+    host cores, on a bounded sample: the full layer shape at a reduced batch."""
+    import numpy as np
+    from oracle import oracle as orc
+    sample_bs = max(1, min(bs, args.cpu_batch))
+    Bkv = sample_bs * nkv
+    K, V = orc.make_kv(1234, Bkv, L, D)
+    q = np.random.default_rng(5).standard_normal((Bkv * groups, D)).astype(np.float16)
+    t0 = time.perf_counter()
+    Kp, Vp = orc.prune_rows(K, kth), orc.prune_rows(V, kth)
+    t_prune = time.perf_counter() - t0
+    orc.dense_masked_attention(q, Kp, Vp, groups)  # warm-up
+    reps, t_att = 0, 0.0
+    while reps < 3 or (t_att < 10.0 and reps < 50):
+        t0 = time.perf_counter()
+        orc.dense_masked_attention(q, Kp, Vp, groups)
+        t_att += time.perf_counter() - t0
+        reps += 1
+    per_layer_us = t_att / reps * 1e6 * (bs / sample_bs)
+    return {
+        "value": round(per_layer_us, 1),
+        "unit": "us/layer",
+        "cores": orc.num_threads(),
+        "kind": "port",
+        "sample": "oracle dense masked decode attention, batch %d of %d (x%d heads, ctx %d), %d timed runs, "
+                  "scaled to the full batch; pruning of that sample took %.2f s once (single thread)"
+                  % (sample_bs, bs, nkv * groups, L, reps, t_prune),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sparsity", type=float, default=0.7)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--ctx", type=int, default=4096)
+    ap.add_argument("--caches", type=int, default=6, help="distinct compressed caches rotated between steps")
+    ap.add_argument("--cpu-batch", type=int, default=2, help="batch entries in the CPU-baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one GPU "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from mustafar_amd import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    bs, nq, nkv, D, L = args.batch, 32, 8, 128, args.ctx
+    groups = nq // nkv
+    Bkv, Bq = bs * nkv, bs * nq
+    kth = ops.kth_from_sparsity(args.sparsity, D)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(20260312)
+
+    # ---- build the rotating compressed caches (also times the fused prune+compress kernels)
+    caches = []
+    t_ck = t_cv = 0.0
+    for i in range(args.caches):
+        K, V = make_kv(torch, dev, Bkv, L, D, gen)
+        cap = K.numel()
+        if i == 0:
+            ops.compress(K, False, kth=kth, capacity_halfs=cap)  # warm-up (module load)
+        t_ck += event_time_us(torch, lambda: caches.append([ops.compress(K, False, kth=kth, capacity_halfs=cap)]), 1)
+        t_cv += event_time_us(torch, lambda: caches[-1].append(ops.compress(V, True, kth=kth, capacity_halfs=cap)), 1)
+        del K, V
+    t_ck /= args.caches
+    t_cv /= args.caches
+    kbytes = caches[0][0].bmp.numel() * 8 + caches[0][0].idx.numel() * 4 + int(caches[0][0].total_halfs.item()) * 2
+    vbytes = caches[0][1].bmp.numel() * 8 + caches[0][1].idx.numel() * 4 + int(caches[0][1].total_halfs.item()) * 2
+
+    q = torch.randn((Bq, 1, D), generator=gen, device=dev, dtype=torch.float32).half()
+    s = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
+    p = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
+    o = torch.empty((Bq, 1, D), dtype=torch.float16, device=dev)
+    it = [0]
+
+    def step():
+        ck, cv = caches[it[0] % args.caches]
+        it[0] += 1
+        ops.key_spmv(ck, q, groups, out=s)
+        ops.scale_softmax(s, D, out=p)
+        ops.value_spmv(cv, p, groups, out=o)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
+
+    # ---- per-kernel averages over back-to-back launches on rotating caches (HIP events)
+    def key_only():
+        ck = caches[it[0] % args.caches][0]
+        it[0] += 1
+        ops.key_spmv(ck, q, groups, out=s)
+
+    def value_only():
+        cv = caches[it[0] % args.caches][1]
+        it[0] += 1
+        ops.value_spmv(cv, p, groups, out=o)
+
+    n = max(args.steps, 50)
+    key_us = event_time_us(torch, key_only, n)
+    val_us = event_time_us(torch, value_only, n)
+    sm_us = event_time_us(torch, lambda: ops.scale_softmax(s, D, out=p), n)
+
+    # algorithmic bytes per launch: compressed side read once per KV head + weights in + result out (one row per head)
+    key_alg = kbytes + Bq * D * 2 + Bq * L * 2
+    val_alg = vbytes + Bq * L * 2 + Bq * D * 2
+    if val_us >= key_us:
+        dom, dom_us, dom_bytes = "value_spmv_kernel", val_us, val_alg
+    else:
+        dom, dom_us, dom_bytes = "key_spmv_kernel", key_us, key_alg
+    achieved = dom_bytes / dom_us / 1e3  # GB/s
+
+    out = {
+        "metric": "sparse decode-attn us/layer (Llama-3-8B shape, bs=%d, ctx=%d, %d%% K/V sparsity)"
+                  % (bs, L, round(args.sparsity * 100)),
+        "value": round(wall_us, 2),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_us / 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: Llama-3-8B GQA decode-attention layer, batch %d, 32 query / 8 KV heads, "
+                        "head_dim 128, %d cached tokens, per-token magnitude pruning %.0f%% on K and V, one new token; "
+                        "step = key SpMV + scale/softmax + value SpMV; %d caches rotated (cold HBM reads)"
+                        % (bs, L, args.sparsity * 100, args.caches),
+            "compressed_bytes_per_token_per_kv_head": {"key": round(kbytes / Bkv / L, 2),
+                                                       "value": round(vbytes / Bkv / L, 2)},
+        },
+        "tokens_per_s": round(bs / (wall_us * 1e-6), 1),
+        "stages_us": {"key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
+                      "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
+        "hbm_gbs_on_compressed_bytes": {"key_spmv": round(key_alg / key_us / 1e3, 1),
+                                        "value_spmv": round(val_alg / val_us / 1e3, 1),
+                                        "decode_attn": round((key_alg + val_alg) / wall_us / 1e3, 1)},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": int(dom_bytes), "avg_launch_us": round(dom_us, 2)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args, bs, nkv, groups, L, D, kth)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
