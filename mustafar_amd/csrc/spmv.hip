@@ -1,96 +1,218 @@
 // Batched key / value SpMV over the bitmap format, and the scale+softmax glue between them.
 //
-// Both products share one inner loop.  A "chunk" is 64 consecutive tiles of one KV head:
-//   key   chunk = 64 channels x 64 tokens of one token block      (lane = token)
-//   value chunk = 64 tokens  x 64 channels of one half of head_dim (lane = channel)
-// In both cases tile t of the chunk contributes  D[t][lane] * w[n][t]  to accumulator n of the
-// lane, where D[t][lane] is element `lane` of tile t (0 when its bitmap bit is clear) and w is
-// the query row (key) or the probability row (value).  A wavefront owns a chunk: it streams the
-// chunk's packed values (contiguous, 16-byte aligned) from HBM into its private LDS buffer with
-// 16-byte loads, then rebuilds D[t][lane] with a popcount rank (v_mbcnt) per tile and feeds
-// pairs of tiles to v_dot2_f32_f16 with the two weights in one scalar register.  Bitmaps, tile
-// offsets and weights are wave-uniform and come through scalar loads.
+// Both products share one inner loop over runs of consecutive tiles of one KV head:
+//   key   : 64 tokens of one token block, tiles = channels       (lane = token)
+//   value : 64 channels of one half of head_dim, tiles = tokens   (lane = channel)
+// In both cases tile t contributes  D[t][lane] * w[n][t]  to accumulator n of the lane, where
+// D[t][lane] is element `lane` of tile t (0 when its bitmap bit is clear) and w is the query row
+// (key) or the probability row (value).  A wavefront streams the packed values of 32 tiles at a
+// time (contiguous, 16-byte aligned) from HBM straight into its private LDS double buffer
+// (global_load_lds, 16 bytes per lane), rebuilds D[t][lane] with a popcount rank (v_mbcnt) per
+// tile and feeds groups of four tiles to v_mfma_f32_4x4x4f16, which multiplies them with the weights of
+// four accumulators (the GQA query group) at once, so the products cost no vector-ALU issue slots.
+// Bitmaps and tile offsets are wave-uniform and come through scalar loads; weights are staged in
+// LDS by the same LDS-direct loads.
 #include "common.hpp"
 
 namespace mstf {
 
-constexpr int kChunkBytes = 64 * 64 * 2;       // worst case: 64 full tiles
-constexpr int kWaveLds = kChunkBytes + 16;     // + a 16-byte zero slot read by lanes whose bit is clear
+#ifndef MSTF_SUB_TILES
+#define MSTF_SUB_TILES 32
+#endif
+constexpr int kSubTiles = MSTF_SUB_TILES;      // tiles per staged piece ("sub-chunk"): 16 or 32
+constexpr int kSubBytes = kSubTiles * 64 * 2;  // worst case: every tile full
+constexpr int kOffsLds = kSubTiles * 4;          // per-tile value offsets of the sub-chunk being decompressed
+constexpr int kNzLds = 2 * kSubBytes + 16 + kOffsLds;  // value double buffer + zero slot (lanes whose bit is clear) + offsets
 
-struct ChunkRegs {
-    uint4 r[8];
-};
+#define MSTF_GLOBAL __attribute__((address_space(1)))
 
-// Per-lane 16-byte pieces of a chunk: piece i of lane l is bytes [(i*64+l)*16, +16).
-__device__ __forceinline__ void chunk_fetch(ChunkRegs& cr, const char* src, uint32_t bytes, int lane)
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ h4_t as_h4(uint32_t lo, uint32_t hi)
+{
+    const u32x2_t v = {lo, hi};
+    return __builtin_bit_cast(h4_t, v);
+}
+
+__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// LDS-direct loads: data goes from global memory straight into LDS without passing through
+// registers; lane l of the instruction writes `size` bytes at dst + l*size.  Completion is
+// tracked by vmcnt only, the caller waits with wait_vm0() before reading the LDS.
+__device__ __forceinline__ void dma16(const void* src, void* dst_wave_uniform)
+{
+    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void* src, void* dst_wave_uniform)
+{
+    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 4, 0, 0);
+}
+
+// Streams `bytes` (a multiple of 16, <= kSubBytes) into LDS: piece i of lane l lands at dst + (i*64 + l)*16.
+__device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char* dst, int lane)
 {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < kSubBytes / 1024; i++) {
         if ((uint32_t)(i * 1024) < bytes) {
-            uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
-            if (o < bytes) cr.r[i] = *reinterpret_cast<const uint4*>(src + o);
+            const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+            if (o < bytes) dma16(src + o, dst + i * 1024);
         }
     }
 }
-__device__ __forceinline__ void chunk_stage(const ChunkRegs& cr, char* dst, uint32_t bytes, int lane)
+
+// lanes whose bit of the wave-uniform mask m is set take `yes`, the others `no`.  Written as one
+// v_cndmask on the mask register pair so the compiler keeps the decompression straight-line
+// (it otherwise turns the select into an exec-masked branch per tile).
+__device__ __forceinline__ uint32_t select_lane(uint64_t m, uint32_t yes, uint32_t no)
 {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        if ((uint32_t)(i * 1024) < bytes) {
-            uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
-            if (o < bytes) *reinterpret_cast<uint4*>(dst + o) = cr.r[i];
-        }
-    }
+    uint32_t r;
+    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(m));
+    return r;
 }
 
-// acc[n] += sum_t D[t][lane] * w[n][t] for the 64 tiles of one chunk.
-//   bm, ix : the chunk's 64 bitmaps / 64 tile offsets (4-byte units), wave-uniform pointers
-//   sbase  : LDS byte address of the staged chunk minus 4*ix[0]
-//   zaddr  : LDS byte address of two zero bytes
-//   w      : weights of accumulator 0 for tile 0 (fp16), wstride halfs between accumulators
-template <int NW>
-__device__ __forceinline__ void chunk_accumulate(const uint64_t* bm, const uint32_t* ix, uint32_t sbase,
-                                                 uint32_t zaddr, const _Float16* w, size_t wstride, float (&acc)[NW])
+// Packed pair (D[t][lane], D[t+1][lane]) of two tiles as fp16x2.
+//   m0, m1 : tile bitmaps, MSB-first (wave-uniform, scalar registers)
+//   o0, o1 : offsets of the tiles' values inside the staged buffer, fp16 units (wave-uniform, vector registers)
+//   buf    : LDS byte address of the staged buffer;  zaddr: LDS address of two zero bytes
+// rank = offset + popcount(mask below lane) comes from v_mbcnt with the offset as its addend;
+// lanes whose element is absent read the zero slot.  (16-bit LDS loads cannot merge into one
+// register here: with SRAM ECC they clear the other half, hence the explicit pack.)
+__device__ __forceinline__ uint32_t tile_pair(uint32_t m0lo, uint32_t m0hi, uint32_t m1lo, uint32_t m1hi, uint32_t o0,
+                                              uint32_t o1, uint32_t buf, uint32_t zaddr)
 {
-#pragma unroll 1
-    for (int tt = 0; tt < 64; tt += 8) {
-        const u32x16_t mv = *reinterpret_cast<const u32x16_a4*>(bm + tt);
-        const u32x8_t iv = *reinterpret_cast<const u32x8_a4*>(ix + tt);
-        uint32_t v[4];
+    const uint64_t m0 = lanes_of(u64_of(m0lo, m0hi));
+    const uint64_t m1 = lanes_of(u64_of(m1lo, m1hi));
+    const uint32_t r0 = __builtin_amdgcn_mbcnt_hi((uint32_t)(m0 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m0, o0));
+    const uint32_t r1 = __builtin_amdgcn_mbcnt_hi((uint32_t)(m1 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m1, o1));
+    const uint32_t a0 = select_lane(m0, r0 * 2u + buf, zaddr);
+    const uint32_t a1 = select_lane(m1, r1 * 2u + buf, zaddr);
+    h2_t p;
+    p.x = lds_load_h(a0);
+    p.y = lds_load_h(a1);
+    return as_u32(p);
+}
+
+// One staged sub-chunk (kSubTiles tiles).  For every group of 4 tiles the lane builds its own four
+// values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator
+// (lane & 3) of each accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in
+// lane 4b+j, the sums of positions 4b..4b+3 for accumulator 4m+j:
+//     acc[m][r] += sum_t D[t][4b + r] * w[4m + j][t]
+//   bm     : the sub-chunk's bitmaps (wave-uniform pointer; one batch of scalar loads)
+//   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
+//   offs   : LDS byte address of the per-tile offsets (fp16 units, relative to buf)
+//   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
+template <int NM>
+__device__ __forceinline__ void sub_accumulate(const uint64_t* bm, uint32_t buf, uint32_t zaddr, uint32_t offs,
+                                               uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
+{
+    u32x16_t mvs[kSubTiles / 8];
 #pragma unroll
-        for (int u = 0; u < 8; u += 2) {
-            const uint64_t m0 = lanes_of(u64_of(mv[2 * u], mv[2 * u + 1]));
-            const uint64_t m1 = lanes_of(u64_of(mv[2 * u + 2], mv[2 * u + 3]));
-            const uint32_t o0 = iv[u] * 4u + sbase;
-            const uint32_t o1 = iv[u + 1] * 4u + sbase;
-            const uint32_t a0 = lane_bit(m0) ? (o0 + rank_below(m0) * 2u) : zaddr;
-            const uint32_t a1 = lane_bit(m1) ? (o1 + rank_below(m1) * 2u) : zaddr;
-            h2_t p;
-            p.x = lds_load_h(a0);
-            p.y = lds_load_h(a1);
-            v[u / 2] = as_u32(p);
-        }
+    for (int g = 0; g < kSubTiles / 8; g++) mvs[g] = *reinterpret_cast<const u32x16_a4*>(bm + 8 * g);
 #pragma unroll
-        for (int n = 0; n < NW; n++) {
-            const u32x4_t q = *reinterpret_cast<const u32x4_a4*>(w + (size_t)n * wstride + tt);
+    for (int g = 0; g < kSubTiles / 8; g++) {
+        const u32x16_t mv = mvs[g];
+        const int tt = g * 8;
+        // the same address in every lane: the LDS unit broadcasts the offsets of the 8 tiles
+        const u32x4_t oa = *(MSTF_LDS const u32x4_t*)(uintptr_t)(offs + (uint32_t)tt * 4u);
+        const u32x4_t ob = *(MSTF_LDS const u32x4_t*)(uintptr_t)(offs + (uint32_t)tt * 4u + 16u);
+        const uint32_t v0 = tile_pair(mv[0], mv[1], mv[2], mv[3], oa[0], oa[1], buf, zaddr);
+        const uint32_t v1 = tile_pair(mv[4], mv[5], mv[6], mv[7], oa[2], oa[3], buf, zaddr);
+        const uint32_t v2 = tile_pair(mv[8], mv[9], mv[10], mv[11], ob[0], ob[1], buf, zaddr);
+        const uint32_t v3 = tile_pair(mv[12], mv[13], mv[14], mv[15], ob[2], ob[3], buf, zaddr);
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            const u32x4_t q = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup + (uint32_t)tt * 2u);
             const uint32_t q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
-            acc[n] = __builtin_amdgcn_fdot2(as_h2(v[0]), as_h2(q0), acc[n], false);
-            acc[n] = __builtin_amdgcn_fdot2(as_h2(v[1]), as_h2(q1), acc[n], false);
-            acc[n] = __builtin_amdgcn_fdot2(as_h2(v[2]), as_h2(q2), acc[n], false);
-            acc[n] = __builtin_amdgcn_fdot2(as_h2(v[3]), as_h2(q3), acc[n], false);
+            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
+            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
         }
     }
 }
 
-__device__ __forceinline__ uint32_t chunk_bytes(const uint32_t* ix)
+__device__ __forceinline__ uint32_t sub_bytes(uint32_t start, uint32_t end)
 {
-    uint32_t b = (ix[64] - ix[0]) * 4u;
-    return b > (uint32_t)kChunkBytes ? (uint32_t)kChunkBytes : b;  // a well-formed chunk never exceeds this
+    const uint32_t b = (end - start) * 4u;
+    return b > (uint32_t)kSubBytes ? (uint32_t)kSubBytes : b;  // a well-formed sub-chunk never exceeds this
+}
+
+// Each lane l < kSubTiles also loads the bitmap of tile l of the coming sub-chunk with a vector load
+// issued together with the value stream.  That serves two purposes: the popcounts give, through
+// a wave prefix sum, the offset of every tile inside the staged buffer (the format pads each tile
+// to a multiple of 8 values, so offsets follow from the bitmaps and idx is only read once per
+// sub-chunk), and it pulls the bitmap lines into L2 before the scalar loads ask for them.
+__device__ __forceinline__ uint2 bitmap_of_lane(const uint64_t* bm, int lane)
+{
+    uint2 b = make_uint2(0u, 0u);
+    if (lane < kSubTiles) b = *reinterpret_cast<const uint2*>(bm + lane);
+    return b;
+}
+// Waits for every outstanding vector-memory operation (LDS-direct loads included).
+__device__ __forceinline__ void wait_vm0_keep(uint2& b)
+{
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(b.x), "+v"(b.y)::"memory");
+}
+// offs[l] = sum over tiles t < l of the padded value count of tile t (fp16 units), l < kSubTiles.
+__device__ __forceinline__ void write_tile_offsets(uint2 b, char* offs, int lane)
+{
+    const uint32_t cnt = (uint32_t)(__popc(b.x) + __popc(b.y));
+    const uint32_t padded = (cnt + 7u) & ~7u;
+    uint32_t inc = padded;
+#pragma unroll
+    for (int o = 1; o < kSubTiles; o <<= 1) {
+        const uint32_t t = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += t;
+    }
+    if (lane < kSubTiles) reinterpret_cast<uint32_t*>(offs)[lane] = inc - padded;
+}
+
+// Walks `nsubs` sub-chunks of one KV head with a two-deep pipeline: while sub-chunk n is being
+// decompressed out of one LDS buffer, sub-chunk n+1 streams from HBM into the other.
+//   tile_of(n)    : first tile of sub-chunk n
+//   stage_w(n)    : issues the LDS-direct loads of the weights sub-chunk n needs (may be a no-op)
+//   waddr_of(n)   : LDS byte address of w[lane & 3][first tile of sub-chunk n]
+template <int NM, class TileOf, class StageW, class WAddrOf>
+__device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stage_w, WAddrOf waddr_of, uint32_t wgroup,
+                                          const uint64_t* bmk, const uint32_t* ixk, const char* nzk, char* my, int lane,
+                                          f4_t (&acc)[NM])
+{
+    const uint32_t lbase = lds_addr(my);
+    const uint32_t zaddr = lbase + 2 * kSubBytes;
+    char* offs = my + 2 * kSubBytes + 16;
+    if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
+    if (nsubs <= 0) return;
+    size_t t_cur = tile_of(0);
+    const uint32_t s0 = ixk[t_cur];
+    sub_issue(nzk + (size_t)s0 * 4u, sub_bytes(s0, ixk[t_cur + kSubTiles]), my, lane);
+    stage_w(0);
+    uint2 lane_bm = bitmap_of_lane(bmk + t_cur, lane);
+    size_t t_nxt = nsubs > 1 ? tile_of(1) : t_cur;
+    uint32_t s_nxt = ixk[t_nxt], e_nxt = ixk[t_nxt + kSubTiles];
+    for (int n = 0; n < nsubs; n++) {
+        wait_vm0_keep(lane_bm);  // sub-chunk n (values, weights, lane bitmaps) has landed
+        write_tile_offsets(lane_bm, offs, lane);
+        if (n + 1 < nsubs) {
+            sub_issue(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), my + ((n + 1) & 1) * kSubBytes, lane);
+            stage_w(n + 1);
+            lane_bm = bitmap_of_lane(bmk + t_nxt, lane);
+        }
+        const size_t t_now = t_cur;
+        t_cur = t_nxt;
+        if (n + 2 < nsubs) {
+            t_nxt = tile_of(n + 2);
+            s_nxt = ixk[t_nxt];
+            e_nxt = ixk[t_nxt + kSubTiles];
+        }
+        sub_accumulate<NM>(bmk + t_now, lbase + (uint32_t)(n & 1) * kSubBytes, zaddr, lds_addr(offs), waddr_of(n),
+                           wgroup, acc);
+        wait_lgkm0();  // all LDS reads of buffer n&1 and of the offsets are done before they are rewritten
+    }
 }
 
 // ------------------------------------------------------------------------------- key
-// One wavefront per (KV head, token block): loops over the D/64 channel chunks of the block.
-// C[(kv*NW + n)*Lc + token] = sum_d K[token][d] * Bm[(kv*NW + n)*D + d].
+// One wavefront per (KV head, token block): walks the D/32 channel sub-chunks of the block.
+// C[(kv*rows + row0 + n)*Lc + token] = sum_d K[token][d] * Bm[(kv*rows + row0 + n)*D + d],  n < NW.
+// LDS per wavefront: value double buffer + zero slot + tile offsets + the NW query rows (4*NM rows reserved).
 template <int NW>
 __global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restrict__ bmp, const char* __restrict__ nz,
                                                        const uint32_t* __restrict__ idx,
@@ -99,6 +221,9 @@ __global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restric
                                                        int Lc, int D, int nblk, int ntasks, int bm_rows_per_kv,
                                                        int row0)
 {
+    constexpr int NM = (NW + 3) / 4;
+    constexpr int kMaxD = 128;
+    constexpr int kWaveLds = kNzLds + NM * 4 * kMaxD * 2;
     __shared__ __attribute__((aligned(16))) char lds[4][kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
@@ -107,52 +232,65 @@ __global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restric
     const int kv = task / nblk;
     const int tb = task - kv * nblk;
     const size_t T = (size_t)Lc * D / 64;
-    const uint64_t* bmk = bmp + (size_t)kv * T + (size_t)tb * D;
-    const uint32_t* ixk = idx + (size_t)kv * (T + 1) + (size_t)tb * D;
+    const uint64_t* bmk = bmp + (size_t)kv * T;
+    const uint32_t* ixk = idx + (size_t)kv * (T + 1);
     const char* nzk = nz + (size_t)nz_off[kv] * 16u;
-    const _Float16* wk = Bm + ((size_t)kv * bm_rows_per_kv + row0) * D;
+    const char* wsrc = reinterpret_cast<const char*>(Bm + ((size_t)kv * bm_rows_per_kv + row0) * D);
     char* my = lds[wave];
-    const uint32_t lbase = lds_addr(my);
-    const uint32_t zaddr = lbase + kChunkBytes;
-    if (lane < 4) reinterpret_cast<uint32_t*>(my + kChunkBytes)[lane] = 0u;
+    char* wl = my + kNzLds;                       // [4*NM rows][D] fp16; rows >= NW stay unwritten
+    const uint32_t wbytes = (uint32_t)NW * D * 2u;  // the NW rows are contiguous in Bm
 
-    float acc[NW];
+    f4_t acc[NM];
 #pragma unroll
-    for (int n = 0; n < NW; n++) acc[n] = 0.f;
-
-    const int nchunks = D / 64;
-    ChunkRegs cr;
-    uint32_t bytes = chunk_bytes(ixk);
-    chunk_fetch(cr, nzk + (size_t)ixk[0] * 4u, bytes, lane);
-    for (int c = 0; c < nchunks; c++) {
-        const uint32_t* ixc = ixk + c * 64;
-        const uint32_t start = ixc[0];
-        chunk_stage(cr, my, bytes, lane);
-        if (c + 1 < nchunks) {
-            bytes = chunk_bytes(ixc + 64);
-            chunk_fetch(cr, nzk + (size_t)ixc[64] * 4u, bytes, lane);
+    for (int m = 0; m < NM; m++) acc[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const size_t tile0 = (size_t)tb * D;
+    const uint32_t wrow = lds_addr(wl) + (uint32_t)(lane & 3) * (uint32_t)D * 2u;
+    walk_subs<NM>(
+        D / kSubTiles, [=](int n) { return tile0 + (size_t)n * kSubTiles; },
+        [=](int n) {
+            if (n != 0) return;  // the query rows are staged once per task
+#pragma unroll
+            for (int i = 0; i < (NW * kMaxD * 2 + 1023) / 1024; i++) {
+                const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+                if (o < wbytes) dma16(wsrc + o, wl + i * 1024);
+            }
+        },
+        [=](int n) { return wrow + (uint32_t)n * kSubTiles * 2u; }, (uint32_t)D * 8u, bmk, ixk, nzk, my, lane, acc);
+    // lane 4b+j holds tokens 4b..4b+3 of accumulator 4m+j
+    const int j = lane & 3;
+    _Float16* out = C + ((size_t)kv * bm_rows_per_kv + row0) * Lc + (size_t)tb * 64 + (lane & ~3);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        if (4 * m + j < NW) {
+            h4_t o;
+            o[0] = (_Float16)acc[m][0];
+            o[1] = (_Float16)acc[m][1];
+            o[2] = (_Float16)acc[m][2];
+            o[3] = (_Float16)acc[m][3];
+            *reinterpret_cast<h4_t*>(out + (size_t)(4 * m + j) * Lc) = o;
         }
-        __builtin_amdgcn_wave_barrier();
-        chunk_accumulate<NW>(bmk + c * 64, ixc, lbase - start * 4u, zaddr, wk + c * 64, (size_t)D, acc);
-        __builtin_amdgcn_wave_barrier();
     }
-    _Float16* out = C + ((size_t)kv * bm_rows_per_kv + row0) * Lc + (size_t)tb * 64 + lane;
-#pragma unroll
-    for (int n = 0; n < NW; n++) out[(size_t)n * Lc] = (_Float16)acc[n];
 }
 
 // ------------------------------------------------------------------------------- value
 // grid = (token splits, D/64 halves, KV heads); WAVES wavefronts per workgroup, each walking
 // `nbpw` token blocks of its half and keeping fp32 sums per channel; the workgroup then adds
 // its wavefronts' sums through LDS and writes one partial row per accumulator:
-//   nsplit == 1 : C[(kv*NW+n)*D + d]                       (fp16, final)
-//   nsplit  > 1 : part[((kv*NW+n)*nsplit + split)*D + d]   (fp32, merged by value_merge_kernel)
+//   nsplit == 1 : C[(kv*rows+row0+n)*D + d]                       (fp16, final)
+//   nsplit  > 1 : part[((kv*rows+row0+n)*nsplit + split)*D + d]   (fp32, merged by value_merge_kernel)
+// LDS per wavefront: value double buffer + zero slot + tile offsets + double-buffered probability rows
+// (4*NM rows x kSubTiles tokens per sub-chunk).
 template <int NW, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void value_spmv_kernel(
     const uint64_t* __restrict__ bmp, const char* __restrict__ nz, const uint32_t* __restrict__ idx,
     const uint32_t* __restrict__ nz_off, const _Float16* __restrict__ P, _Float16* __restrict__ C,
     float* __restrict__ part, int Lc, int D, int nblk, int nbpw, int nsplit, int p_rows_per_kv, int row0)
 {
+    constexpr int NM = (NW + 3) / 4;
+    constexpr int kWRow = kSubTiles * 2;          // bytes of one probability row per sub-chunk
+    constexpr int kWBuf = NM * 4 * kWRow;         // one weight buffer
+    constexpr int kNeed = kNzLds + 2 * kWBuf;
+    constexpr int kWaveLds = kNeed > NW * 256 ? kNeed : NW * 256;  // the per-wave sums are parked here at the end
     __shared__ __attribute__((aligned(16))) char lds[WAVES][kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
@@ -160,45 +298,46 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_kernel(
     const int half = (int)blockIdx.y;
     const int kv = (int)blockIdx.z;
     const size_t T = (size_t)Lc * D / 64;
-    const uint64_t* bmk = bmp + (size_t)kv * T + (size_t)half * 64;
-    const uint32_t* ixk = idx + (size_t)kv * (T + 1) + (size_t)half * 64;
+    const uint64_t* bmk = bmp + (size_t)kv * T;
+    const uint32_t* ixk = idx + (size_t)kv * (T + 1);
     const char* nzk = nz + (size_t)nz_off[kv] * 16u;
     const _Float16* wk = P + ((size_t)kv * p_rows_per_kv + row0) * Lc;
     char* my = lds[wave];
-    const uint32_t lbase = lds_addr(my);
-    const uint32_t zaddr = lbase + kChunkBytes;
-    if (lane < 4) reinterpret_cast<uint32_t*>(my + kChunkBytes)[lane] = 0u;
+    char* wl = my + kNzLds;
 
-    float acc[NW];
+    f4_t acc[NM];
 #pragma unroll
-    for (int n = 0; n < NW; n++) acc[n] = 0.f;
+    for (int m = 0; m < NM; m++) acc[m] = f4_t{0.f, 0.f, 0.f, 0.f};
 
     const int first = (split * WAVES + wave) * nbpw;
     int last = first + nbpw;
     if (last > nblk) last = nblk;
-    if (first < last) {
-        ChunkRegs cr;
-        uint32_t bytes = chunk_bytes(ixk + (size_t)first * D);
-        chunk_fetch(cr, nzk + (size_t)ixk[(size_t)first * D] * 4u, bytes, lane);
-        for (int tb = first; tb < last; tb++) {
-            const uint32_t* ixc = ixk + (size_t)tb * D;
-            const uint32_t start = ixc[0];
-            chunk_stage(cr, my, bytes, lane);
-            if (tb + 1 < last) {
-                bytes = chunk_bytes(ixc + D);
-                chunk_fetch(cr, nzk + (size_t)ixc[D] * 4u, bytes, lane);
+    constexpr int subs_per_blk = 64 / kSubTiles;
+    const uint32_t wrow = lds_addr(wl) + (uint32_t)(lane & 3) * kWRow;
+    walk_subs<NM>(
+        (last - first) * subs_per_blk,
+        [=](int n) {
+            return (size_t)(first + n / subs_per_blk) * D + (size_t)half * 64 + (size_t)(n % subs_per_blk) * kSubTiles;
+        },
+        [=](int n) {
+            // the sub-chunk's probabilities, [row][kSubTiles] fp16: one instruction moves 256 bytes = kRowsPer rows
+            constexpr int kDwPerRow = kSubTiles / 2, kRowsPer = 64 / kDwPerRow;
+            const size_t tok0 = (size_t)(first + n / subs_per_blk) * 64 + (size_t)(n % subs_per_blk) * kSubTiles;
+#pragma unroll
+            for (int i = 0; i < (NM * 4 + kRowsPer - 1) / kRowsPer; i++) {
+                const int row = kRowsPer * i + lane / kDwPerRow;
+                if (row < NW) dma4(wk + (size_t)row * Lc + tok0 + 2 * (lane % kDwPerRow), wl + (n & 1) * kWBuf + i * 256);
             }
-            __builtin_amdgcn_wave_barrier();
-            chunk_accumulate<NW>(bmk + (size_t)tb * D, ixc, lbase - start * 4u, zaddr, wk + (size_t)tb * 64,
-                                 (size_t)Lc, acc);
-            __builtin_amdgcn_wave_barrier();
-        }
-    }
-    // workgroup reduction: every wavefront parks its sums in its own chunk buffer (NW*256 <= 8192 bytes)
+        },
+        [=](int n) { return wrow + (uint32_t)(n & 1) * kWBuf; }, 4u * kWRow, bmk, ixk, nzk, my, lane, acc);
+    // workgroup reduction: every wavefront parks its sums [accumulator][channel] in its own LDS area
     __syncthreads();
     float* mine = reinterpret_cast<float*>(my);
+    const int j = lane & 3;
 #pragma unroll
-    for (int n = 0; n < NW; n++) mine[n * 64 + lane] = acc[n];
+    for (int m = 0; m < NM; m++) {
+        if (4 * m + j < NW) *reinterpret_cast<f4_t*>(mine + (4 * m + j) * 64 + (lane & ~3)) = acc[m];
+    }
     __syncthreads();
     for (int o = (int)threadIdx.x; o < NW * 64; o += WAVES * 64) {
         float s = 0.f;
@@ -275,7 +414,7 @@ static int check_spmv_args(const void* bmp, const void* nz, const void* idx, con
     if (!bmp || !nz || !idx || !nz_off || !Bm || !C) return MSTF_EINVAL;
     if (tokens <= 0 || head_dim <= 0 || Bq <= 0 || groups <= 0 || n_rows <= 0) return MSTF_EINVAL;
     if (Bq % groups != 0) return MSTF_EINVAL;
-    if (tokens % 64 != 0 || head_dim % 64 != 0) return MSTF_EUNSUPPORTED;
+    if (tokens % 64 != 0 || head_dim % 64 != 0 || head_dim > 128) return MSTF_EUNSUPPORTED;
     if (!aligned_to(bmp, 8) || !aligned_to(nz, 16) || !aligned_to(idx, 4) || !aligned_to(nz_off, 4) ||
         !aligned_to(Bm, 4) || !aligned_to(C, 2))
         return MSTF_EALIGN;
@@ -316,7 +455,7 @@ static ValuePlan plan_value(int Lc, int D, int Bkv, int nw)
     p.waves = nw > 8 ? 4 : 8;
     // aim at ~4096 resident wavefronts on 256 CUs, at least two token blocks each to pipeline
     long nb = (chunks + 4095) / 4096;
-    if (nb < 2) nb = 2;
+    if (nb < 1) nb = 1;
     if (nb > nblk) nb = nblk;
     p.nbpw = (int)nb;
     p.nsplit = (nblk + p.waves * p.nbpw - 1) / (p.waves * p.nbpw);
