@@ -1,0 +1,55 @@
+"""Drop-in for the reference's kernel_quant/compression_quant.py (convert_key_batched_quant :159-264,
+convert_value_batched_quant :425-529): same arguments and return tuples.  The reference hard-codes
+2-bit codes; `bit` is exposed here as an extra keyword (2, 4 or 8; capacity = 32 // bit).
+
+inputs: [B, M, N] fp16 on the GPU, already pruned, M % 64 == 0.
+"""
+import torch
+
+from . import ops
+from ._lib import check, lib
+
+
+def _convert(inputs, is_value, bit, kth=0):
+    assert inputs.is_cuda
+    assert inputs.dim() == 3
+    B, M, N = inputs.shape
+    assert M % 64 == 0
+    if inputs.dtype != torch.float16:
+        raise RuntimeError("inputs must be float16")
+    x = inputs.contiguous()
+    dev = x.device
+    T = M * N // 64
+    L = lib()
+    bmp = torch.empty((B, T), dtype=torch.int64, device=dev)
+    tile_off = torch.empty((B, T), dtype=torch.int32, device=dev)
+    counts = torch.empty((B, T), dtype=torch.int32, device=dev)
+    units = torch.empty((B, T), dtype=torch.int32, device=dev)
+    scales = torch.empty((B, T), dtype=torch.float16, device=dev)
+    zeros = torch.empty((B, T), dtype=torch.float16, device=dev)
+    total = torch.empty((1,), dtype=torch.int64, device=dev)
+    ws = ops.workspace(dev, L.mstf_compress_quant_workspace_bytes(B, M, N))
+    fn = L.mstf_compress_value_quant if is_value else L.mstf_compress_key_quant
+    name = "mstf_compress_value_quant" if is_value else "mstf_compress_key_quant"
+    st = torch.cuda.current_stream().cuda_stream
+    # worst case: every element kept -> T * (64 // capacity) words; sized exactly after the count phase
+    # (one host read of the total, as the reference's .item() does)
+    args = (x.data_ptr(), B, M, N, int(kth), int(bit), bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(),
+            units.data_ptr(), scales.data_ptr(), zeros.data_ptr(), total.data_ptr())
+    check(fn(st, *args, None, 0, ws.data_ptr(), ws.numel()), name)
+    n = int(total.item())
+    packed = torch.zeros((max(n, 1),), dtype=torch.int32, device=dev)
+    if n > 0:
+        check(fn(st, *args, packed.data_ptr(), n, ws.data_ptr(), ws.numel()), name)
+    return bmp, tile_off, packed[:n] if n > 0 else packed[:0], counts, units, scales, zeros
+
+
+def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2):
+    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit)
+    if return_metadata:
+        return bmp, tile_off, packed, counts, units, scales, zeros
+    return bmp, tile_off, packed, scales, zeros
+
+
+def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2):
+    return _convert(inputs, True, bit)

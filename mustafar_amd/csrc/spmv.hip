@@ -12,7 +12,7 @@
 // four accumulators (the GQA query group) at once, so the products cost no vector-ALU issue slots.
 // Bitmaps and tile offsets are wave-uniform and come through scalar loads; weights are staged in
 // LDS by the same LDS-direct loads.
-#include "common.hpp"
+#include "spmv_common.hpp"
 
 namespace mstf {
 
@@ -352,21 +352,6 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_kernel(
     }
 }
 
-// Adds the token-split partials of rows [row0, row0+nw) of every KV head and rounds to fp16.
-__global__ __launch_bounds__(256) void value_merge_kernel(const float* __restrict__ part, _Float16* __restrict__ C,
-                                                          int nsplit, int D, int rows_per_kv, int row0, int nw,
-                                                          size_t total)
-{
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const size_t d = i % D;
-    const size_t r = i / D;
-    const size_t row = (r / nw) * rows_per_kv + row0 + (r % nw);
-    float s = 0.f;
-    for (int k = 0; k < nsplit; k++) s += part[(row * nsplit + k) * D + d];
-    C[row * D + d] = (_Float16)s;
-}
-
 // ------------------------------------------------------------------------------- softmax
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float* sh)
 {
@@ -421,15 +406,6 @@ static int check_spmv_args(const void* bmp, const void* nz, const void* idx, con
     return MSTF_OK;
 }
 
-// Largest accumulator count with an instantiated kernel that fits in `left`.
-static int pick_nw(int left)
-{
-    const int opts[] = {32, 16, 8, 4, 2, 1};
-    for (int o : opts)
-        if (o <= left) return o;
-    return 1;
-}
-
 template <int NW>
 static void launch_key(hipStream_t st, const uint64_t* bmp, const char* nz, const uint32_t* idx,
                        const uint32_t* nz_off, const _Float16* Bm, _Float16* C, int Lc, int D, int Bkv, int rows_per_kv,
@@ -439,27 +415,6 @@ static void launch_key(hipStream_t st, const uint64_t* bmp, const char* nz, cons
     const int ntasks = Bkv * nblk;
     hipLaunchKernelGGL(key_spmv_kernel<NW>, dim3((ntasks + 3) / 4), dim3(256), 0, st, bmp, nz, idx, nz_off, Bm, C, Lc,
                        D, nblk, ntasks, rows_per_kv, row0);
-}
-
-struct ValuePlan {
-    int waves;   // wavefronts per workgroup
-    int nbpw;    // token blocks per wavefront
-    int nsplit;  // workgroups along the token axis
-};
-
-static ValuePlan plan_value(int Lc, int D, int Bkv, int nw)
-{
-    ValuePlan p;
-    const int nblk = Lc / 64;
-    const long chunks = (long)nblk * (D / 64) * Bkv;
-    p.waves = nw > 8 ? 4 : 8;
-    // aim at ~4096 resident wavefronts on 256 CUs, at least two token blocks each to pipeline
-    long nb = (chunks + 4095) / 4096;
-    if (nb < 1) nb = 1;
-    if (nb > nblk) nb = nblk;
-    p.nbpw = (int)nb;
-    p.nsplit = (nblk + p.waves * p.nbpw - 1) / (p.waves * p.nbpw);
-    return p;
 }
 
 template <int NW, int WAVES>
@@ -508,16 +463,7 @@ extern "C" size_t mstf_value_spmv_workspace_bytes(int M, int K, int Bq, int grou
 {
     if (M <= 0 || K <= 0 || Bq <= 0 || groups <= 0 || n_rows <= 0 || K % 64 != 0 || M % 64 != 0 || Bq % groups != 0)
         return 0;
-    const int rows_per_kv = groups * n_rows;
-    size_t worst = 0;
-    for (int row0 = 0; row0 < rows_per_kv;) {
-        const int nw = pick_nw(rows_per_kv - row0);
-        const ValuePlan pl = plan_value(K, M, Bq / groups, nw);
-        const size_t need = pl.nsplit > 1 ? (size_t)Bq * n_rows * pl.nsplit * M * sizeof(float) : 0;
-        if (need > worst) worst = need;
-        row0 += nw;
-    }
-    return round_up(worst, 256);
+    return value_workspace_bytes(M, K, Bq, groups, n_rows);
 }
 
 extern "C" int mstf_value_spmv_f16(void* stream, const uint64_t* bmp, const mstf_half* nz, const uint32_t* idx,
@@ -551,9 +497,7 @@ extern "C" int mstf_value_spmv_f16(void* stream, const uint64_t* bmp, const mstf
         rc = check_launch();
         if (rc != MSTF_OK) return rc;
         if (pl.nsplit > 1) {
-            const size_t total = (size_t)Bkv * nw * M;
-            hipLaunchKernelGGL(value_merge_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, part, c,
-                               pl.nsplit, M, rows_per_kv, row0, nw, total);
+            launch_value_merge(st, part, c, pl.nsplit, M, rows_per_kv, row0, nw, Bkv);
             rc = check_launch();
             if (rc != MSTF_OK) return rc;
         }

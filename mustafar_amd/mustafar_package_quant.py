@@ -1,0 +1,116 @@
+"""Drop-in for the reference's `mustafar_package_quant` extension
+(kernel_quant/kernel_wrapper/pybind_quant.cpp:10-177, mustafar_wrapper_quant.cu): the four operators
+and their four aliases, same keyword names, checks and output shapes.
+
+Differences that do not change results: `split_k` and `value_tile_config` only steer how the
+reference splits its launch (its tile64 / fused configurations address the wrong tiles); here the
+split is chosen by the library and both arguments are accepted and ignored.  `tile_counts` /
+`tile_units` are validated but not read: they follow from the bitmaps.
+"""
+import torch
+
+from . import ops
+from ._lib import check, lib
+
+
+def _common_checks(B, tensors, int_names, half_names):
+    dev = B.device
+    for name, t in tensors.items():
+        if t.device != dev:
+            raise RuntimeError("All input tensors must be on the same device.")
+    if B.dtype != torch.float16:
+        raise RuntimeError("Tensor B must be of type float16.")
+    if tensors["bmp"].dtype != torch.int64:
+        raise RuntimeError("Tensor bmp must be of type int64.")
+    for name in int_names:
+        if tensors[name].dtype != torch.int32:
+            raise RuntimeError("Tensor %s must be of type int32." % name)
+    for name in half_names:
+        if tensors[name].dtype != torch.float16:
+            raise RuntimeError("Tensor %s must be of type float16." % name)
+    if not all(t.is_contiguous() for t in tensors.values()):
+        raise RuntimeError("All tensors must be contiguous.")
+    if not (B.is_cuda and all(t.is_cuda for t in tensors.values())):
+        raise RuntimeError("All tensors must be on CUDA device.")
+    if tensors["NZ_quant"].numel() == 0:
+        raise RuntimeError("NZ_quant is empty.")
+
+
+def _key(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B, M_Global, K_Global, Batch_Size,
+         num_key_value_groups, bit, capacity, dequant_mode):
+    tensors = {"bmp": bmp, "NZ_quant": NZ_quant, "tile_offsets": tile_offsets, "scales": scales, "zeros": zeros}
+    ints = ["NZ_quant", "tile_offsets"]
+    if tile_counts is not None:
+        tensors["tile_counts"], tensors["tile_units"] = tile_counts, tile_units
+        ints += ["tile_counts", "tile_units"]
+    _common_checks(B, tensors, ints, ["scales", "zeros"])
+    if not B.is_contiguous():
+        raise RuntimeError("All tensors must be contiguous.")
+    if B.numel() != Batch_Size * 8 * K_Global:
+        raise RuntimeError("Tensor B must hold Batch_Size x 8 x K_Global elements.")
+    C = torch.empty((Batch_Size, 8, M_Global), dtype=torch.float16, device=B.device)
+    check(lib().mstf_key_spmv_quant(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
+                                    tile_offsets.data_ptr(),
+                                    tile_counts.data_ptr() if tile_counts is not None else None,
+                                    tile_units.data_ptr() if tile_units is not None else None, scales.data_ptr(),
+                                    zeros.data_ptr(), B.data_ptr(), C.data_ptr(), int(M_Global), int(K_Global),
+                                    int(Batch_Size), int(num_key_value_groups), 8, int(bit), int(capacity),
+                                    int(dequant_mode)), "mustafar_key_formulation_quant")
+    return C
+
+
+def mustafar_key_formulation_quant(bmp, NZ_quant, tile_offsets, scales, zeros, B, M_Global, K_Global, Batch_Size,
+                                   num_key_value_groups, bit, capacity, dequant_mode=0):
+    return _key(bmp, NZ_quant, tile_offsets, None, None, scales, zeros, B, M_Global, K_Global, Batch_Size,
+                num_key_value_groups, bit, capacity, dequant_mode)
+
+
+def mustafar_key_formulation_quant_meta(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B, M_Global,
+                                        K_Global, Batch_Size, num_key_value_groups, bit, capacity, dequant_mode=0):
+    return _key(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B, M_Global, K_Global, Batch_Size,
+                num_key_value_groups, bit, capacity, dequant_mode)
+
+
+def _value(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, P, n_rows, M_Global, K_Global,
+           Batch_Size, num_key_value_groups, bit, capacity, dequant_mode, what):
+    tensors = {"bmp": bmp, "NZ_quant": NZ_quant, "tile_offsets": tile_offsets, "tile_counts": tile_counts,
+               "tile_units": tile_units, "scales": scales, "zeros": zeros}
+    _common_checks(P, tensors, ["NZ_quant", "tile_offsets", "tile_counts", "tile_units"], ["scales", "zeros"])
+    if P.numel() != Batch_Size * n_rows * K_Global:
+        raise RuntimeError("score tensor has the wrong number of elements.")
+    P = P.contiguous()
+    L = lib()
+    shape = (Batch_Size, 8, M_Global) if n_rows == 8 else (Batch_Size, M_Global)
+    C = torch.empty(shape, dtype=torch.float16, device=P.device)
+    wsb = L.mstf_value_spmv_quant_workspace_bytes(int(M_Global), int(K_Global), int(Batch_Size),
+                                                  int(num_key_value_groups), n_rows)
+    ws = ops.workspace(P.device, wsb)
+    check(L.mstf_value_spmv_quant(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
+                                  tile_offsets.data_ptr(), tile_counts.data_ptr(), tile_units.data_ptr(),
+                                  scales.data_ptr(), zeros.data_ptr(), P.data_ptr(), C.data_ptr(), int(M_Global),
+                                  int(K_Global), int(Batch_Size), int(num_key_value_groups), n_rows, int(bit),
+                                  int(capacity), int(dequant_mode), ws.data_ptr(), ws.numel()), what)
+    return C
+
+
+def mustafar_value_formulation_quant(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B,
+                                     Reduction_Workspace, M_Global, K_Global, Batch_Size, num_key_value_groups, bit,
+                                     capacity, dequant_mode=0, split_k=1, value_tile_config=0):
+    return _value(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B, 8, M_Global, K_Global,
+                  Batch_Size, num_key_value_groups, bit, capacity, dequant_mode, "mustafar_value_formulation_quant")
+
+
+def mustafar_value_formulation_quant_decode_n1(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros,
+                                               score, Reduction_Workspace, M_Global, K_Global, Batch_Size,
+                                               num_key_value_groups, bit, capacity, dequant_mode=0, split_k=1):
+    """score: [Batch_Size, K_Global] -> [Batch_Size, M_Global]."""
+    return _value(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, score, 1, M_Global, K_Global,
+                  Batch_Size, num_key_value_groups, bit, capacity, dequant_mode,
+                  "mustafar_value_formulation_quant_decode_n1")
+
+
+# aliases the reference exports for its model code (pybind_quant.cpp:96-176)
+mustafar_quant_sparse_forward = mustafar_key_formulation_quant
+mustafar_quant_sparse_forward_meta = mustafar_key_formulation_quant_meta
+mustafar_quant_sparse_value_forward = mustafar_value_formulation_quant
+mustafar_quant_sparse_value_forward_decode_n1 = mustafar_value_formulation_quant_decode_n1

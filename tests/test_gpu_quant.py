@@ -1,0 +1,159 @@
+"""GPU parity of the quantised path (2- and 4-bit) against the CPU oracle, through the C ABI.
+
+Bit-exact against the oracle: bitmaps, raw counts, units, global tile offsets, fp16 scales / zeros
+and the packed codes (the oracle evaluates the reference's closed forms in fp32 and rounds once;
+parity with the Triton original's intermediate precision is not pinned by any reference fixture).
+Within 1e-2 (relative to the row maximum): quantised key / value products against the dense masked
+attention on the dequantised cache, and against the fp32 sums of the oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+QTOL = 1e-2  # tolerance of the north-star metric for 4-bit and 2-bit non-zeros
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def to_gpu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev())
+
+
+def rel_rowmax(a, b):
+    a = a.astype(np.float64).reshape(-1, a.shape[-1])
+    b = b.astype(np.float64).reshape(-1, b.shape[-1])
+    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
+
+
+def pruned(seed, B, M, kth=89):
+    K, V = orc.make_kv(seed, B, M)
+    K[0, :64, 7] = 0          # an empty key tile
+    V[0, 3, :] = 0            # empty value tiles
+    K[0, 64:128, 11] = np.float16(1.25)   # a constant tile: scale falls back to 1
+    return orc.prune_rows(K, kth), orc.prune_rows(V, kth)
+
+
+@pytest.mark.parametrize("bit", [2, 4])
+@pytest.mark.parametrize("is_value", [0, 1])
+def test_quant_compress_bit_exact(bit, is_value):
+    from mustafar_amd import compression_quant as cq
+    Kp, Vp = pruned(31 + bit, 3, 256)
+    x = Vp if is_value else Kp
+    ref = orc.compress_quant(x, is_value, bit)
+    if is_value:
+        got = cq.convert_value_batched_quant(to_gpu(x), bit=bit)
+    else:
+        got = cq.convert_key_batched_quant(to_gpu(x), return_metadata=True, bit=bit)
+        short = cq.convert_key_batched_quant(to_gpu(x), bit=bit)
+        assert len(short) == 5
+    names = ["bitmaps", "tile_offsets", "packed", "counts", "units", "scales", "zeros"]
+    dtypes = [torch.int64, torch.int32, torch.int32, torch.int32, torch.int32, torch.float16, torch.float16]
+    for name, g, r, dt in zip(names, got, ref, dtypes):
+        assert g.dtype == dt, name
+        g = g.cpu().numpy()
+        if g.dtype == np.float16:
+            assert np.array_equal(g.view(np.uint16), r.view(np.uint16)), name
+        else:
+            assert np.array_equal(g, r), name
+
+
+@pytest.mark.parametrize("bit", [2, 4])
+@pytest.mark.parametrize("dequant_mode", [0, 1])
+def test_quant_formulations_reference_api(bit, dequant_mode):
+    """The drop-in operators with the reference's argument lists (models/llama_mustafar_quant_kernel.py:445-567)."""
+    from mustafar_amd import compression_quant as cq, mustafar_package_quant as mq
+    groups, Bkv, Lc, D = 4, 2, 256, 128
+    Bq = Bkv * groups
+    cap = 32 // bit
+    Kp, Vp = pruned(41, Bkv, Lc)
+    kb, ko, kp, kc, ku, ks, kz = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
+    vb, vo, vp, vc, vu, vs, vz = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    rk = orc.compress_quant(Kp, 0, bit)
+    rv = orc.compress_quant(Vp, 1, bit)
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((Bq, 1, D)).astype(np.float16)
+    padded_query = torch.nn.functional.pad(to_gpu(q), (0, 0, 0, 7)).contiguous()
+    att = mq.mustafar_key_formulation_quant(kb, kp, ko, ks, kz, padded_query, Lc, D, Bq, groups, bit, cap,
+                                            dequant_mode=dequant_mode)
+    att_meta = mq.mustafar_quant_sparse_forward_meta(kb, kp, ko, kc, ku, ks, kz, padded_query, Lc, D, Bq, groups, bit,
+                                                     cap, dequant_mode)
+    assert tuple(att.shape) == (Bq, 8, Lc) and att.dtype == torch.float16
+    assert torch.equal(att, att_meta)
+    C, Cf = orc.spmv_quant(rk[0], rk[2], rk[1], rk[5], rk[6], padded_query.cpu().numpy(), 0, Lc, D, groups, bit,
+                           dequant_mode)
+    assert rel_rowmax(att.cpu().numpy()[:, 0], Cf[:, 0]) < 2e-3
+    assert not att[:, 1:].any()
+
+    P = orc.scale_softmax(C[:, 0], D)
+    padded_score = torch.nn.functional.pad(to_gpu(P).view(Bq, 1, Lc), (0, 0, 0, 7)).contiguous()
+    ws = torch.zeros(1, dtype=torch.float16, device=dev())
+    out = mq.mustafar_value_formulation_quant(vb, vp, vo, vc, vu, vs, vz, padded_score, ws, D, Lc, Bq, groups, bit, cap,
+                                              dequant_mode=dequant_mode, split_k=4, value_tile_config=1)
+    assert tuple(out.shape) == (Bq, 8, D)
+    O, Of = orc.spmv_quant(rv[0], rv[2], rv[1], rv[5], rv[6], padded_score.cpu().numpy(), 1, Lc, D, groups, bit,
+                           dequant_mode)
+    assert rel_rowmax(out.cpu().numpy()[:, 0], Of[:, 0]) < 2e-3
+    n1 = mq.mustafar_value_formulation_quant_decode_n1(vb, vp, vo, vc, vu, vs, vz, to_gpu(P), ws, D, Lc, Bq, groups,
+                                                       bit, cap, dequant_mode)
+    assert tuple(n1.shape) == (Bq, D)
+    assert rel_rowmax(n1.cpu().numpy(), Of[:, 0]) < 2e-3
+    with pytest.raises(RuntimeError):
+        mq.mustafar_key_formulation_quant(kb, kp, ko, ks.float(), kz, padded_query, Lc, D, Bq, groups, bit, cap)
+    with pytest.raises(RuntimeError):   # capacity must be 32 // bit
+        mq.mustafar_key_formulation_quant(kb, kp, ko, ks, kz, padded_query, Lc, D, Bq, groups, bit, cap + 1)
+
+
+@pytest.mark.parametrize("bit", [2, 4])
+@pytest.mark.parametrize("groups,Bkv,Lc", [(4, 2, 1024), (1, 3, 256), (8, 1, 512)])
+def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc):
+    """Quantised compress -> key SpMV -> softmax -> value SpMV against the oracle's dense masked attention run
+    on the dequantised cache (the reference semantics of the quantised path), one query token per head."""
+    from mustafar_amd import compression_quant as cq, mustafar_package_quant as mq, ops
+    D = 128
+    Bq = Bkv * groups
+    cap = 32 // bit
+    K, V = orc.make_kv(500 + Lc + bit, Bkv, Lc, D)
+    Kp, Vp = orc.prune_rows(K, 89), orc.prune_rows(V, 89)
+    rk = orc.compress_quant(Kp, 0, bit)
+    rv = orc.compress_quant(Vp, 1, bit)
+    Kd = np.stack([orc.decode_quant(rk[0], rk[2], rk[1], rk[5], rk[6], b, Lc, D, 0, bit, 0) for b in range(Bkv)])
+    Vd = np.stack([orc.decode_quant(rv[0], rv[2], rv[1], rv[5], rv[6], b, Lc, D, 1, bit, 0) for b in range(Bkv)])
+    q = np.random.default_rng(Lc).standard_normal((Bq, D)).astype(np.float16)
+    sc_ref, pr_ref, out_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
+
+    kb, ko, kp, kc, ku, ks, kz = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
+    vb, vo, vp, vc, vu, vs, vz = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    L = __import__("mustafar_amd._lib", fromlist=["lib"]).lib()
+    st = torch.cuda.current_stream().cuda_stream
+    s = torch.empty((Bq, 1, Lc), dtype=torch.float16, device=dev())
+    qg = to_gpu(q).view(Bq, 1, D)
+    assert L.mstf_key_spmv_quant(st, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), None, None, ks.data_ptr(),
+                                 kz.data_ptr(), qg.data_ptr(), s.data_ptr(), Lc, D, Bq, groups, 1, bit, cap, 0) == 0
+    assert rel_rowmax(s.cpu().numpy()[:, 0], sc_ref) < QTOL
+    p = ops.scale_softmax(s, D)
+    o = mq.mustafar_value_formulation_quant_decode_n1(vb, vp, vo, vc, vu, vs, vz, p.view(Bq, Lc), None, D, Lc, Bq,
+                                                      groups, bit, cap)
+    assert rel_rowmax(p.cpu().numpy()[:, 0], pr_ref) < QTOL
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
+    # the quantisation itself stays within half a step of the fp16 cache
+    err = np.abs(Kd.astype(np.float32) - np.where(Kp != 0, Kp, 0).astype(np.float32))
+    step = np.repeat(rk[5].astype(np.float32).reshape(Bkv, Lc // 64, D), 64, axis=1)   # key tile = 64 tokens x 1 channel
+    assert (err <= 0.5 * step * 1.01 + 2e-3 * np.abs(Kp.astype(np.float32)) + 1e-6).all()
+
+
+def test_quant_c_abi_rejects_bad_arguments():
+    from mustafar_amd._lib import lib
+    L = lib()
+    z = torch.zeros(256, dtype=torch.int64, device=dev())
+    a = z.data_ptr()
+    assert L.mstf_key_spmv_quant(None, a, a, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 3, 10, 0) == -3   # bit
+    assert L.mstf_key_spmv_quant(None, a, a, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 2, 8, 0) == -1    # capacity
+    assert L.mstf_key_spmv_quant(None, a, a, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 2, 16, 2) == -1   # mode
+    assert L.mstf_key_spmv_quant(None, a, None, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 2, 16, 0) == -1
+    assert L.mstf_compress_key_quant(None, a, 1, 64, 128, 0, 2, a, a, a, a, a, a, a, None, 0, None, 0) == -4
