@@ -1,0 +1,78 @@
+"""The caller's cache state machine (prefill split, 256-token chunk appends) on the GPU: the appended
+cache must be byte-identical to a one-shot compression of the same tokens, and every decode step must
+match the oracle's dense masked attention over [pruned compressed part | dense window]."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_rowmax(a, b):
+    a = a.astype(np.float64).reshape(-1, a.shape[-1])
+    b = b.astype(np.float64).reshape(-1, b.shape[-1])
+    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
+
+
+def test_prefill_decode_append_matches_one_shot_and_oracle():
+    from mustafar_amd import ops
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D, res = 2, 2, 4, 128, 256
+    L0, steps = 700, 330                       # prefill: Lc = 256, window 444; appends at kv_len 768 and 1024
+    total = L0 + steps
+    K, V = orc.make_kv(77, bs * n_kv, total, D)
+    rng = np.random.default_rng(1)
+    Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
+    cache = SparseKVCache(g, D, 0.7, 0.7, res)
+    cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
+    assert cache.compressed_length == ((L0 - res) // 256) * 256 == 256
+    checked = 0
+    for t in range(steps):
+        pos = L0 + t
+        Lc_before = cache.compressed_length
+        q = torch.from_numpy(Q[t]).to(dev).view(bs, n_kv * g, 1, D)
+        out = cache.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
+        if t % 37 == 0 or cache.compressed_length != Lc_before or t == steps - 1:
+            Kf, Vf = K[:, :pos + 1].copy(), V[:, :pos + 1].copy()
+            Kf[:, :Lc_before] = orc.prune_rows(np.ascontiguousarray(Kf[:, :Lc_before]), 89)
+            Vf[:, :Lc_before] = orc.prune_rows(np.ascontiguousarray(Vf[:, :Lc_before]), 89)
+            _, _, ref = orc.dense_masked_attention(Q[t], Kf, Vf, g)
+            assert rel_rowmax(out.cpu().numpy().reshape(-1, D), ref) < 2e-3, (t, pos)
+            checked += 1
+    assert cache.kv_len == total and cache.compressed_length == 768      # two appends happened
+    assert cache.k_win.shape[2] == total - 768
+    assert checked >= 10
+    # incremental == one-shot, byte for byte
+    Lc = cache.compressed_length
+    for side, is_value in ((cache.k, 0), (cache.v, 1)):
+        src = V if is_value else K
+        rb, ri, rnz, roff = orc.compress(orc.prune_rows(np.ascontiguousarray(src[:, :Lc]), 89), is_value)
+        assert np.array_equal(side.bmp.cpu().numpy(), rb)
+        assert np.array_equal(side.idx.cpu().numpy(), ri)
+        assert np.array_equal(side.nz_off.cpu().numpy(), roff)
+        assert np.array_equal(side.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+    one = ops.compress(Kt[:, :, :Lc].reshape(bs * n_kv, Lc, D).contiguous(), False, kth=89)
+    assert torch.equal(one.bmp, cache.k.bmp) and torch.equal(one.idx, cache.k.idx)
+    assert torch.equal(one.packed(), cache.k.packed())
+
+
+def test_short_prompt_stays_dense_until_first_chunk():
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D = 1, 2, 2, 128
+    K, V = orc.make_kv(5, bs * n_kv, 300, D)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, 300, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, 300, D)
+    cache = SparseKVCache(g, D, 0.5, 0.5, 32)
+    cache.prefill(Kt[:, :, :200], Vt[:, :, :200])       # (200 - 32) // 256 == 0 -> nothing compressed
+    assert cache.compressed_length == 0 and cache.k is None
+    q = torch.randn((bs, n_kv * g, 1, D), device=dev, dtype=torch.float16)
+    for pos in range(200, 300):
+        out = cache.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
+    assert cache.compressed_length == 256 and cache.kv_len == 300   # 288 - 32 - 0 == 256 triggers the first chunk
+    assert torch.isfinite(out).all()
