@@ -108,6 +108,21 @@ int mstf_value_spmv_f16(void* stream, const uint64_t* bmp, const mstf_half* nz, 
 int mstf_scale_softmax_f16(void* stream, const mstf_half* s, mstf_half* p, int64_t rows, int L, int64_t s_stride,
                            int64_t p_stride, int head_dim);
 
+/* ------------------------------------------------------------------ fused decode attention
+ * One launch for the whole compressed part of a decode step, i.e. the sequence
+ * mustafar_key_formulation -> / sqrt(head_dim) -> softmax(fp32) -> mustafar_value_formulation of the
+ * caller (models/llama_mustafar_kernel.py:394-396,405,425,434-436) for one query row per head:
+ *   out[bq, :] = softmax_t( fp16(q[bq].Ktilde[t]) / sqrt(d) ) . Vtilde[t, :]     over the `tokens` cached tokens
+ * q, out: [Bq, head_dim] fp16 (head_dim 128, groups <= 8).  Scores and probabilities stay on chip.
+ * lse_out (nullable) [Bq, 2] fp32 receives (max, sum of exp(w - max)) per row, so a caller that keeps a
+ * dense local window can combine that window's attention with this result under one softmax. */
+size_t mstf_decode_attention_workspace_bytes(int tokens, int head_dim, int Bq, int groups);
+int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                              const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                              const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out,
+                              float* lse_out, int tokens, int head_dim, int Bq, int groups, void* workspace,
+                              size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),
  * with the bit width a parameter (the reference hard-codes 2).  Same tiles and bitmaps as above;

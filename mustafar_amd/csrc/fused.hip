@@ -1,0 +1,304 @@
+// Fused sparse decode attention: key SpMV -> scale + softmax -> value SpMV in one launch.
+//
+// One wavefront owns one (KV head, 64-token block).  It streams the block's 128 key tiles and then
+// its 128 value tiles through the same LDS double buffer (the first value loads are issued while
+// the last key tiles are still being decompressed - they do not depend on the scores):
+//   key phase   : lane = token, MFMA accumulators hold q.K^T for the block's 64 tokens x the
+//                 GQA query heads of the KV head;
+//   softmax     : scores are rounded to fp16, divided by sqrt(d) in fp16 (as the reference's glue
+//                 does), the block maximum and the sum of exp(w - max) are reduced over the wavefront,
+//                 and the un-normalised weights exp(w - max) go to LDS as the fp16 B operand;
+//   value phase : lane = channel, MFMA accumulators hold sum_t weight[t] * V[t][channel].
+// The wavefronts of a workgroup (consecutive token blocks of one KV head) then combine their
+// (max, sum, output) triples through LDS; token splits across workgroups are combined by a small
+// merge kernel.  Scores and probabilities never touch HBM.
+#include "spmv_common.hpp"
+#include "spmv_device.hpp"
+
+namespace mstf {
+
+constexpr int kFusedD = 128;
+constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
+constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
+constexpr int kFusedWaves = 8;
+
+__device__ __forceinline__ float wave_max_same_column(float v)
+{
+    // lanes 4b+j for b = 0..15 hold column j: combine over b with xor shuffles of 4, 8, 16, 32
+#pragma unroll
+    for (int o = 4; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_same_column(float v)
+{
+#pragma unroll
+    for (int o = 4; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns token block
+// s*kFusedWaves + w.  NM = accumulator groups of four query heads (groups <= 4*NM).
+//   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
+//   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
+template <int NM>
+__global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
+    const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
+    const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
+    const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
+    _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int Lc, int groups, int nblk,
+    int nsplit, int write_final, float sqrt_d)
+{
+    constexpr int D = kFusedD;
+    constexpr int kQLds = NM * 4 * D * 2;          // query rows [4*NM][D] fp16
+    constexpr int kPRow = 64 * 2;                  // one row of block weights: 64 tokens fp16
+    constexpr int kPLds = NM * 4 * kPRow;
+    constexpr int kNeed = kNzLds + kQLds + kPLds;
+    constexpr int kPark = NM * 4 * D * 4 + 64;     // per-wave (output, max, sum) parked for the workgroup combine
+    constexpr int kWaveLds = kNeed > kPark ? kNeed : kPark;
+    __shared__ __attribute__((aligned(16))) char lds[kFusedWaves][kWaveLds];
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int split = (int)blockIdx.x;
+    const int kv = (int)blockIdx.y;
+    const int tb = split * kFusedWaves + wave;
+    const bool active = tb < nblk;  // wave-uniform
+    const int j = lane & 3;
+    const size_t T = (size_t)Lc * D / 64;
+    char* my = lds[wave];
+    char* ql = my + kNzLds;
+    char* pl = ql + kQLds;
+    const uint32_t lbase = lds_addr(my);
+    const uint32_t zaddr = lbase + 2 * kSubBytes;
+
+    f4_t acc_v[NM][2];
+    float m_run[NM], l_run[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        acc_v[m][0] = f4_t{0.f, 0.f, 0.f, 0.f};
+        acc_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+        m_run[m] = -INFINITY;
+        l_run[m] = 0.f;
+    }
+
+    if (active) {
+        const uint64_t* bmK = k_bmp + (size_t)kv * T + (size_t)tb * D;
+        const uint32_t* ixK = k_idx + (size_t)kv * (T + 1) + (size_t)tb * D;
+        const char* nzK = k_nz + (size_t)k_nz_off[kv] * 16u;
+        const uint64_t* bmV = v_bmp + (size_t)kv * T + (size_t)tb * D;
+        const uint32_t* ixV = v_idx + (size_t)kv * (T + 1) + (size_t)tb * D;
+        const char* nzV = v_nz + (size_t)v_nz_off[kv] * 16u;
+        if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
+
+        // sub-chunk n of the walk: n < kKeySubs -> key tiles n*32.., else value tiles (n-kKeySubs)*32..
+        auto bm_of = [&](int n) { return n < kKeySubs ? bmK + n * kSubTiles : bmV + (n - kKeySubs) * kSubTiles; };
+        auto ix_of = [&](int n) { return n < kKeySubs ? ixK + n * kSubTiles : ixV + (n - kKeySubs) * kSubTiles; };
+        auto nz_of = [&](int n) { return n < kKeySubs ? nzK : nzV; };
+        // idx at the boundaries of all sub-chunks, fetched by one vector load (lanes 0.. hold the key
+        // boundaries, lanes 16.. the value boundaries): no stage then waits for a scalar load from HBM
+        // before it can issue its value stream
+        static_assert(kKeySubs < 16 && kValSubs < 48, "boundary lanes");
+        uint32_t bnd = 0u;
+        if (lane <= kKeySubs) bnd = ixK[lane * kSubTiles];
+        else if (lane >= 16 && lane <= 16 + kValSubs) bnd = ixV[(lane - 16) * kSubTiles];
+        auto issue = [&](int n) {
+            const int bl = n < kKeySubs ? n : 16 + n - kKeySubs;
+            const uint32_t s0 = __builtin_amdgcn_readlane(bnd, bl);
+            const uint32_t s1 = __builtin_amdgcn_readlane(bnd, bl + 1);
+            sub_issue(nz_of(n) + (size_t)s0 * 4u, sub_bytes(s0, s1), my + (n & 1) * kSubBytes, lane);
+            return touch_sub(bm_of(n), ix_of(n), lane);
+        };
+
+        // the query rows of this KV head: groups x D fp16, contiguous
+        {
+            const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
+            const uint32_t qbytes = (uint32_t)groups * D * 2u;
+#pragma unroll
+            for (int i = 0; i < (kQLds + 1023) / 1024; i++) {
+                const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+                if (o < qbytes) dma16(qsrc + o, ql + i * 1024);
+            }
+        }
+        Touch touch = issue(0);
+
+        f4_t acc_k[NM];
+#pragma unroll
+        for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+        const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
+        const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
+
+#pragma unroll
+        for (int n = 0; n < kKeySubs + kValSubs; n++) {
+            wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for n == 0)
+            if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
+            const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
+            if (n < kKeySubs) {
+                sub_accumulate<NM>(bm_of(n), ix_of(n), buf, zaddr, qrow + (uint32_t)n * kSubTiles * 2u,
+                                   (uint32_t)D * 8u, acc_k);
+            } else {
+                if (n == kKeySubs) {
+                    // ---- softmax statistics of the block; lane 4b+j holds tokens 4b..4b+3 of head 4m+j
+#pragma unroll
+                    for (int m = 0; m < NM; m++) {
+                        float w[4];
+                        float mx = -INFINITY;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const _Float16 s16 = (_Float16)acc_k[m][r];
+                            w[r] = (float)(_Float16)((float)s16 / sqrt_d);
+                            mx = fmaxf(mx, w[r]);
+                        }
+                        mx = wave_max_same_column(mx);
+                        float sum = 0.f;
+                        h4_t e16;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const float e = __expf(w[r] - mx);
+                            e16[r] = (_Float16)e;
+                            sum += (float)e16[r];  // the sum matches the fp16 weights that multiply V
+                        }
+                        sum = wave_sum_same_column(sum);
+                        m_run[m] = mx;
+                        l_run[m] = sum;
+                        *reinterpret_cast<h4_t*>(pl + (m * 4 + j) * kPRow + (lane & ~3) * 2) = e16;
+                    }
+                }
+                const int vs = n - kKeySubs;                      // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
+                constexpr int kSubsPerHalf = 64 / kSubTiles;
+                const int half = vs / kSubsPerHalf;
+                const uint32_t wa = prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u;
+                f4_t tmp[NM];
+#pragma unroll
+                for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
+                sub_accumulate<NM>(bm_of(n), ix_of(n), buf, zaddr, wa, 4u * kPRow, tmp);
+#pragma unroll
+                for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
+            }
+            wait_lgkm0();
+        }
+    }
+
+    // ---- workgroup combine: park (output[4*NM][D], max, sum) of every wavefront, then one thread per (head, channel)
+    __syncthreads();
+    {
+        float* po = reinterpret_cast<float*>(my);
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + (lane & ~3)) = acc_v[m][0];
+            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + 64 + (lane & ~3)) = acc_v[m][1];
+            if (lane < 4) {
+                po[NM * 4 * D + (m * 4 + j) * 2] = m_run[m];
+                po[NM * 4 * D + (m * 4 + j) * 2 + 1] = l_run[m];
+            }
+        }
+    }
+    __syncthreads();
+    for (int o = (int)threadIdx.x; o < groups * D; o += kFusedWaves * 64) {
+        const int h = o / D, c = o - h * D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; w++)
+            M = fmaxf(M, reinterpret_cast<const float*>(lds[w])[NM * 4 * D + h * 2]);
+        float so = 0.f, sl = 0.f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; w++) {
+            const float* pw = reinterpret_cast<const float*>(lds[w]);
+            const float mw = pw[NM * 4 * D + h * 2];
+            const float f = mw == -INFINITY ? 0.f : __expf(mw - M);
+            so += f * pw[h * D + c];
+            sl += f * pw[NM * 4 * D + h * 2 + 1];
+        }
+        const size_t row = (size_t)kv * groups + h;
+        if (write_final) {
+            out[row * D + c] = (_Float16)(so / sl);
+        } else {
+            part_o[(row * nsplit + split) * D + c] = so;
+            if (c == 0) {
+                part_ml[(row * nsplit + split) * 2] = M;
+                part_ml[(row * nsplit + split) * 2 + 1] = sl;
+            }
+        }
+    }
+}
+
+// grid = Bq, 128 threads: log-sum-exp combine of the token splits.
+__global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restrict__ part_o,
+                                                           const float* __restrict__ part_ml,
+                                                           _Float16* __restrict__ out, float* __restrict__ lse_out,
+                                                           int nsplit, int D)
+{
+    const size_t row = blockIdx.x;
+    const int c = (int)threadIdx.x;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; s++) M = fmaxf(M, part_ml[(row * nsplit + s) * 2]);
+    float so = 0.f, sl = 0.f;
+    for (int s = 0; s < nsplit; s++) {
+        const float f = __expf(part_ml[(row * nsplit + s) * 2] - M);
+        so += f * part_o[(row * nsplit + s) * D + c];
+        sl += f * part_ml[(row * nsplit + s) * 2 + 1];
+    }
+    if (c < D) out[row * D + c] = (_Float16)(so / sl);
+    if (lse_out && c == 0) {
+        lse_out[row * 2] = M;
+        lse_out[row * 2 + 1] = sl;
+    }
+}
+
+static int fused_nsplit(int tokens) { return (tokens / 64 + kFusedWaves - 1) / kFusedWaves; }
+
+}  // namespace mstf
+
+using namespace mstf;
+
+extern "C" size_t mstf_decode_attention_workspace_bytes(int tokens, int head_dim, int Bq, int groups)
+{
+    if (tokens <= 0 || head_dim != kFusedD || Bq <= 0 || groups <= 0 || tokens % 64 != 0 || Bq % groups != 0) return 0;
+    const int ns = fused_nsplit(tokens);
+    return round_up((size_t)Bq * ns * (head_dim + 2) * sizeof(float), 256);
+}
+
+extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                         const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
+                                         const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
+                                         const mstf_half* q, mstf_half* out, float* lse_out, int tokens, int head_dim,
+                                         int Bq, int groups, void* workspace, size_t workspace_bytes)
+{
+    if (!k_bmp || !k_nz || !k_idx || !k_nz_off || !v_bmp || !v_nz || !v_idx || !v_nz_off || !q || !out)
+        return MSTF_EINVAL;
+    if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (!aligned_to(k_bmp, 8) || !aligned_to(v_bmp, 8) || !aligned_to(k_nz, 16) || !aligned_to(v_nz, 16) ||
+        !aligned_to(k_idx, 4) || !aligned_to(v_idx, 4) || !aligned_to(k_nz_off, 4) || !aligned_to(v_nz_off, 4) ||
+        !aligned_to(q, 16) || !aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4)))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int Bkv = Bq / groups, nblk = tokens / 64, ns = fused_nsplit(tokens);
+    float* part_o = reinterpret_cast<float*>(workspace);
+    float* part_ml = part_o + (size_t)Bq * ns * head_dim;
+    // with one split and no (max, sum) requested the kernel writes the final output itself
+    const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
+    const dim3 grid((unsigned)ns, (unsigned)Bkv);
+    const char* knz = reinterpret_cast<const char*>(k_nz);
+    const char* vnz = reinterpret_cast<const char*>(v_nz);
+    const _Float16* qh = reinterpret_cast<const _Float16*>(q);
+    _Float16* oh = reinterpret_cast<_Float16*>(out);
+    const float sq = sqrtf((float)head_dim);
+    if (groups <= 4)
+        hipLaunchKernelGGL(decode_attention_kernel<1>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
+                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, ns, write_final,
+                           sq);
+    else
+        hipLaunchKernelGGL(decode_attention_kernel<2>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
+                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, ns, write_final,
+                           sq);
+    int rc = check_launch();
+    if (rc != MSTF_OK) return rc;
+    if (!write_final) {
+        hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, st, part_o, part_ml, oh, lse_out, ns,
+                           head_dim);
+        rc = check_launch();
+    }
+    return rc;
+}

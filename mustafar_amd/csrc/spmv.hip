@@ -10,209 +10,18 @@
 // (global_load_lds, 16 bytes per lane), rebuilds D[t][lane] with a popcount rank (v_mbcnt) per
 // tile and feeds groups of four tiles to v_mfma_f32_4x4x4f16, which multiplies them with the weights of
 // four accumulators (the GQA query group) at once, so the products cost no vector-ALU issue slots.
-// Bitmaps and tile offsets are wave-uniform and come through scalar loads; weights are staged in
-// LDS by the same LDS-direct loads.
+// Bitmaps arrive one per lane by a coalesced vector load and are broadcast with v_readlane; tile
+// offsets are a running sum of padded popcounts on the scalar ALU; weights are staged in LDS by the
+// same LDS-direct loads.
 #include "spmv_common.hpp"
+#include "spmv_device.hpp"
 
 namespace mstf {
-
-#ifndef MSTF_SUB_TILES
-#define MSTF_SUB_TILES 32
-#endif
-constexpr int kSubTiles = MSTF_SUB_TILES;      // tiles per staged piece ("sub-chunk"): 16 or 32
-constexpr int kSubBytes = kSubTiles * 64 * 2;  // worst case: every tile full
-constexpr int kOffsLds = kSubTiles * 4;          // per-tile value offsets of the sub-chunk being decompressed
-constexpr int kNzLds = 2 * kSubBytes + 16 + kOffsLds;  // value double buffer + zero slot (lanes whose bit is clear) + offsets
-
-#define MSTF_GLOBAL __attribute__((address_space(1)))
-
-typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
-typedef float f4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ h4_t as_h4(uint32_t lo, uint32_t hi)
-{
-    const u32x2_t v = {lo, hi};
-    return __builtin_bit_cast(h4_t, v);
-}
-
-__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-
-// LDS-direct loads: data goes from global memory straight into LDS without passing through
-// registers; lane l of the instruction writes `size` bytes at dst + l*size.  Completion is
-// tracked by vmcnt only, the caller waits with wait_vm0() before reading the LDS.
-__device__ __forceinline__ void dma16(const void* src, void* dst_wave_uniform)
-{
-    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 16, 0, 0);
-}
-__device__ __forceinline__ void dma4(const void* src, void* dst_wave_uniform)
-{
-    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 4, 0, 0);
-}
-
-// Streams `bytes` (a multiple of 16, <= kSubBytes) into LDS: piece i of lane l lands at dst + (i*64 + l)*16.
-__device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char* dst, int lane)
-{
-#pragma unroll
-    for (int i = 0; i < kSubBytes / 1024; i++) {
-        if ((uint32_t)(i * 1024) < bytes) {
-            const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
-            if (o < bytes) dma16(src + o, dst + i * 1024);
-        }
-    }
-}
-
-// lanes whose bit of the wave-uniform mask m is set take `yes`, the others `no`.  Written as one
-// v_cndmask on the mask register pair so the compiler keeps the decompression straight-line
-// (it otherwise turns the select into an exec-masked branch per tile).
-__device__ __forceinline__ uint32_t select_lane(uint64_t m, uint32_t yes, uint32_t no)
-{
-    uint32_t r;
-    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(m));
-    return r;
-}
-
-// Packed pair (D[t][lane], D[t+1][lane]) of two tiles as fp16x2.
-//   m0, m1 : tile bitmaps, MSB-first (wave-uniform, scalar registers)
-//   o0, o1 : offsets of the tiles' values inside the staged buffer, fp16 units (wave-uniform, vector registers)
-//   buf    : LDS byte address of the staged buffer;  zaddr: LDS address of two zero bytes
-// rank = offset + popcount(mask below lane) comes from v_mbcnt with the offset as its addend;
-// lanes whose element is absent read the zero slot.  (16-bit LDS loads cannot merge into one
-// register here: with SRAM ECC they clear the other half, hence the explicit pack.)
-__device__ __forceinline__ uint32_t tile_pair(uint32_t m0lo, uint32_t m0hi, uint32_t m1lo, uint32_t m1hi, uint32_t o0,
-                                              uint32_t o1, uint32_t buf, uint32_t zaddr)
-{
-    const uint64_t m0 = lanes_of(u64_of(m0lo, m0hi));
-    const uint64_t m1 = lanes_of(u64_of(m1lo, m1hi));
-    const uint32_t r0 = __builtin_amdgcn_mbcnt_hi((uint32_t)(m0 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m0, o0));
-    const uint32_t r1 = __builtin_amdgcn_mbcnt_hi((uint32_t)(m1 >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m1, o1));
-    const uint32_t a0 = select_lane(m0, r0 * 2u + buf, zaddr);
-    const uint32_t a1 = select_lane(m1, r1 * 2u + buf, zaddr);
-    h2_t p;
-    p.x = lds_load_h(a0);
-    p.y = lds_load_h(a1);
-    return as_u32(p);
-}
-
-// One staged sub-chunk (kSubTiles tiles).  For every group of 4 tiles the lane builds its own four
-// values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator
-// (lane & 3) of each accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in
-// lane 4b+j, the sums of positions 4b..4b+3 for accumulator 4m+j:
-//     acc[m][r] += sum_t D[t][4b + r] * w[4m + j][t]
-//   bm     : the sub-chunk's bitmaps (wave-uniform pointer; one batch of scalar loads)
-//   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
-//   offs   : LDS byte address of the per-tile offsets (fp16 units, relative to buf)
-//   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
-template <int NM>
-__device__ __forceinline__ void sub_accumulate(const uint64_t* bm, uint32_t buf, uint32_t zaddr, uint32_t offs,
-                                               uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
-{
-    u32x16_t mvs[kSubTiles / 8];
-#pragma unroll
-    for (int g = 0; g < kSubTiles / 8; g++) mvs[g] = *reinterpret_cast<const u32x16_a4*>(bm + 8 * g);
-#pragma unroll
-    for (int g = 0; g < kSubTiles / 8; g++) {
-        const u32x16_t mv = mvs[g];
-        const int tt = g * 8;
-        // the same address in every lane: the LDS unit broadcasts the offsets of the 8 tiles
-        const u32x4_t oa = *(MSTF_LDS const u32x4_t*)(uintptr_t)(offs + (uint32_t)tt * 4u);
-        const u32x4_t ob = *(MSTF_LDS const u32x4_t*)(uintptr_t)(offs + (uint32_t)tt * 4u + 16u);
-        const uint32_t v0 = tile_pair(mv[0], mv[1], mv[2], mv[3], oa[0], oa[1], buf, zaddr);
-        const uint32_t v1 = tile_pair(mv[4], mv[5], mv[6], mv[7], oa[2], oa[3], buf, zaddr);
-        const uint32_t v2 = tile_pair(mv[8], mv[9], mv[10], mv[11], ob[0], ob[1], buf, zaddr);
-        const uint32_t v3 = tile_pair(mv[12], mv[13], mv[14], mv[15], ob[2], ob[3], buf, zaddr);
-#pragma unroll
-        for (int m = 0; m < NM; m++) {
-            const u32x4_t q = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup + (uint32_t)tt * 2u);
-            const uint32_t q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
-            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
-            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
-        }
-    }
-}
-
-__device__ __forceinline__ uint32_t sub_bytes(uint32_t start, uint32_t end)
-{
-    const uint32_t b = (end - start) * 4u;
-    return b > (uint32_t)kSubBytes ? (uint32_t)kSubBytes : b;  // a well-formed sub-chunk never exceeds this
-}
-
-// Each lane l < kSubTiles also loads the bitmap of tile l of the coming sub-chunk with a vector load
-// issued together with the value stream.  That serves two purposes: the popcounts give, through
-// a wave prefix sum, the offset of every tile inside the staged buffer (the format pads each tile
-// to a multiple of 8 values, so offsets follow from the bitmaps and idx is only read once per
-// sub-chunk), and it pulls the bitmap lines into L2 before the scalar loads ask for them.
-__device__ __forceinline__ uint2 bitmap_of_lane(const uint64_t* bm, int lane)
-{
-    uint2 b = make_uint2(0u, 0u);
-    if (lane < kSubTiles) b = *reinterpret_cast<const uint2*>(bm + lane);
-    return b;
-}
-// Waits for every outstanding vector-memory operation (LDS-direct loads included).
-__device__ __forceinline__ void wait_vm0_keep(uint2& b)
-{
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(b.x), "+v"(b.y)::"memory");
-}
-// offs[l] = sum over tiles t < l of the padded value count of tile t (fp16 units), l < kSubTiles.
-__device__ __forceinline__ void write_tile_offsets(uint2 b, char* offs, int lane)
-{
-    const uint32_t cnt = (uint32_t)(__popc(b.x) + __popc(b.y));
-    const uint32_t padded = (cnt + 7u) & ~7u;
-    uint32_t inc = padded;
-#pragma unroll
-    for (int o = 1; o < kSubTiles; o <<= 1) {
-        const uint32_t t = __shfl_up(inc, o, 64);
-        if (lane >= o) inc += t;
-    }
-    if (lane < kSubTiles) reinterpret_cast<uint32_t*>(offs)[lane] = inc - padded;
-}
-
-// Walks `nsubs` sub-chunks of one KV head with a two-deep pipeline: while sub-chunk n is being
-// decompressed out of one LDS buffer, sub-chunk n+1 streams from HBM into the other.
-//   tile_of(n)    : first tile of sub-chunk n
-//   stage_w(n)    : issues the LDS-direct loads of the weights sub-chunk n needs (may be a no-op)
-//   waddr_of(n)   : LDS byte address of w[lane & 3][first tile of sub-chunk n]
-template <int NM, class TileOf, class StageW, class WAddrOf>
-__device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stage_w, WAddrOf waddr_of, uint32_t wgroup,
-                                          const uint64_t* bmk, const uint32_t* ixk, const char* nzk, char* my, int lane,
-                                          f4_t (&acc)[NM])
-{
-    const uint32_t lbase = lds_addr(my);
-    const uint32_t zaddr = lbase + 2 * kSubBytes;
-    char* offs = my + 2 * kSubBytes + 16;
-    if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
-    if (nsubs <= 0) return;
-    size_t t_cur = tile_of(0);
-    const uint32_t s0 = ixk[t_cur];
-    sub_issue(nzk + (size_t)s0 * 4u, sub_bytes(s0, ixk[t_cur + kSubTiles]), my, lane);
-    stage_w(0);
-    uint2 lane_bm = bitmap_of_lane(bmk + t_cur, lane);
-    size_t t_nxt = nsubs > 1 ? tile_of(1) : t_cur;
-    uint32_t s_nxt = ixk[t_nxt], e_nxt = ixk[t_nxt + kSubTiles];
-    for (int n = 0; n < nsubs; n++) {
-        wait_vm0_keep(lane_bm);  // sub-chunk n (values, weights, lane bitmaps) has landed
-        write_tile_offsets(lane_bm, offs, lane);
-        if (n + 1 < nsubs) {
-            sub_issue(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), my + ((n + 1) & 1) * kSubBytes, lane);
-            stage_w(n + 1);
-            lane_bm = bitmap_of_lane(bmk + t_nxt, lane);
-        }
-        const size_t t_now = t_cur;
-        t_cur = t_nxt;
-        if (n + 2 < nsubs) {
-            t_nxt = tile_of(n + 2);
-            s_nxt = ixk[t_nxt];
-            e_nxt = ixk[t_nxt + kSubTiles];
-        }
-        sub_accumulate<NM>(bmk + t_now, lbase + (uint32_t)(n & 1) * kSubBytes, zaddr, lds_addr(offs), waddr_of(n),
-                           wgroup, acc);
-        wait_lgkm0();  // all LDS reads of buffer n&1 and of the offsets are done before they are rewritten
-    }
-}
 
 // ------------------------------------------------------------------------------- key
 // One wavefront per (KV head, token block): walks the D/32 channel sub-chunks of the block.
 // C[(kv*rows + row0 + n)*Lc + token] = sum_d K[token][d] * Bm[(kv*rows + row0 + n)*D + d],  n < NW.
-// LDS per wavefront: value double buffer + zero slot + tile offsets + the NW query rows (4*NM rows reserved).
+// LDS per wavefront: value double buffer + zero slot + the NW query rows (4*NM rows reserved).
 template <int NW>
 __global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restrict__ bmp, const char* __restrict__ nz,
                                                        const uint32_t* __restrict__ idx,
@@ -278,7 +87,7 @@ __global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restric
 // its wavefronts' sums through LDS and writes one partial row per accumulator:
 //   nsplit == 1 : C[(kv*rows+row0+n)*D + d]                       (fp16, final)
 //   nsplit  > 1 : part[((kv*rows+row0+n)*nsplit + split)*D + d]   (fp32, merged by value_merge_kernel)
-// LDS per wavefront: value double buffer + zero slot + tile offsets + double-buffered probability rows
+// LDS per wavefront: value double buffer + zero slot + double-buffered probability rows
 // (4*NM rows x kSubTiles tokens per sub-chunk).
 template <int NW, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void value_spmv_kernel(

@@ -1,0 +1,203 @@
+// Device-side building blocks shared by the SpMV kernels (spmv.hip) and the fused decode kernel
+// (fused.hip): LDS-direct staging, tile decompression and the MFMA accumulation of a sub-chunk.
+#pragma once
+#include "common.hpp"
+
+namespace mstf {
+
+#ifndef MSTF_SUB_TILES
+#define MSTF_SUB_TILES 32
+#endif
+constexpr int kSubTiles = MSTF_SUB_TILES;      // tiles per staged piece ("sub-chunk"): 16 or 32
+constexpr int kSubBytes = kSubTiles * 64 * 2;  // worst case: every tile full
+constexpr int kNzLds = 2 * kSubBytes + 16;     // value double buffer + zero slot (read by lanes whose bit is clear)
+
+#define MSTF_GLOBAL __attribute__((address_space(1)))
+
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ h4_t as_h4(uint32_t lo, uint32_t hi)
+{
+    const u32x2_t v = {lo, hi};
+    return __builtin_bit_cast(h4_t, v);
+}
+
+__device__ __forceinline__ void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// LDS-direct loads: data goes from global memory straight into LDS without passing through
+// registers; lane l of the instruction writes `size` bytes at dst + l*size.  Completion is
+// tracked by vmcnt only, the caller waits with wait_vm0() before reading the LDS.
+__device__ __forceinline__ void dma16(const void* src, void* dst_wave_uniform)
+{
+    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void* src, void* dst_wave_uniform)
+{
+    __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 4, 0, 0);
+}
+
+// Streams `bytes` (a multiple of 16, <= kSubBytes) into LDS: piece i of lane l lands at dst + (i*64 + l)*16.
+__device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char* dst, int lane)
+{
+#pragma unroll
+    for (int i = 0; i < kSubBytes / 1024; i++) {
+        if ((uint32_t)(i * 1024) < bytes) {
+            const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+            if (o < bytes) dma16(src + o, dst + i * 1024);
+        }
+    }
+}
+
+// lanes whose bit of the wave-uniform mask m is set take `yes`, the others `no`.  Written as one
+// v_cndmask on the mask register pair so the compiler keeps the decompression straight-line
+// (it otherwise turns the select into an exec-masked branch per tile).
+__device__ __forceinline__ uint32_t select_lane(uint64_t m, uint32_t yes, uint32_t no)
+{
+    uint32_t r;
+    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(m));
+    return r;
+}
+
+// LDS byte address of D[t][lane] for one tile (the zero slot when the lane's element is absent).
+//   b     : tile bitmap, MSB-first (wave-uniform, scalar registers)
+//   base  : LDS byte address of the tile's values (wave-uniform, scalar: one s_lshl2_add on idx[t])
+// rank = popcount(mask below lane) comes from v_mbcnt.
+__device__ __forceinline__ uint32_t tile_addr(uint64_t b, uint32_t base, uint32_t zaddr)
+{
+    const uint64_t m = lanes_of(b);
+    return select_lane(m, rank_below(m) * 2u + base, zaddr);
+}
+// (16-bit LDS loads cannot merge into one register here: with SRAM ECC they clear the other half,
+// hence the explicit pack of two tiles into one fp16x2 register.)
+__device__ __forceinline__ uint32_t pack_h2(_Float16 lo, _Float16 hi)
+{
+    h2_t p;
+    p.x = lo;
+    p.y = hi;
+    return as_u32(p);
+}
+
+// One staged sub-chunk (kSubTiles tiles).  For every group of 4 tiles the lane builds its own four
+// values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator
+// (lane & 3) of each accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in
+// lane 4b+j, the sums of positions 4b..4b+3 for accumulator 4m+j:
+//     acc[m][r] += sum_t D[t][4b + r] * w[4m + j][t]
+//   bm, ix : the sub-chunk's bitmaps and tile offsets (wave-uniform pointers: scalar loads, 8 tiles per
+//            batch, the next batch requested before the current one is decompressed).  Per tile the
+//            scalar unit spends one s_brev_b64 and one s_lshl2_add, the vector unit two v_mbcnt, one
+//            v_lshl_add, one v_cndmask and half a v_perm.
+//   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
+//   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
+template <int NM>
+__device__ __forceinline__ void sub_accumulate(const uint64_t* bm, const uint32_t* ix, uint32_t buf, uint32_t zaddr,
+                                               uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
+{
+    constexpr int G = kSubTiles / 8;
+    u32x16_t mv = *reinterpret_cast<const u32x16_a4*>(bm);
+    u32x8_t ov = *reinterpret_cast<const u32x8_a4*>(ix);
+    const uint32_t rel = buf - ov[0] * 4u;  // idx counts 4-byte units from the start of the KV head's values
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        u32x16_t mv_n = mv;
+        u32x8_t ov_n = ov;
+        if (g + 1 < G) {
+            // requested a whole batch ahead and pinned at the top of the batch: left to itself the
+            // scheduler sinks these loads to their first use and every batch waits out an L2 round trip
+            __builtin_amdgcn_sched_barrier(0);
+            mv_n = *reinterpret_cast<const u32x16_a4*>(bm + 8 * (g + 1));
+            ov_n = *reinterpret_cast<const u32x8_a4*>(ix + 8 * (g + 1));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int tt = g * 8;
+        uint32_t a[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(mv[2 * i], mv[2 * i + 1]), ov[i] * 4u + rel, zaddr);
+        _Float16 h[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
+        const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
+        const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup + (uint32_t)tt * 2u);
+            const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
+            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
+            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
+        }
+        mv = mv_n;
+        ov = ov_n;
+    }
+}
+
+__device__ __forceinline__ uint32_t sub_bytes(uint32_t start, uint32_t end)
+{
+    const uint32_t b = (end - start) * 4u;
+    return b > (uint32_t)kSubBytes ? (uint32_t)kSubBytes : b;  // a well-formed sub-chunk never exceeds this
+}
+
+// The decompression reads bitmaps and tile offsets through the scalar cache.  So that those loads find
+// their lines in L2 instead of waiting for HBM, every lane also touches one bitmap / one offset of the
+// coming sub-chunk with a coalesced vector load, issued together with the value stream of that sub-chunk
+// and completed by the same wait.
+struct Touch {
+    uint2 bm;
+    uint32_t ix;
+};
+__device__ __forceinline__ Touch touch_sub(const uint64_t* bm, const uint32_t* ix, int lane)
+{
+    Touch t;
+    t.bm = make_uint2(0u, 0u);
+    t.ix = 0u;
+    if (lane < kSubTiles) t.bm = *reinterpret_cast<const uint2*>(bm + lane);
+    if (lane <= kSubTiles) t.ix = ix[lane];
+    return t;
+}
+// Waits for every outstanding vector-memory operation (LDS-direct loads included).
+__device__ __forceinline__ void wait_vm0_keep(Touch& t)
+{
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(t.bm.x), "+v"(t.bm.y), "+v"(t.ix)::"memory");
+}
+
+// Walks `nsubs` sub-chunks of one KV head with a two-deep pipeline: while sub-chunk n is being
+// decompressed out of one LDS buffer, sub-chunk n+1 streams from HBM into the other.
+//   tile_of(n)    : first tile of sub-chunk n
+//   stage_w(n)    : issues the LDS-direct loads of the weights sub-chunk n needs (may be a no-op)
+//   waddr_of(n)   : LDS byte address of w[lane & 3][first tile of sub-chunk n]
+template <int NM, class TileOf, class StageW, class WAddrOf>
+__device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stage_w, WAddrOf waddr_of, uint32_t wgroup,
+                                          const uint64_t* bmk, const uint32_t* ixk, const char* nzk, char* my, int lane,
+                                          f4_t (&acc)[NM])
+{
+    const uint32_t lbase = lds_addr(my);
+    const uint32_t zaddr = lbase + 2 * kSubBytes;
+    if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
+    if (nsubs <= 0) return;
+    size_t t_cur = tile_of(0);
+    const uint32_t s0 = ixk[t_cur];
+    sub_issue(nzk + (size_t)s0 * 4u, sub_bytes(s0, ixk[t_cur + kSubTiles]), my, lane);
+    stage_w(0);
+    Touch touch = touch_sub(bmk + t_cur, ixk + t_cur, lane);
+    size_t t_nxt = nsubs > 1 ? tile_of(1) : t_cur;
+    uint32_t s_nxt = ixk[t_nxt], e_nxt = ixk[t_nxt + kSubTiles];
+    for (int n = 0; n < nsubs; n++) {
+        wait_vm0_keep(touch);  // sub-chunk n (values, weights) has landed
+        if (n + 1 < nsubs) {
+            sub_issue(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), my + ((n + 1) & 1) * kSubBytes, lane);
+            stage_w(n + 1);
+            touch = touch_sub(bmk + t_nxt, ixk + t_nxt, lane);
+        }
+        const size_t t_now = t_cur;
+        t_cur = t_nxt;
+        if (n + 2 < nsubs) {
+            t_nxt = tile_of(n + 2);
+            s_nxt = ixk[t_nxt];
+            e_nxt = ixk[t_nxt + kSubTiles];
+        }
+        sub_accumulate<NM>(bmk + t_now, ixk + t_now, lbase + (uint32_t)(n & 1) * kSubBytes, zaddr, waddr_of(n), wgroup,
+                           acc);
+        wait_lgkm0();  // all LDS reads of buffer n&1 are done before it is refilled
+    }
+}
+
+}  // namespace mstf

@@ -126,6 +126,24 @@ def value_spmv(cv, p, groups, n_rows=1, out=None):
     return C
 
 
+def decode_attention(ck, cv, q, groups, out=None, lse=None):
+    """Fused key SpMV -> scale+softmax -> value SpMV over the compressed tokens, one query row per head.
+
+    q: [Bq, D] fp16 -> out [Bq, D] fp16.  lse (optional fp32 [Bq, 2]) receives (max, sum) of every row."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    D = ck.head_dim
+    Bq = q.numel() // D
+    L = lib()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups))
+    check(L.mstf_decode_attention_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
+                                      ck.nz_off.data_ptr(), cv.bmp.data_ptr(), cv.nz.data_ptr(), cv.idx.data_ptr(),
+                                      cv.nz_off.data_ptr(), q.data_ptr(), o.data_ptr(),
+                                      lse.data_ptr() if lse is not None else None, ck.tokens, D, Bq, groups,
+                                      ws.data_ptr(), ws.numel()), "mstf_decode_attention_f16")
+    return o
+
+
 def scale_softmax(s, head_dim, out=None):
     """softmax(s / sqrt(head_dim), dtype=float32).to(float16) over the last axis."""
     assert s.dtype == torch.float16 and s.stride(-1) == 1

@@ -1,0 +1,62 @@
+"""Fused decode attention (one launch) against the oracle's dense masked attention and against the
+three-launch path, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_rowmax(a, b):
+    a = a.astype(np.float64).reshape(-1, a.shape[-1])
+    b = b.astype(np.float64).reshape(-1, b.shape[-1])
+    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
+
+
+@pytest.mark.parametrize("groups,Bkv,Lc,sparsity", [(4, 2, 1024, 0.7), (4, 3, 64, 0.7), (1, 4, 576, 0.5),
+                                                    (8, 1, 1536, 0.7), (2, 2, 512, 0.9), (4, 1, 4096, 0.7)])
+def test_fused_decode_attention(groups, Bkv, Lc, sparsity):
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    D = 128
+    Bq = Bkv * groups
+    kth = orc.kth_from_sparsity(sparsity, D)
+    K, V = orc.make_kv(900 + Lc + groups, Bkv, Lc, D)
+    q = np.random.default_rng(Lc + groups).standard_normal((Bq, D)).astype(np.float16)
+    Kp, Vp = orc.prune_rows(K, kth), orc.prune_rows(V, kth)
+    sc_ref, pr_ref, out_ref = orc.dense_masked_attention(q, Kp, Vp, groups)
+    ck = ops.compress(torch.from_numpy(K).to(dev), False, kth=kth)
+    cv = ops.compress(torch.from_numpy(V).to(dev), True, kth=kth)
+    qg = torch.from_numpy(q).to(dev)
+    lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
+    o = ops.decode_attention(ck, cv, qg, groups, lse=lse)
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3
+    o2 = ops.decode_attention(ck, cv, qg, groups)            # route without (max, sum) output
+    assert rel_rowmax(o2.cpu().numpy(), out_ref) < 2e-3
+    # (max, sum) against the oracle's scaled scores
+    w = (sc_ref.astype(np.float32) / np.float32(np.sqrt(128.0))).astype(np.float16).astype(np.float32)
+    m_ref = w.max(-1)
+    l_ref = np.exp(w - m_ref[:, None]).sum(-1)
+    got = lse.cpu().numpy()
+    assert np.abs(got[:, 0] - m_ref).max() <= 2e-2 * np.maximum(np.abs(m_ref).max(), 1)
+    assert np.abs(got[:, 1] * np.exp(got[:, 0] - m_ref) - l_ref).max() <= 5e-3 * l_ref.max()
+    # and against the three-launch path
+    s = ops.key_spmv(ck, qg.view(Bq, 1, D), groups)
+    p = ops.scale_softmax(s, D)
+    o3 = ops.value_spmv(cv, p, groups)
+    assert rel_rowmax(o.cpu().numpy(), o3.cpu().numpy()[:, 0]) < 2e-3
+
+
+def test_fused_rejects_bad_arguments():
+    from mustafar_amd._lib import lib
+    L = lib()
+    z = torch.zeros(1024, dtype=torch.int64, device="cuda:0")
+    a = z.data_ptr()
+    args = (a, a, a, a, a, a, a, a, a, a, None)
+    assert L.mstf_decode_attention_f16(None, *args, 64, 128, 4, 4, None, 0) == -4
+    assert L.mstf_decode_attention_f16(None, *args, 64, 64, 4, 4, a, 1 << 13) == -3
+    assert L.mstf_decode_attention_f16(None, *args, 100, 128, 4, 4, a, 1 << 13) == -3
+    assert L.mstf_decode_attention_f16(None, *args, 64, 128, 5, 4, a, 1 << 13) == -1
+    assert L.mstf_decode_attention_workspace_bytes(4096, 128, 256, 4) == 256 * 8 * 130 * 4
