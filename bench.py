@@ -3,11 +3,12 @@
 
 Workload (BASELINE.json configs[1]): batch 8, 32 query / 8 KV heads, head_dim 128, 4096 cached
 tokens, per-token magnitude pruning at 70 % on K and V, fp16.  A step is one decode-attention
-pass for one new token: key SpMV -> scale+softmax -> value SpMV over the compressed cache.
-Several distinct caches are rotated between steps so that reads come from HBM, not from the
-256 MB Infinity Cache.  Prints exactly one JSON line.
+pass for one new token over the compressed cache: key SpMV -> scale+softmax -> value SpMV, run as
+the fused kernel plus its split merge (or, with --unfused, as the three separate operator launches
+of the reference's call sequence).  Several distinct caches are rotated between steps so that
+reads come from HBM, not from the 256 MB Infinity Cache.  Prints exactly one JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu] [--unfused]
 """
 import argparse
 import json
@@ -19,6 +20,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_attention_bs8_ctx4096_s70_traffic.txt")
+
+
+def measured_traffic(args):
+    """HBM bytes per launch of the fused kernel from the committed counter summary (FETCH_SIZE + WRITE_SIZE,
+    calibrated on a copy of known size); only valid for the default workload, None otherwise."""
+    if (args.batch, args.ctx, args.sparsity, args.unfused) != (8, 4096, 0.7, False) or not os.path.exists(TRAFFIC_FILE):
+        return None
+    for line in open(TRAFFIC_FILE):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return int(float(line.split(":", 1)[1]))
+    return None
 
 
 def make_kv(torch, dev, Bkv, L, D, gen):
@@ -87,6 +100,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=2, help="batch entries in the CPU-baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
+    ap.add_argument("--unfused", action="store_true", help="step = the three separate operator launches")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one GPU "
@@ -124,16 +138,21 @@ def main():
     vbytes = caches[0][1].bmp.numel() * 8 + caches[0][1].idx.numel() * 4 + int(caches[0][1].total_halfs.item()) * 2
 
     q = torch.randn((Bq, 1, D), generator=gen, device=dev, dtype=torch.float32).half()
+    q2 = q.view(Bq, D)
     s = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
     p = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
     o = torch.empty((Bq, 1, D), dtype=torch.float16, device=dev)
+    o2 = o.view(Bq, D)
     it = [0]
 
     def launch(i):
         ck, cv = caches[i % args.caches]
-        ops.key_spmv(ck, q, groups, out=s)
-        ops.scale_softmax(s, D, out=p)
-        ops.value_spmv(cv, p, groups, out=o)
+        if args.unfused:
+            ops.key_spmv(ck, q, groups, out=s)
+            ops.scale_softmax(s, D, out=p)
+            ops.value_spmv(cv, p, groups, out=o)
+        else:
+            ops.decode_attention(ck, cv, q2, groups, out=o2)
 
     # One HIP graph per cache (the launches of a step are captured once and replayed), so that the timed
     # region measures the GPU work of a step rather than the Python call overhead of its four launches.
@@ -170,30 +189,47 @@ def main():
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
 
-    # ---- per-kernel averages over back-to-back launches on rotating caches (HIP events)
-    def key_only():
-        ck = caches[it[0] % args.caches][0]
+    # ---- per-kernel averages over back-to-back launches on rotating caches (HIP events on the launch stream)
+    def rot(j):
+        c = caches[it[0] % args.caches][j]
         it[0] += 1
-        ops.key_spmv(ck, q, groups, out=s)
+        return c
 
-    def value_only():
-        cv = caches[it[0] % args.caches][1]
+    def fused_only():
+        i = it[0] % args.caches
         it[0] += 1
-        ops.value_spmv(cv, p, groups, out=o)
+        ops.decode_attention_partial(caches[i][0], caches[i][1], q2, groups)
 
     n = max(args.steps, 50)
-    key_us = event_time_us(torch, key_only, n)
-    val_us = event_time_us(torch, value_only, n)
+    launch(0)
+    fused_us = event_time_us(torch, fused_only, n)
+    ws = ops.decode_attention_partial(caches[0][0], caches[0][1], q2, groups)
+    merge_us = event_time_us(torch, lambda: ops.decode_attention_merge(ws, L, D, Bq, groups, out=o2), n)
+    key_us = event_time_us(torch, lambda: ops.key_spmv(rot(0), q, groups, out=s), n)
+    val_us = event_time_us(torch, lambda: ops.value_spmv(rot(1), p, groups, out=o), n)
     sm_us = event_time_us(torch, lambda: ops.scale_softmax(s, D, out=p), n)
+
+    # a copy of known size, so that a counter run of this same command can be calibrated (outside every timed region)
+    cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    for _ in range(5):
+        torch.add(cal_src, 1, out=cal_dst)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
 
     # algorithmic bytes per launch: compressed side read once per KV head + weights in + result out (one row per head)
     key_alg = kbytes + Bq * D * 2 + Bq * L * 2
     val_alg = vbytes + Bq * L * 2 + Bq * D * 2
-    if val_us >= key_us:
+    fused_alg = kbytes + vbytes + Bq * D * 2 + Bq * D * 2
+    if not args.unfused:
+        dom, dom_us, dom_bytes = "decode_attention_kernel", fused_us, fused_alg
+    elif val_us >= key_us:
         dom, dom_us, dom_bytes = "value_spmv_kernel", val_us, val_alg
     else:
         dom, dom_us, dom_bytes = "key_spmv_kernel", key_us, key_alg
     achieved = dom_bytes / dom_us / 1e3  # GB/s
+    step_desc = ("step = the three operator launches (key SpMV, scale/softmax, value SpMV)" if args.unfused
+                 else "step = fused decode-attention kernel + split merge")
 
     out = {
         "metric": "sparse decode-attn us/layer (Llama-3-8B shape, bs=%d, ctx=%d, %d%% K/V sparsity)"
@@ -212,20 +248,22 @@ def main():
         "config": {
             "workload": "BASELINE configs[1]: Llama-3-8B GQA decode-attention layer, batch %d, 32 query / 8 KV heads, "
                         "head_dim 128, %d cached tokens, per-token magnitude pruning %.0f%% on K and V, one new token; "
-                        "step = key SpMV + scale/softmax + value SpMV; %d caches rotated (cold HBM reads); %s"
-                        % (bs, L, args.sparsity * 100, args.caches,
+                        "%s; %d caches rotated (cold HBM reads); %s"
+                        % (bs, L, args.sparsity * 100, step_desc, args.caches,
                            "steps replayed from HIP graphs" if graphs is not None else "steps launched from Python"),
             "compressed_bytes_per_token_per_kv_head": {"key": round(kbytes / Bkv / L, 2),
                                                        "value": round(vbytes / Bkv / L, 2)},
         },
         "tokens_per_s": round(bs / (wall_us * 1e-6), 1),
-        "stages_us": {"key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
+        "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
+                      "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
                       "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
-        "hbm_gbs_on_compressed_bytes": {"key_spmv": round(key_alg / key_us / 1e3, 1),
+        "hbm_gbs_on_compressed_bytes": {"fused_decode_attention": round(fused_alg / fused_us / 1e3, 1),
+                                        "key_spmv": round(key_alg / key_us / 1e3, 1),
                                         "value_spmv": round(val_alg / val_us / 1e3, 1),
-                                        "decode_attn": round((key_alg + val_alg) / wall_us / 1e3, 1)},
+                                        "whole_step": round(fused_alg / wall_us / 1e3, 1)},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args),
                      "algorithmic_bytes": int(dom_bytes), "avg_launch_us": round(dom_us, 2)},
     }
     if not args.no_cpu:

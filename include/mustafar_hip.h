@@ -122,6 +122,17 @@ int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_ha
                               const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out,
                               float* lse_out, int tokens, int head_dim, int Bq, int groups, void* workspace,
                               size_t workspace_bytes);
+/* The two phases of mstf_decode_attention_f16 as separate calls, for a caller that shards the cached
+ * tokens (each shard runs `partial` on its tokens, the (max, sum, output) triples are then combined).
+ * partial: per 512-token split s and query row: workspace = float part_o[Bq][ns][head_dim] followed by
+ *   float part_ml[Bq][ns][2] = (max, sum of exp(w - max)), part_o un-normalised; ns = ceil(tokens / 512).
+ * merge: log-sum-exp combine of the ns splits into out (fp16) and, if given, lse_out. */
+int mstf_decode_attention_partial_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                                      const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                                      const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q, int tokens,
+                                      int head_dim, int Bq, int groups, void* workspace, size_t workspace_bytes);
+int mstf_decode_attention_merge_f16(void* stream, const void* workspace, size_t workspace_bytes, mstf_half* out,
+                                    float* lse_out, int tokens, int head_dim, int Bq, int groups);
 
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),

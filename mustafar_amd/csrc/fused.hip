@@ -256,29 +256,32 @@ extern "C" size_t mstf_decode_attention_workspace_bytes(int tokens, int head_dim
     return round_up((size_t)Bq * ns * (head_dim + 2) * sizeof(float), 256);
 }
 
-extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
-                                         const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
-                                         const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
-                                         const mstf_half* q, mstf_half* out, float* lse_out, int tokens, int head_dim,
-                                         int Bq, int groups, void* workspace, size_t workspace_bytes)
+// Shared argument checks of the fused entry points.
+static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, const void* k_nz_off, const void* v_bmp,
+                        const void* v_nz, const void* v_idx, const void* v_nz_off, const void* q, int tokens,
+                        int head_dim, int Bq, int groups, const void* workspace, size_t workspace_bytes)
 {
-    if (!k_bmp || !k_nz || !k_idx || !k_nz_off || !v_bmp || !v_nz || !v_idx || !v_nz_off || !q || !out)
-        return MSTF_EINVAL;
+    if (!k_bmp || !k_nz || !k_idx || !k_nz_off || !v_bmp || !v_nz || !v_idx || !v_nz_off || !q) return MSTF_EINVAL;
     if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
     if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
     if (!aligned_to(k_bmp, 8) || !aligned_to(v_bmp, 8) || !aligned_to(k_nz, 16) || !aligned_to(v_nz, 16) ||
         !aligned_to(k_idx, 4) || !aligned_to(v_idx, 4) || !aligned_to(k_nz_off, 4) || !aligned_to(v_nz_off, 4) ||
-        !aligned_to(q, 16) || !aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4)))
+        !aligned_to(q, 16))
         return MSTF_EALIGN;
     const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
-    hipStream_t st = as_stream(stream);
+    return MSTF_OK;
+}
+
+static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                         const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
+                         const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
+                         int groups, void* workspace, int write_final)
+{
     const int Bkv = Bq / groups, nblk = tokens / 64, ns = fused_nsplit(tokens);
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * ns * head_dim;
-    // with one split and no (max, sum) requested the kernel writes the final output itself
-    const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
     const dim3 grid((unsigned)ns, (unsigned)Bkv);
     const char* knz = reinterpret_cast<const char*>(k_nz);
     const char* vnz = reinterpret_cast<const char*>(v_nz);
@@ -293,12 +296,56 @@ extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, co
         hipLaunchKernelGGL(decode_attention_kernel<2>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
                            v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, ns, write_final,
                            sq);
-    int rc = check_launch();
+    return check_launch();
+}
+
+extern "C" int mstf_decode_attention_partial_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                                 const uint32_t* k_idx, const uint32_t* k_nz_off,
+                                                 const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
+                                                 const uint32_t* v_nz_off, const mstf_half* q, int tokens, int head_dim,
+                                                 int Bq, int groups, void* workspace, size_t workspace_bytes)
+{
+    const int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, tokens, head_dim, Bq,
+                                groups, workspace, workspace_bytes);
     if (rc != MSTF_OK) return rc;
-    if (!write_final) {
-        hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, st, part_o, part_ml, oh, lse_out, ns,
-                           head_dim);
-        rc = check_launch();
-    }
-    return rc;
+    return decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, nullptr,
+                         tokens, head_dim, Bq, groups, workspace, 0);
+}
+
+extern "C" int mstf_decode_attention_merge_f16(void* stream, const void* workspace, size_t workspace_bytes,
+                                               mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq,
+                                               int groups)
+{
+    if (!out) return MSTF_EINVAL;
+    if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16) || !aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
+    const int ns = fused_nsplit(tokens);
+    const float* part_o = reinterpret_cast<const float*>(workspace);
+    const float* part_ml = part_o + (size_t)Bq * ns * head_dim;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, as_stream(stream), part_o, part_ml,
+                       reinterpret_cast<_Float16*>(out), lse_out, ns, head_dim);
+    return check_launch();
+}
+
+extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                         const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
+                                         const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
+                                         const mstf_half* q, mstf_half* out, float* lse_out, int tokens, int head_dim,
+                                         int Bq, int groups, void* workspace, size_t workspace_bytes)
+{
+    if (!out) return MSTF_EINVAL;
+    int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, tokens, head_dim, Bq, groups,
+                          workspace, workspace_bytes);
+    if (rc != MSTF_OK) return rc;
+    if (!aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
+    // with one split and no (max, sum) requested the kernel writes the final output itself
+    const int write_final = (fused_nsplit(tokens) == 1 && !lse_out) ? 1 : 0;
+    rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, out, tokens,
+                       head_dim, Bq, groups, workspace, write_final);
+    if (rc != MSTF_OK || write_final) return rc;
+    return mstf_decode_attention_merge_f16(stream, workspace, workspace_bytes, out, lse_out, tokens, head_dim, Bq,
+                                           groups);
 }

@@ -144,6 +144,30 @@ def decode_attention(ck, cv, q, groups, out=None, lse=None):
     return o
 
 
+def decode_attention_partial(ck, cv, q, groups, ws=None):
+    """First phase of decode_attention: un-normalised outputs and (max, sum) per 512-token split, left in `ws`."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    D = ck.head_dim
+    Bq = q.numel() // D
+    L = lib()
+    if ws is None:
+        ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups))
+    check(L.mstf_decode_attention_partial_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
+                                              ck.nz_off.data_ptr(), cv.bmp.data_ptr(), cv.nz.data_ptr(),
+                                              cv.idx.data_ptr(), cv.nz_off.data_ptr(), q.data_ptr(), ck.tokens, D, Bq,
+                                              groups, ws.data_ptr(), ws.numel()), "mstf_decode_attention_partial_f16")
+    return ws
+
+
+def decode_attention_merge(ws, tokens, head_dim, Bq, groups, out=None, lse=None):
+    """Second phase of decode_attention: combines the splits left in `ws` by decode_attention_partial."""
+    o = torch.empty((Bq, head_dim), dtype=torch.float16, device=ws.device) if out is None else out
+    check(lib().mstf_decode_attention_merge_f16(_stream(), ws.data_ptr(), ws.numel(), o.data_ptr(),
+                                                lse.data_ptr() if lse is not None else None, tokens, head_dim, Bq,
+                                                groups), "mstf_decode_attention_merge_f16")
+    return o
+
+
 def scale_softmax(s, head_dim, out=None):
     """softmax(s / sqrt(head_dim), dtype=float32).to(float16) over the last axis."""
     assert s.dtype == torch.float16 and s.stride(-1) == 1

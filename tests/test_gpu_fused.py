@@ -49,6 +49,33 @@ def test_fused_decode_attention(groups, Bkv, Lc, sparsity):
     assert rel_rowmax(o.cpu().numpy(), o3.cpu().numpy()[:, 0]) < 2e-3
 
 
+def test_partial_then_merge_equals_fused():
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    D, groups, Bkv, Lc = 128, 4, 2, 1600
+    Bq = Bkv * groups
+    kth = orc.kth_from_sparsity(0.7, D)
+    K, V = orc.make_kv(77, Bkv, Lc, D)
+    ck = ops.compress(torch.from_numpy(K).to(dev), False, kth=kth)
+    cv = ops.compress(torch.from_numpy(V).to(dev), True, kth=kth)
+    qg = torch.from_numpy(np.random.default_rng(3).standard_normal((Bq, D)).astype(np.float16)).to(dev)
+    lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
+    lse2 = torch.empty_like(lse)
+    o = ops.decode_attention(ck, cv, qg, groups, lse=lse)
+    ws = ops.decode_attention_partial(ck, cv, qg, groups)
+    o2 = ops.decode_attention_merge(ws, Lc, D, Bq, groups, lse=lse2)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+    # the splits themselves: (max, sum, un-normalised output) of every 512-token range, combined on the host
+    ns = (Lc // 64 + 7) // 8
+    raw = ws[: Bq * ns * (D + 2) * 4].view(torch.float32).cpu().numpy()
+    po = raw[: Bq * ns * D].reshape(Bq, ns, D).astype(np.float64)
+    ml = raw[Bq * ns * D:].reshape(Bq, ns, 2).astype(np.float64)
+    M = ml[:, :, 0].max(1, keepdims=True)
+    f = np.exp(ml[:, :, 0] - M)
+    host = (f[:, :, None] * po).sum(1) / (f * ml[:, :, 1]).sum(1, keepdims=True)
+    assert rel_rowmax(o.cpu().numpy(), host) < 1e-3
+
+
 def test_fused_rejects_bad_arguments():
     from mustafar_amd._lib import lib
     L = lib()
@@ -60,3 +87,6 @@ def test_fused_rejects_bad_arguments():
     assert L.mstf_decode_attention_f16(None, *args, 100, 128, 4, 4, a, 1 << 13) == -3
     assert L.mstf_decode_attention_f16(None, *args, 64, 128, 5, 4, a, 1 << 13) == -1
     assert L.mstf_decode_attention_workspace_bytes(4096, 128, 256, 4) == 256 * 8 * 130 * 4
+    assert L.mstf_decode_attention_partial_f16(None, *args[:9], 64, 128, 4, 4, None, 0) == -4
+    assert L.mstf_decode_attention_merge_f16(None, a, 1 << 13, None, None, 64, 128, 4, 4) == -1
+    assert L.mstf_decode_attention_merge_f16(None, a, 16, a, None, 64, 128, 4, 4) == -4
