@@ -154,9 +154,11 @@ def main():
         else:
             ops.decode_attention(ck, cv, q2, groups, out=o2)
 
-    # One HIP graph per cache (the launches of a step are captured once and replayed), so that the timed
-    # region measures the GPU work of a step rather than the Python call overhead of its four launches.
-    graphs = None
+    # The launches are captured once and replayed, so that the timed region measures the GPU work of a step
+    # rather than the Python call overhead of its launches: one graph holds one step on each of the rotating
+    # caches back to back (as a decode iteration holds the attention of consecutive layers in one graph), and
+    # one single-step graph per cache serves the remainder when K is not a multiple of the cache count.
+    graphs = ring = None
     if not args.no_graph:
         try:
             for i in range(args.caches):
@@ -168,24 +170,36 @@ def main():
                 with torch.cuda.graph(g):
                     launch(i)
                 graphs.append(g)
+            ring = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(ring):
+                for i in range(args.caches):
+                    launch(i)
         except Exception as e:  # pragma: no cover - reported in the JSON line
             print("graph capture failed (%s); launching from Python" % e, file=sys.stderr)
-            graphs = None
+            graphs = ring = None
 
-    def step():
-        i = it[0] % args.caches
-        it[0] += 1
-        if graphs is not None:
-            graphs[i].replay()
-        else:
-            launch(i)
+    def run_steps(k):
+        """Exactly k steps, continuing the rotation over the caches."""
+        if graphs is None:
+            for _ in range(k):
+                launch(it[0] % args.caches)
+                it[0] += 1
+            return
+        while k > 0:
+            i = it[0] % args.caches
+            if i == 0 and k >= args.caches:
+                ring.replay()
+                it[0] += args.caches
+                k -= args.caches
+            else:
+                graphs[i].replay()
+                it[0] += 1
+                k -= 1
 
-    for _ in range(args.warmup):
-        step()
+    run_steps(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    run_steps(args.steps)
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
 
@@ -250,7 +264,7 @@ def main():
                         "head_dim 128, %d cached tokens, per-token magnitude pruning %.0f%% on K and V, one new token; "
                         "%s; %d caches rotated (cold HBM reads); %s"
                         % (bs, L, args.sparsity * 100, step_desc, args.caches,
-                           "steps replayed from HIP graphs" if graphs is not None else "steps launched from Python"),
+                           "steps replayed from HIP graphs (%d consecutive steps per graph)" % args.caches if graphs is not None else "steps launched from Python"),
             "compressed_bytes_per_token_per_kv_head": {"key": round(kbytes / Bkv / L, 2),
                                                        "value": round(vbytes / Bkv / L, 2)},
         },

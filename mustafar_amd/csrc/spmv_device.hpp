@@ -78,15 +78,62 @@ __device__ __forceinline__ uint32_t pack_h2(_Float16 lo, _Float16 hi)
     return as_u32(p);
 }
 
-// One staged sub-chunk (kSubTiles tiles).  For every group of 4 tiles the lane builds its own four
-// values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator
-// (lane & 3) of each accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in
-// lane 4b+j, the sums of positions 4b..4b+3 for accumulator 4m+j:
+// Bitmaps and tile offsets of 8 consecutive tiles, in scalar registers (two scalar loads).
+struct Batch {
+    u32x16_t mv;  // 8 bitmaps as (lo, hi) pairs
+    u32x8_t ov;   // idx of the 8 tiles (4-byte units from the start of the KV head's values)
+};
+__device__ __forceinline__ Batch load_batch(const uint64_t* bm, const uint32_t* ix)
+{
+    Batch b;
+    b.mv = *reinterpret_cast<const u32x16_a4*>(bm);
+    b.ov = *reinterpret_cast<const u32x8_a4*>(ix);
+    return b;
+}
+
+// Decompresses 8 staged tiles and accumulates them.  For every group of 4 tiles the lane builds its own
+// four values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator (lane & 3) of each
+// accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in lane 4b+j, the sums of
+// positions 4b..4b+3 for accumulator 4m+j:
 //     acc[m][r] += sum_t D[t][4b + r] * w[4m + j][t]
-//   bm, ix : the sub-chunk's bitmaps and tile offsets (wave-uniform pointers: scalar loads, 8 tiles per
-//            batch, the next batch requested before the current one is decompressed).  Per tile the
-//            scalar unit spends one s_brev_b64 and one s_lshl2_add, the vector unit two v_mbcnt, one
-//            v_lshl_add, one v_cndmask and half a v_perm.
+// Per tile the scalar unit spends one s_brev_b64, a shift and an add, the vector unit two v_mbcnt, one
+// v_lshl_add, one v_cndmask and half a v_perm.
+//   rel    : LDS byte address of the staged values minus 4 * idx of the first staged tile
+//   zaddr  : LDS address of two zero bytes
+//   waddr  : LDS byte address of w[lane & 3][first tile of the batch]; wgroup: bytes between groups of 4 rows
+template <int NM>
+__device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, uint32_t zaddr, uint32_t waddr,
+                                                 uint32_t wgroup, f4_t (&acc)[NM])
+{
+    uint32_t a[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(b.mv[2 * i], b.mv[2 * i + 1]), b.ov[i] * 4u + rel, zaddr);
+    _Float16 h[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
+    const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
+    const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
+        const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
+    }
+}
+
+// The next batch's scalar loads, requested a whole batch ahead and pinned where they are written: left to
+// itself the scheduler sinks them to their first use and every batch waits out an L2 round trip.
+__device__ __forceinline__ Batch prefetch_batch(const uint64_t* bm, const uint32_t* ix)
+{
+    __builtin_amdgcn_sched_barrier(0);
+    const Batch b = load_batch(bm, ix);
+    __builtin_amdgcn_sched_barrier(0);
+    return b;
+}
+
+// One staged sub-chunk (kSubTiles tiles).
+//   bm, ix : the sub-chunk's bitmaps and tile offsets (wave-uniform pointers)
 //   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
 //   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
 template <int NM>
@@ -94,39 +141,14 @@ __device__ __forceinline__ void sub_accumulate(const uint64_t* bm, const uint32_
                                                uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
 {
     constexpr int G = kSubTiles / 8;
-    u32x16_t mv = *reinterpret_cast<const u32x16_a4*>(bm);
-    u32x8_t ov = *reinterpret_cast<const u32x8_a4*>(ix);
-    const uint32_t rel = buf - ov[0] * 4u;  // idx counts 4-byte units from the start of the KV head's values
+    Batch cur = load_batch(bm, ix);
+    const uint32_t rel = buf - cur.ov[0] * 4u;
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        u32x16_t mv_n = mv;
-        u32x8_t ov_n = ov;
-        if (g + 1 < G) {
-            // requested a whole batch ahead and pinned at the top of the batch: left to itself the
-            // scheduler sinks these loads to their first use and every batch waits out an L2 round trip
-            __builtin_amdgcn_sched_barrier(0);
-            mv_n = *reinterpret_cast<const u32x16_a4*>(bm + 8 * (g + 1));
-            ov_n = *reinterpret_cast<const u32x8_a4*>(ix + 8 * (g + 1));
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        const int tt = g * 8;
-        uint32_t a[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(mv[2 * i], mv[2 * i + 1]), ov[i] * 4u + rel, zaddr);
-        _Float16 h[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
-        const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
-        const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
-#pragma unroll
-        for (int m = 0; m < NM; m++) {
-            const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup + (uint32_t)tt * 2u);
-            const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
-            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
-            acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
-        }
-        mv = mv_n;
-        ov = ov_n;
+        Batch nxt = cur;
+        if (g + 1 < G) nxt = prefetch_batch(bm + 8 * (g + 1), ix + 8 * (g + 1));
+        batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
+        cur = nxt;
     }
 }
 
