@@ -159,7 +159,9 @@ int mstf_compress_value_quant(void* stream, const mstf_half* x, int B, int M, in
  * SpMM_Kernel_Quant.cuh:510-735).  Same products as the fp16 entry points on the dequantised
  * matrix (q - zero) * scale; dequant_mode 0 = fp32 arithmetic rounded once to fp16, 1 = fp16
  * arithmetic (SpMM_Kernel_Quant.cuh:190-191,238-240).  counts/units may be NULL (derived from the
- * bitmaps, as the non-_meta key entry point does).  bit in {2, 4, 8}; capacity must equal 32 / bit. */
+ * bitmaps, as the non-_meta key entry point does).  bit in {2, 4, 8}; capacity must equal 32 / bit.
+ * tile_off must be the running sum of the tiles' word counts (what the producer writes), scales and zeros
+ * 4-byte aligned, head_dim 64 or 128. */
 int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
                         const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
                         const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq, int groups,

@@ -52,6 +52,7 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p)
 }
 __device__ __forceinline__ _Float16 lds_load_h(uint32_t a) { return *(MSTF_LDS const _Float16*)(uintptr_t)a; }
 __device__ __forceinline__ uint32_t lds_load_u32(uint32_t a) { return *(MSTF_LDS const uint32_t*)(uintptr_t)a; }
+__device__ __forceinline__ uint32_t lds_load_u16(uint32_t a) { return *(MSTF_LDS const uint16_t*)(uintptr_t)a; }
 
 // ---------------------------------------------------------------- host side
 void set_last_hip_error(int e);

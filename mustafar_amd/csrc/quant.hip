@@ -1,15 +1,11 @@
-// Quantised variant of the bitmap format: producer (bitmaps, per-tile scale / zero-point, packed
-// 2/4/8-bit codes) and the key / value SpMVs with dequantisation fused into the decompression.
+// Quantised variant of the bitmap format: the producer (bitmaps, per-tile scale / zero-point, packed
+// 2/4/8-bit codes).  The consumers are in quant_spmv.hip.
 //
 // Same tiles, bitmaps and work units as the fp16 format; per tile the non-zeros are replaced by
 // codes  q = clamp(floor(v / scale + 0.5) + zero, 0, 2^bit - 1)  packed `capacity = 32 / bit` to a
 // 4-byte word (code j of a tile at bits bit*(j % capacity) of word j / capacity), and tile_off[b][t]
 // is the GLOBAL word offset of the tile inside the flat `packed` buffer.
 //
-// The consumers read the packed words directly from global memory: a tile's codes are at most 64
-// bytes (4-bit) and the lanes of a wavefront touch one or two cache lines per tile, so unlike the
-// fp16 path there is nothing worth staging; the work per tile is dominated by the unpack and
-// dequantise arithmetic.
 #include "compress_common.hpp"
 #include "spmv_common.hpp"
 
@@ -167,120 +163,6 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
     }
 }
 
-// ------------------------------------------------------------------------------- consumers
-// Dequantised element `lane` of a tile (0 when absent), as fp16.
-//   m     : the tile's lane mask (bit i <=> element i present), wave-uniform
-//   words : the tile's packed words (global memory)
-template <int MODE>
-__device__ __forceinline__ _Float16 tile_value_q(uint64_t m, const uint32_t* __restrict__ words, uint32_t scale_bits,
-                                                 uint32_t zero_bits, int bit, int cap_shift, uint32_t cmask)
-{
-    const uint32_t r = rank_below(m);
-    const bool present = lane_bit(m);
-    const uint32_t word = present ? words[r >> cap_shift] : 0u;
-    const uint32_t q = (word >> ((r & ((1u << cap_shift) - 1u)) * (uint32_t)bit)) & cmask;
-    _Float16 v;
-    if (MODE == 1) {
-        const _Float16 d = (_Float16)(int)q - as_h((uint16_t)zero_bits);  // fp16 arithmetic, rounded after each step
-        v = d * as_h((uint16_t)scale_bits);
-    } else {
-        v = (_Float16)(((float)q - half_bits_to_float(zero_bits)) * half_bits_to_float(scale_bits));
-    }
-    return present ? v : (_Float16)0;
-}
-
-// acc[n] += sum over the 64 tiles starting at `tile` of D[t][lane] * w[n][t]; w: fp16 pairs through scalar loads.
-template <int NW, int MODE>
-__device__ __forceinline__ void chunk_accumulate_q(const uint64_t* __restrict__ bm, const uint32_t* __restrict__ toff,
-                                                   const uint16_t* __restrict__ sc, const uint16_t* __restrict__ zp,
-                                                   const uint32_t* __restrict__ packed, const _Float16* w,
-                                                   size_t wstride, int bit, int cap_shift, uint32_t cmask,
-                                                   float (&acc)[NW])
-{
-#pragma unroll 1
-    for (int tt = 0; tt < 64; tt += 2) {
-        const uint64_t m0 = lanes_of(bm[tt]);
-        const uint64_t m1 = lanes_of(bm[tt + 1]);
-        h2_t p;
-        p.x = tile_value_q<MODE>(m0, packed + toff[tt], sc[tt], zp[tt], bit, cap_shift, cmask);
-        p.y = tile_value_q<MODE>(m1, packed + toff[tt + 1], sc[tt + 1], zp[tt + 1], bit, cap_shift, cmask);
-#pragma unroll
-        for (int n = 0; n < NW; n++) {
-            const uint32_t q = *reinterpret_cast<const uint32_t*>(w + (size_t)n * wstride + tt);
-            acc[n] = __builtin_amdgcn_fdot2(p, as_h2(q), acc[n], false);
-        }
-    }
-}
-
-// One wavefront per (KV head, token block).
-template <int NW, int MODE>
-__global__ __launch_bounds__(256) void key_spmv_quant_kernel(
-    const uint64_t* __restrict__ bmp, const uint32_t* __restrict__ packed, const uint32_t* __restrict__ tile_off,
-    const uint16_t* __restrict__ scales, const uint16_t* __restrict__ zeros, const _Float16* __restrict__ Bm,
-    _Float16* __restrict__ C, int Lc, int D, int nblk, int ntasks, int rows_per_kv, int row0, int bit, int cap_shift)
-{
-    const int lane = lane_id();
-    const int task = (int)blockIdx.x * 4 + wave_id();
-    if (task >= ntasks) return;
-    const int kv = task / nblk, tb = task - kv * nblk;
-    const size_t T = (size_t)Lc * D / 64;
-    const size_t t0 = (size_t)kv * T + (size_t)tb * D;
-    const _Float16* wk = Bm + ((size_t)kv * rows_per_kv + row0) * D;
-    const uint32_t cmask = (1u << bit) - 1u;
-    float acc[NW];
-#pragma unroll
-    for (int n = 0; n < NW; n++) acc[n] = 0.f;
-    for (int c = 0; c < D / 64; c++)
-        chunk_accumulate_q<NW, MODE>(bmp + t0 + c * 64, tile_off + t0 + c * 64, scales + t0 + c * 64,
-                                     zeros + t0 + c * 64, packed, wk + c * 64, (size_t)D, bit, cap_shift, cmask, acc);
-    _Float16* out = C + ((size_t)kv * rows_per_kv + row0) * Lc + (size_t)tb * 64 + lane;
-#pragma unroll
-    for (int n = 0; n < NW; n++) out[(size_t)n * Lc] = (_Float16)acc[n];
-}
-
-// grid = (token splits, D/64 halves, KV heads), WAVES wavefronts each walking nbpw token blocks.
-template <int NW, int WAVES, int MODE>
-__global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
-    const uint64_t* __restrict__ bmp, const uint32_t* __restrict__ packed, const uint32_t* __restrict__ tile_off,
-    const uint16_t* __restrict__ scales, const uint16_t* __restrict__ zeros, const _Float16* __restrict__ P,
-    _Float16* __restrict__ C, float* __restrict__ part, int Lc, int D, int nblk, int nbpw, int nsplit, int rows_per_kv,
-    int row0, int bit, int cap_shift)
-{
-    __shared__ float red[WAVES][NW * 64];
-    const int lane = lane_id();
-    const int wave = wave_id();
-    const int split = (int)blockIdx.x, half = (int)blockIdx.y, kv = (int)blockIdx.z;
-    const size_t T = (size_t)Lc * D / 64;
-    const size_t th = (size_t)kv * T + (size_t)half * 64;
-    const _Float16* wk = P + ((size_t)kv * rows_per_kv + row0) * Lc;
-    const uint32_t cmask = (1u << bit) - 1u;
-    float acc[NW];
-#pragma unroll
-    for (int n = 0; n < NW; n++) acc[n] = 0.f;
-    const int first = (split * WAVES + wave) * nbpw;
-    int last = first + nbpw;
-    if (last > nblk) last = nblk;
-    for (int tb = first; tb < last; tb++) {
-        const size_t t0 = th + (size_t)tb * D;
-        chunk_accumulate_q<NW, MODE>(bmp + t0, tile_off + t0, scales + t0, zeros + t0, packed, wk + (size_t)tb * 64,
-                                     (size_t)Lc, bit, cap_shift, cmask, acc);
-    }
-#pragma unroll
-    for (int n = 0; n < NW; n++) red[wave][n * 64 + lane] = acc[n];
-    __syncthreads();
-    for (int o = (int)threadIdx.x; o < NW * 64; o += WAVES * 64) {
-        float s = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < WAVES; wv++) s += red[wv][o];
-        const int n = o >> 6, ch = o & 63;
-        const size_t row = (size_t)kv * rows_per_kv + row0 + n;
-        if (nsplit == 1)
-            C[row * D + (size_t)half * 64 + ch] = (_Float16)s;
-        else
-            part[(row * nsplit + split) * D + (size_t)half * 64 + ch] = s;
-    }
-}
-
 // ------------------------------------------------------------------------------- host
 static int cap_shift_of(int bit)
 {
@@ -343,44 +225,6 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     return MSTF_OK;
 }
 
-static int check_quant_spmv(const void* bmp, const void* packed, const void* tile_off, const void* scales,
-                            const void* zeros, const void* Bm, const void* C, int tokens, int head_dim, int Bq,
-                            int groups, int n_rows, int bit, int capacity, int dequant_mode)
-{
-    if (!bmp || !packed || !tile_off || !scales || !zeros || !Bm || !C) return MSTF_EINVAL;
-    if (tokens <= 0 || head_dim <= 0 || Bq <= 0 || groups <= 0 || n_rows <= 0 || Bq % groups != 0) return MSTF_EINVAL;
-    if (dequant_mode != 0 && dequant_mode != 1) return MSTF_EINVAL;
-    if (cap_shift_of(bit) < 0) return MSTF_EUNSUPPORTED;
-    if (capacity != 32 / bit) return MSTF_EINVAL;
-    if (tokens % 64 != 0 || head_dim % 64 != 0) return MSTF_EUNSUPPORTED;
-    if (!aligned_to(bmp, 8) || !aligned_to(packed, 4) || !aligned_to(tile_off, 4) || !aligned_to(scales, 2) ||
-        !aligned_to(zeros, 2) || !aligned_to(Bm, 4) || !aligned_to(C, 2))
-        return MSTF_EALIGN;
-    return MSTF_OK;
-}
-
-#define MSTF_Q_KEY(NWV)                                                                                              \
-    case NWV:                                                                                                        \
-        if (dequant_mode == 1)                                                                                       \
-            hipLaunchKernelGGL((key_spmv_quant_kernel<NWV, 1>), grid, dim3(256), 0, st, bmp, packed, tile_off, sc,    \
-                               zp, b, c, M, K, nblk, ntasks, rows_per_kv, row0, bit, cs);                             \
-        else                                                                                                         \
-            hipLaunchKernelGGL((key_spmv_quant_kernel<NWV, 0>), grid, dim3(256), 0, st, bmp, packed, tile_off, sc,    \
-                               zp, b, c, M, K, nblk, ntasks, rows_per_kv, row0, bit, cs);                             \
-        break;
-
-#define MSTF_Q_VALUE(NWV, WV)                                                                                        \
-    case NWV:                                                                                                        \
-        if (dequant_mode == 1)                                                                                       \
-            hipLaunchKernelGGL((value_spmv_quant_kernel<NWV, WV, 1>), grid, dim3(WV * 64), 0, st, bmp, packed,        \
-                               tile_off, sc, zp, p, c, part, K, M, K / 64, pl.nbpw, pl.nsplit, rows_per_kv, row0,     \
-                               bit, cs);                                                                             \
-        else                                                                                                         \
-            hipLaunchKernelGGL((value_spmv_quant_kernel<NWV, WV, 0>), grid, dim3(WV * 64), 0, st, bmp, packed,        \
-                               tile_off, sc, zp, p, c, part, K, M, K / 64, pl.nbpw, pl.nsplit, rows_per_kv, row0,     \
-                               bit, cs);                                                                             \
-        break;
-
 }  // namespace mstf
 
 using namespace mstf;
@@ -407,88 +251,4 @@ extern "C" int mstf_compress_value_quant(void* stream, const mstf_half* x, int B
 {
     return compress_quant_impl<true>(stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
                                      total_words, packed, packed_capacity_words, workspace, workspace_bytes);
-}
-
-extern "C" int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
-                                   const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
-                                   const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq,
-                                   int groups, int n_rows, int bit, int capacity, int dequant_mode)
-{
-    (void)counts;  // raw counts and units follow from the bitmaps; accepted for interface compatibility
-    (void)units;
-    int rc = check_quant_spmv(bmp, packed, tile_off, scales, zeros, Bm, C, M, K, Bq, groups, n_rows, bit, capacity,
-                              dequant_mode);
-    if (rc != MSTF_OK) return rc;
-    hipStream_t st = as_stream(stream);
-    const int Bkv = Bq / groups, rows_per_kv = groups * n_rows, cs = cap_shift_of(bit);
-    const int nblk = M / 64, ntasks = Bkv * nblk;
-    const dim3 grid((unsigned)((ntasks + 3) / 4));
-    const _Float16* b = reinterpret_cast<const _Float16*>(Bm);
-    _Float16* c = reinterpret_cast<_Float16*>(C);
-    const uint16_t* sc = scales;
-    const uint16_t* zp = zeros;
-    for (int row0 = 0; row0 < rows_per_kv;) {
-        int nw = pick_nw(rows_per_kv - row0);
-        if (nw > 8) nw = 8;
-        switch (nw) {
-            MSTF_Q_KEY(8)
-            MSTF_Q_KEY(4)
-            MSTF_Q_KEY(2)
-            MSTF_Q_KEY(1)
-        }
-        if ((rc = check_launch()) != MSTF_OK) return rc;
-        row0 += nw;
-    }
-    return MSTF_OK;
-}
-
-extern "C" size_t mstf_value_spmv_quant_workspace_bytes(int M, int K, int Bq, int groups, int n_rows)
-{
-    if (M <= 0 || K <= 0 || Bq <= 0 || groups <= 0 || n_rows <= 0 || K % 64 != 0 || M % 64 != 0 || Bq % groups != 0)
-        return 0;
-    // the quantised passes cover at most 8 accumulators each; their plan never has fewer splits than a wider one
-    const ValuePlan pl = plan_value(K, M, Bq / groups, 8);
-    return pl.nsplit > 1 ? round_up((size_t)Bq * n_rows * pl.nsplit * M * sizeof(float), 256) : 0;
-}
-
-extern "C" int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed,
-                                     const uint32_t* tile_off, const uint32_t* counts, const uint32_t* units,
-                                     const mstf_half* scales, const mstf_half* zeros, const mstf_half* P, mstf_half* C,
-                                     int M, int K, int Bq, int groups, int n_rows, int bit, int capacity,
-                                     int dequant_mode, void* workspace, size_t workspace_bytes)
-{
-    (void)counts;
-    (void)units;
-    int rc = check_quant_spmv(bmp, packed, tile_off, scales, zeros, P, C, K, M, Bq, groups, n_rows, bit, capacity,
-                              dequant_mode);
-    if (rc != MSTF_OK) return rc;
-    const size_t need = mstf_value_spmv_quant_workspace_bytes(M, K, Bq, groups, n_rows);
-    if (need > 0 && (!workspace || workspace_bytes < need)) return MSTF_EWORKSPACE;
-    if (workspace && !aligned_to(workspace, 16)) return MSTF_EALIGN;
-    hipStream_t st = as_stream(stream);
-    const int Bkv = Bq / groups, rows_per_kv = groups * n_rows, cs = cap_shift_of(bit);
-    const _Float16* p = reinterpret_cast<const _Float16*>(P);
-    _Float16* c = reinterpret_cast<_Float16*>(C);
-    float* part = reinterpret_cast<float*>(workspace);
-    const uint16_t* sc = scales;
-    const uint16_t* zp = zeros;
-    const ValuePlan pl = plan_value(K, M, Bkv, 8);
-    const dim3 grid((unsigned)pl.nsplit, (unsigned)(M / 64), (unsigned)Bkv);
-    for (int row0 = 0; row0 < rows_per_kv;) {
-        int nw = pick_nw(rows_per_kv - row0);
-        if (nw > 8) nw = 8;
-        switch (nw) {
-            MSTF_Q_VALUE(8, 8)
-            MSTF_Q_VALUE(4, 8)
-            MSTF_Q_VALUE(2, 8)
-            MSTF_Q_VALUE(1, 8)
-        }
-        if ((rc = check_launch()) != MSTF_OK) return rc;
-        if (pl.nsplit > 1) {
-            launch_value_merge(st, part, c, pl.nsplit, M, rows_per_kv, row0, nw, Bkv);
-            if ((rc = check_launch()) != MSTF_OK) return rc;
-        }
-        row0 += nw;
-    }
-    return MSTF_OK;
 }

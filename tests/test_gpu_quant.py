@@ -147,6 +147,60 @@ def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc
     assert (err <= 0.5 * step * 1.01 + 2e-3 * np.abs(Kp.astype(np.float32)) + 1e-6).all()
 
 
+@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("dequant_mode", [0, 1])
+def test_quant_dequantised_values_bit_exact(bit, dequant_mode):
+    """One-hot query rows / probability rows turn the SpMVs into a read-out of the dequantised cache: every
+    output is a single product value * 1, so it must equal the oracle's decode bit for bit.  Some tiles sit far
+    from zero (zero-point beyond +-1024), which takes the kernels' literal per-mode arithmetic."""
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    B, M, D, groups = 2, 128, 128, 4
+    Kp, Vp = pruned(57 + bit, B, M)
+    k = np.arange(64)
+    steps = {2: 3, 4: 10, 8: 64}[bit]          # spread chosen so that |zero| lands between 1024 and 8192
+    Kp[1, :64, 5] = (300.0 + (k % steps) * (0.25 if bit < 8 else 0.5)).astype(np.float16)     # zero << -1024
+    Kp[1, 64:, 9] = (-90.0 - (k % {2: 4, 4: 16, 8: 64}[bit]) * 0.0625).astype(np.float16)     # zero >> 1024
+    Vp[1, 7, :64] = (512.0 + (k % steps) * 0.5).astype(np.float16)
+    Bq = B * groups
+    for is_value, x in ((0, Kp), (1, Vp)):
+        ref = orc.compress_quant(x, is_value, bit)
+        assert np.abs(ref[6].astype(np.float32)).max() > 1024      # the slow path is exercised
+        dense = np.stack([orc.decode_quant(ref[0], ref[2], ref[1], ref[5], ref[6], b, M, D, is_value, bit, dequant_mode)
+                          for b in range(B)])                      # [B, M, D]
+        g = [to_gpu(a) for a in ref]
+        if not is_value:
+            # query row n of head h selects channel 8*h + n (+ 32 per pass): four passes cover 128 channels
+            for base in range(0, D, 32):
+                q = np.zeros((Bq, 8, D), np.float16)
+                for h in range(groups):
+                    for n in range(8):
+                        q[h::groups, n, base + 8 * h + n] = 1
+                out = mpq.mustafar_key_formulation_quant_meta(g[0], g[2], g[1], g[3], g[4], g[5], g[6], to_gpu(q), M, D,
+                                                              Bq, groups, bit, 32 // bit, dequant_mode).cpu().numpy()
+                for h in range(groups):
+                    for n in range(8):
+                        for b in range(B):
+                            got = out[b * groups + h, n].view(np.uint16)
+                            want = dense[b, :, base + 8 * h + n].view(np.uint16)
+                            # +0 and -0 are the same value: an absent element is +0 here, -0 after decode of a pruned -x
+                            assert np.array_equal(got & ((got != 0x8000) * 0xFFFF), want & ((want != 0x8000) * 0xFFFF))
+        else:
+            for base in range(0, M, 32):
+                pr = np.zeros((Bq, 8, M), np.float16)
+                for h in range(groups):
+                    for n in range(8):
+                        pr[h::groups, n, base + 8 * h + n] = 1
+                out = mpq.mustafar_value_formulation_quant(g[0], g[2], g[1], g[3], g[4], g[5], g[6], to_gpu(pr), None, D, M,
+                                                           Bq, groups, bit, 32 // bit, dequant_mode).cpu().numpy()
+                for h in range(groups):
+                    for n in range(8):
+                        for b in range(B):
+                            got = out[b * groups + h, n].view(np.uint16)
+                            want = dense[b, base + 8 * h + n, :].view(np.uint16)
+                            assert np.array_equal(got & ((got != 0x8000) * 0xFFFF), want & ((want != 0x8000) * 0xFFFF))
+
+
 def test_quant_c_abi_rejects_bad_arguments():
     from mustafar_amd._lib import lib
     L = lib()
