@@ -54,6 +54,16 @@ __device__ __forceinline__ _Float16 lds_load_h(uint32_t a) { return *(MSTF_LDS c
 __device__ __forceinline__ uint32_t lds_load_u32(uint32_t a) { return *(MSTF_LDS const uint32_t*)(uintptr_t)a; }
 __device__ __forceinline__ uint32_t lds_load_u16(uint32_t a) { return *(MSTF_LDS const uint16_t*)(uintptr_t)a; }
 
+// lanes whose bit of the wave-uniform mask m is set take `yes`, the others `no`.  Written as one
+// v_cndmask on the mask register pair so the compiler keeps the decompression straight-line
+// (it otherwise turns the select into an exec-masked branch per tile).
+__device__ __forceinline__ uint32_t select_lane(uint64_t m, uint32_t yes, uint32_t no)
+{
+    uint32_t r;
+    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(m));
+    return r;
+}
+
 // ---------------------------------------------------------------- host side
 void set_last_hip_error(int e);
 

@@ -2,17 +2,18 @@
 //
 // Work unit = one (KV head, 64-token block): a 64 x 128 fp16 slab (16 KB, contiguous in x),
 // i.e. exactly 128 tiles of either format, whose packed values are contiguous in the output.
-// One wavefront owns a unit.  The slab is streamed into LDS with 16-byte loads and stored with
-// a padded row stride, so that lane = token can read its own row (and column reads over tokens)
-// without bank conflicts.
+// One wavefront owns a unit, lane = token.  The slab goes through LDS in two halves of 64 channels
+// (padded row stride, so that a lane reads its own row without bank conflicts) into registers: a lane
+// holds the 128 values of its token in 64 registers and the wavefront needs 8.25 KB of LDS.
 //
-//   count kernel   : row threshold by a 15-step radix select on the fp16 magnitudes held in
-//                    registers (lane = token), bitmaps by ballot (key) or in-lane packing (value),
-//                    padded counts and their prefix inside the unit.
+//   count kernel   : row threshold by a 15-step radix select on the fp16 magnitudes, bitmaps by ballot
+//                    (key) or in-lane packing (value), padded counts and their prefix inside the unit.
 //   scan kernels   : unit totals -> unit bases per head, head totals -> nz_off.
-//   scatter kernel : re-reads the slab, compacts the survivors of each tile into an LDS image of
-//                    the unit's output (rank by popcount of the tile bitmap below the lane) and
-//                    streams the image out with 16-byte stores.
+//   scatter kernel : re-reads the slab and compacts the survivors, half a unit (64 tiles) at a time,
+//                    into an LDS image of the output that reuses the staging buffer - key: one
+//                    rank-addressed 2-byte write per tile straight from the registers; value: every lane
+//                    walks the 64 channels of its own tile - and streams the image out with 16-byte stores.
+//                    In the fused call it also turns the unit-local tile offsets in idx into final ones.
 #include "compress_common.hpp"
 
 namespace mstf {
@@ -25,17 +26,17 @@ __global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __re
                                                             uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
                                                             uint32_t* __restrict__ unit_tot)
 {
-    __shared__ uint32_t slab[kSlabDw];
+    __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int nblk = M / 64;
     const int unit = (int)blockIdx.x;
     const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
-    slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane);
-    __builtin_amdgcn_wave_barrier();
-
     uint32_t mag[64];
-    const uint32_t thr = row_threshold(slab, lane, kth, mag);
+    unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane, mag);
+#pragma unroll
+    for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
+    const uint32_t thr = threshold_of(mag, kth);
     uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
     unit_bitmaps<IS_VALUE>(mag, thr, lane, bmA, bmB);
     uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
@@ -52,23 +53,32 @@ __global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __re
 }
 
 // ------------------------------------------------------------------------------- scans
-// grid = B, 256 threads: exclusive scan of the head's unit totals, then idx[b][t] += base of
-// its unit, idx[b][T] = head total, head_tot[b] = head total (4-byte units).
+// grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base, idx[b][T] = head total,
+// head_tot[b] = head total (4-byte units).
 __global__ __launch_bounds__(256) void scan_units_kernel(const uint32_t* __restrict__ unit_tot,
-                                                         uint32_t* __restrict__ idx, uint32_t* __restrict__ head_tot,
-                                                         int nblk, int tiles_per_unit)
+                                                         uint32_t* __restrict__ unit_base, uint32_t* __restrict__ idx,
+                                                         uint32_t* __restrict__ head_tot, int nblk, int tiles_per_unit)
 {
     extern __shared__ uint32_t base[];  // nblk entries
     const int b = (int)blockIdx.x;
     const int tid = (int)threadIdx.x;
     const uint32_t total = units_scan(unit_tot + (size_t)b * nblk, base, nblk);
-    const size_t T = (size_t)nblk * tiles_per_unit;
-    uint32_t* ib = idx + (size_t)b * (T + 1);
-    for (size_t t = tid; t < T; t += 256) ib[t] += base[t / tiles_per_unit];
+    for (int i = tid; i < nblk; i += 256) unit_base[(size_t)b * nblk + i] = base[i];
     if (tid == 0) {
-        ib[T] = total;
+        idx[(size_t)b * ((size_t)nblk * tiles_per_unit + 1) + (size_t)nblk * tiles_per_unit] = total;
         head_tot[b] = total;
     }
+}
+
+// grid = (T / 256, B): idx[b][t] += base of its unit (only when no scatter follows, which does it itself).
+__global__ __launch_bounds__(256) void finalize_idx_kernel(uint32_t* __restrict__ idx,
+                                                           const uint32_t* __restrict__ unit_base, int nblk,
+                                                           int tiles_per_unit)
+{
+    const int b = (int)blockIdx.y;
+    const size_t T = (size_t)nblk * tiles_per_unit;
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (t < T) idx[(size_t)b * (T + 1) + t] += unit_base[(size_t)b * nblk + t / tiles_per_unit];
 }
 
 // one workgroup: nz_off[b] = (sum of earlier head totals) / 4 (16-byte units); total in fp16 values.
@@ -80,56 +90,94 @@ __global__ __launch_bounds__(1024) void scan_heads_kernel(const uint32_t* __rest
 }
 
 // ------------------------------------------------------------------------------- scatter
-// grid = B * M/64 units, 64 threads.  bmp / idx / nz_off are final.
-template <bool IS_VALUE>
+// grid = B * M/64 units, 64 threads.  bmp and nz_off are final; idx is final (ADD_BASE false) or still holds
+// the unit-local offsets of the count kernel, which are completed here with unit_base (ADD_BASE true).
+template <bool IS_VALUE, bool ADD_BASE>
 __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, int M,
-                                                              const uint64_t* __restrict__ bmp,
-                                                              const uint32_t* __restrict__ idx,
+                                                              const uint64_t* __restrict__ bmp, uint32_t* idx,
+                                                              const uint32_t* __restrict__ unit_base,
                                                               const uint32_t* __restrict__ nz_off,
                                                               char* __restrict__ nz, uint64_t nz_capacity_halfs)
 {
-    __shared__ uint32_t slab[kSlabDw];
-    __shared__ __attribute__((aligned(16))) char image[64 * kD * 2];
+    // staging buffer of a half-slab, then image of that half's output (at most 64 tiles x 128 bytes);
+    // the dword behind the image takes the writes of the lanes that keep nothing
+    __shared__ __attribute__((aligned(16))) uint32_t buf[kHalfSlabDw];
+    static_assert(kHalfSlabDw * 4 >= 64 * 128 + 4, "image and dump slot fit the staging buffer");
     const int lane = lane_id();
     const int nblk = M / 64;
     const int unit = (int)blockIdx.x;
     const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
     const uint64_t* bmu = bmp + (size_t)b * T + (size_t)tb * kD;
-    const uint32_t* ixu = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
-    const uint32_t start = ixu[0];
-    uint32_t bytes = (ixu[kD] - start) * 4u;
-    if (bytes > (uint32_t)sizeof(image)) bytes = (uint32_t)sizeof(image);
-    const uint64_t head_half0 = 8ull * nz_off[b];
-    if (head_half0 + 2ull * start + bytes / 2 > nz_capacity_halfs) return;  // would not fit: leave untouched
-
-    slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane);
-    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
-        *reinterpret_cast<uint4*>(image + o) = make_uint4(0u, 0u, 0u, 0u);
-    __builtin_amdgcn_wave_barrier();
-
-    const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
-    _Float16* img = reinterpret_cast<_Float16*>(image);
-#pragma unroll 1
-    for (int tt = 0; tt < kD; tt += 8) {
-        const u32x16_t mv = *reinterpret_cast<const u32x16_a4*>(bmu + tt);
-        const u32x8_t iv = *reinterpret_cast<const u32x8_a4*>(ixu + tt);
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const int t = tt + u;
-            const uint64_t m = lanes_of(u64_of(mv[2 * u], mv[2 * u + 1]));
-            const uint32_t off = (iv[u] - start) * 2u;  // halfs inside the image
-            // element `lane` of tile t: key -> (token lane, channel t); value -> (token t%64, channel (t/64)*64+lane)
-            const int row = IS_VALUE ? (t & 63) : lane;
-            const int col = IS_VALUE ? ((t >> 6) * 64 + lane) : t;
-            const _Float16 v = sh[row * (2 * kRowDw) + col];
-            if (lane_bit(m)) img[off + rank_below(m)] = v;
-        }
+    uint32_t* ixu = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
+    // lane l holds the bitmap and the final offset of tiles l and 64 + l
+    const uint64_t bmA = bmu[lane], bmB = bmu[64 + lane];
+    uint32_t iA = ixu[lane], iB = ixu[64 + lane];
+    uint32_t end;
+    if (ADD_BASE) {
+        const uint32_t base = unit_base[(size_t)b * nblk + tb];
+        iA += base;
+        iB += base;
+        ixu[lane] = iA;
+        ixu[64 + lane] = iB;
+        const uint32_t last = __builtin_amdgcn_readlane(iB, 63);
+        end = last + padded_units(u64_of(__builtin_amdgcn_readlane((uint32_t)bmB, 63),
+                                         __builtin_amdgcn_readlane((uint32_t)(bmB >> 32), 63)));
+    } else {
+        end = ixu[kD];
     }
-    __builtin_amdgcn_wave_barrier();
-    char* dst = nz + (head_half0 + 2ull * start) * 2ull;
-    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
-        *reinterpret_cast<uint4*>(dst + o) = *reinterpret_cast<const uint4*>(image + o);
+    const uint32_t start = __builtin_amdgcn_readlane(iA, 0);
+    const uint32_t mid = __builtin_amdgcn_readlane(iB, 0);
+    const uint64_t head_half0 = 8ull * nz_off[b];
+    if (head_half0 + 2ull * end > nz_capacity_halfs) return;  // would not fit: leave untouched (uniform)
+
+    const uint32_t img = lds_addr(buf);
+    const uint32_t dump = img + 64u * 128u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const uint32_t s_h = h == 0 ? start : mid;
+        uint32_t bytes = ((h == 0 ? mid : end) - s_h) * 4u;
+        if (bytes > 64u * 128u) bytes = 64u * 128u;  // never true for offsets that follow from the bitmaps
+        uint32_t v[32];
+        half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, buf, lane);
+        __builtin_amdgcn_wave_barrier();
+        row_of_lane(buf, lane, v, 0);
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+            *(MSTF_LDS u32x4_t*)(uintptr_t)(img + o) = u32x4_t{0u, 0u, 0u, 0u};  // the padding stays +0.0
+        const uint64_t bm_l = h == 0 ? bmA : bmB;
+        const uint32_t ix_l = h == 0 ? iA : iB;
+        if (!IS_VALUE) {
+            // tile c = channel 64h + c over the 64 tokens: lane = token writes its element at the tile's rank
+#pragma unroll
+            for (int c = 0; c < 64; c++) {
+                const uint64_t m = lanes_of(u64_of(__builtin_amdgcn_readlane((uint32_t)bm_l, c),
+                                                   __builtin_amdgcn_readlane((uint32_t)(bm_l >> 32), c)));
+                const uint32_t off = img + (__builtin_amdgcn_readlane(ix_l, c) - s_h) * 4u;
+                const uint32_t a = select_lane(m, rank_below(m) * 2u + off, dump);
+                const uint32_t w = v[c >> 1];
+                *(MSTF_LDS uint16_t*)(uintptr_t)a = (uint16_t)((c & 1) ? (w >> 16) : w);
+            }
+        } else {
+            // tile (h, token = lane): the lane walks its own 64 channels, MSB of the bitmap first
+            uint32_t a = img + (ix_l - s_h) * 4u;
+            const uint32_t hi = (uint32_t)(bm_l >> 32), lo = (uint32_t)bm_l;
+#pragma unroll
+            for (int i = 0; i < 64; i++) {
+                const uint32_t word = i < 32 ? hi : lo;
+                const int32_t keep = (int32_t)(word << (i & 31)) >> 31;  // -1 when channel i is kept
+                const uint32_t w = v[i >> 1];
+                *(MSTF_LDS uint16_t*)(uintptr_t)((a & (uint32_t)keep) | (dump & ~(uint32_t)keep)) =
+                    (uint16_t)((i & 1) ? (w >> 16) : w);
+                a -= 2 * keep;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        char* dst = nz + (head_half0 + 2ull * s_h) * 2ull;
+        for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+            *reinterpret_cast<u32x4_t*>(dst + o) = *(MSTF_LDS const u32x4_t*)(uintptr_t)(img + o);
+        __builtin_amdgcn_wave_barrier();
+    }
 }
 
 // ------------------------------------------------------------------------------- dense prune
@@ -137,44 +185,43 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 __global__ __launch_bounds__(64) void prune_rows_kernel(const _Float16* __restrict__ x, _Float16* y, int64_t rows,
                                                         int kth)
 {
-    __shared__ uint32_t slab[kSlabDw];
+    __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int64_t row0 = (int64_t)blockIdx.x * 64;
-    slab_load(x, row0, rows, slab, lane);
-    __builtin_amdgcn_wave_barrier();
-    uint32_t mag[64];
+    uint32_t r[64], mag[64];
+    unit_rows(x, row0, rows, slab, lane, r);
 #pragma unroll
-    for (int j = 0; j < 64; j++) mag[j] = slab[lane * kRowDw + j] & 0x7FFF7FFFu;
+    for (int j = 0; j < 64; j++) mag[j] = r[j] & 0x7FFF7FFFu;
     const uint32_t thr = select_kth(mag, kth);
     const us2_t t2 = as_us2(thr | (thr << 16));
 #pragma unroll
-    for (int j = 0; j < 64; j++) {
-        const uint32_t d = us2_u32(as_us2(mag[j]) - t2);  // bit 15 / 31 set <=> pruned
-        uint32_t keep = 0x80008000u;                        // the sign always survives (x * 0 = +-0)
-        if (!(d & 0x8000u)) keep |= 0x00007FFFu;
-        if (!(d & 0x80000000u)) keep |= 0x7FFF0000u;
-        slab[lane * kRowDw + j] &= keep;
-    }
-    __builtin_amdgcn_wave_barrier();
-    uint4* dst = reinterpret_cast<uint4*>(y + row0 * kD);
+    for (int h = 0; h < 2; h++) {
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        const int e = j * 64 + lane;
-        const int row = e >> 4, c16 = e & 15;
-        const uint32_t* s = slab + row * kRowDw + c16 * 4;
-        if (row0 + row < rows) dst[e] = make_uint4(s[0], s[1], s[2], s[3]);
+        for (int j = 0; j < 32; j++) {
+            const uint32_t d = us2_u32(as_us2(mag[32 * h + j]) - t2);  // bit 15 / 31 set <=> pruned
+            uint32_t keep = 0x80008000u;                                // the sign always survives (x * 0 = +-0)
+            if (!(d & 0x8000u)) keep |= 0x00007FFFu;
+            if (!(d & 0x80000000u)) keep |= 0x7FFF0000u;
+            slab[lane * kHalfRowDw + j] = r[32 * h + j] & keep;
+        }
+        __builtin_amdgcn_wave_barrier();
+        uint4* dst = reinterpret_cast<uint4*>(y + row0 * kD) + h * 8;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = j * 64 + lane;
+            const int row = e >> 3, c16 = e & 7;
+            const uint32_t* sp = slab + row * kHalfRowDw + c16 * 4;
+            if (row0 + row < rows) dst[row * 16 + c16] = make_uint4(sp[0], sp[1], sp[2], sp[3]);
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
 // ------------------------------------------------------------------------------- host
-struct CompressWs {
-    uint32_t* unit_tot;
-    uint32_t* head_tot;
-};
-
+// workspace: unit totals, unit bases (both [B][M/64]), head totals [B]
 static size_t compress_ws_bytes(int B, int M)
 {
-    return round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
+    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
 }
 
 static int check_compress_args(const void* x, int B, int M, int N, int kth)
@@ -195,9 +242,9 @@ static int scatter_impl(void* stream, const mstf_half* x, int B, int M, int N, c
     if (rc != MSTF_OK) return rc;
     if (!bmp || !idx || !nz_off || !nz) return MSTF_EINVAL;
     if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz_off, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
-    hipLaunchKernelGGL(compress_scatter_kernel<IS_VALUE>, dim3((unsigned)(B * (M / 64))), dim3(64), 0,
-                       as_stream(stream), reinterpret_cast<const _Float16*>(x), M, bmp, idx, nz_off,
-                       reinterpret_cast<char*>(nz), cap);
+    hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, false>), dim3((unsigned)(B * (M / 64))), dim3(64), 0,
+                       as_stream(stream), reinterpret_cast<const _Float16*>(x), M, bmp, const_cast<uint32_t*>(idx),
+                       (const uint32_t*)nullptr, nz_off, reinterpret_cast<char*>(nz), cap);
     return check_launch();
 }
 
@@ -215,18 +262,28 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     if (!aligned_to(ws, 256)) return MSTF_EALIGN;
     hipStream_t st = as_stream(stream);
     const int nblk = M / 64;
+    const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
-    uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + round_up((size_t)B * nblk * 4, 256));
-    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st,
-                       reinterpret_cast<const _Float16*>(x), M, kth, bmp, idx, unit_tot);
+    uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
+    uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
+    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
+    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bmp, idx,
+                       unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, idx, head_tot,
-                       nblk, kD);
+    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
+                       head_tot, nblk, kD);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_heads_kernel, dim3(1), dim3(1024), 0, st, head_tot, nz_off, total_halfs, B);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    if (nz) return scatter_impl<IS_VALUE>(stream, x, B, M, N, bmp, idx, nz_off, nz, cap);
-    return MSTF_OK;
+    if (nz) {
+        if (!aligned_to(nz, 16)) return MSTF_EALIGN;
+        hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M,
+                           bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap);
+    } else {
+        hipLaunchKernelGGL(finalize_idx_kernel, dim3((unsigned)(((size_t)nblk * kD + 255) / 256), (unsigned)B), dim3(256),
+                           0, st, idx, unit_base, nblk, kD);
+    }
+    return check_launch();
 }
 
 }  // namespace mstf

@@ -9,6 +9,11 @@ constexpr int kD = 128;                  // head_dim the slab layout is built fo
 constexpr int kRowDw = kD / 2 + 1;       // dwords per LDS row: 64 of data + 1 of padding
 constexpr int kSlabDw = 64 * kRowDw;     // 16640 bytes
 
+// Half a slab: channels [64h, 64h+64) of the unit's 64 tokens.  Staging through half-slabs keeps the LDS of a
+// wavefront at 8.25 KB (19 wavefronts per CU instead of 9), the rows themselves live in registers.
+constexpr int kHalfRowDw = 32 + 1;             // dwords per LDS row: 32 of data + 1 of padding
+constexpr int kHalfSlabDw = 64 * kHalfRowDw;   // 8448 bytes
+
 typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ us2_t as_us2(uint32_t x) { return __builtin_bit_cast(us2_t, x); }
 __device__ __forceinline__ uint32_t us2_u32(us2_t x) { return __builtin_bit_cast(uint32_t, x); }
@@ -33,21 +38,70 @@ __device__ __forceinline__ void slab_load(const _Float16* x, int64_t row0, int64
     }
 }
 
+// Streams channels [64h, 64h+64) of rows [row0, row0+64) of a [rows, 128] fp16 matrix into the padded
+// half-slab (rows >= rows_valid as zeros); afterwards lane = token reads its own 32 dwords with row_of_lane.
+__device__ __forceinline__ void half_slab_load(const _Float16* x, int64_t row0, int64_t rows_valid, int h, uint32_t* slab,
+                                               int lane)
+{
+    const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD) + h * 8;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int e = j * 64 + lane;  // 16-byte piece index inside the half-slab: 8 pieces per row
+        const int row = e >> 3, c16 = e & 7;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + row < rows_valid) v = src[row * 16 + c16];
+        uint32_t* d = slab + row * kHalfRowDw + c16 * 4;
+        d[0] = v.x;
+        d[1] = v.y;
+        d[2] = v.z;
+        d[3] = v.w;
+    }
+}
+// The 32 dwords (64 channels) of this lane's token out of the staged half-slab, into r[first .. first+32).
+template <int N>
+__device__ __forceinline__ void row_of_lane(const uint32_t* slab, int lane, uint32_t (&r)[N], int first)
+{
+#pragma unroll
+    for (int j = 0; j < 32; j++) r[first + j] = slab[lane * kHalfRowDw + j];
+}
+// Both halves of the lane's row (raw fp16 pairs, signs included) through one half-slab buffer.
+__device__ __forceinline__ void unit_rows(const _Float16* x, int64_t row0, int64_t rows_valid, uint32_t* slab, int lane,
+                                          uint32_t (&r)[64])
+{
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        half_slab_load(x, row0, rows_valid, h, slab, lane);
+        __builtin_amdgcn_wave_barrier();
+        row_of_lane(slab, lane, r, 32 * h);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // kth-th smallest (1-based) of the 128 fp16 magnitudes of this lane's row.
 // mag[j] holds two 15-bit magnitudes.  Greedy MSB-first: the answer is the largest c with
-// #(mag < c) < kth.  (mag - c) wraps above 0x7FFF exactly when mag < c, so bit 15 of the packed
-// 16-bit difference is the comparison result.
+// #(mag < c) < kth.  The count comes from sums of absolute differences, one v_sad_u16 per register:
+// with S(c) = sum |mag - c|, every element below c adds 1 to S(c) - S(c-1) and every other one
+// subtracts 1, so #(mag < c) = (S(c) - S(c-1) + 128) / 2.
 __device__ __forceinline__ uint32_t select_kth(const uint32_t (&mag)[64], int kth)
 {
     uint32_t thr = 0;
 #pragma unroll 1
     for (int bit = 14; bit >= 0; bit--) {
         const uint32_t cand = thr | (1u << bit);
-        const us2_t c2 = as_us2(cand | (cand << 16));
-        us2_t cnt = as_us2(0u);
+        const uint32_t c2 = cand | (cand << 16), d2 = c2 - 0x00010001u;  // cand >= 1
+        // independent partial sums: one chain of dependent instructions would leave the wavefront waiting
+        // on its own results
+        uint32_t sc[4] = {0u, 0u, 0u, 0u}, sd[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int j = 0; j < 64; j++) cnt += (as_us2(mag[j]) - c2) >> (unsigned short)15;
-        const uint32_t below = (uint32_t)cnt.x + (uint32_t)cnt.y;
+        for (int j = 0; j < 64; j += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                sc[u] = __builtin_amdgcn_sad_u16(mag[j + u], c2, sc[u]);
+                sd[u] = __builtin_amdgcn_sad_u16(mag[j + u], d2, sd[u]);
+            }
+        }
+        const uint32_t s_c = (sc[0] + sc[1]) + (sc[2] + sc[3]), s_d = (sd[0] + sd[1]) + (sd[2] + sd[3]);
+        const uint32_t below = (s_c - s_d + 128u) >> 1;
         if (below < (uint32_t)kth) thr = cand;
     }
     return thr;
@@ -111,6 +165,17 @@ __device__ __forceinline__ void unit_bitmaps(const uint32_t (&mag)[64], uint32_t
         bmA = u64_of(w[1], w[0]);
         bmB = u64_of(w[3], w[2]);
     }
+}
+
+// Keep threshold of this lane's row from its magnitudes (kth == 0: input already pruned, keep the non-zeros).
+__device__ __forceinline__ uint32_t threshold_of(const uint32_t (&mag)[64], int kth)
+{
+    uint32_t thr = 1u;
+    if (kth > 0) {
+        thr = select_kth(mag, kth);
+        if (thr == 0u) thr = 1u;  // zeros are never stored
+    }
+    return thr;
 }
 
 // Loads this lane's row magnitudes from the slab and returns the keep threshold

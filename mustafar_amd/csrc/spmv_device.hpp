@@ -49,16 +49,6 @@ __device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char*
     }
 }
 
-// lanes whose bit of the wave-uniform mask m is set take `yes`, the others `no`.  Written as one
-// v_cndmask on the mask register pair so the compiler keeps the decompression straight-line
-// (it otherwise turns the select into an exec-masked branch per tile).
-__device__ __forceinline__ uint32_t select_lane(uint64_t m, uint32_t yes, uint32_t no)
-{
-    uint32_t r;
-    asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(m));
-    return r;
-}
-
 // LDS byte address of D[t][lane] for one tile (the zero slot when the lane's element is absent).
 //   b     : tile bitmap, MSB-first (wave-uniform, scalar registers)
 //   base  : LDS byte address of the tile's values (wave-uniform, scalar: one s_lshl2_add on idx[t])
