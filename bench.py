@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
     ap.add_argument("--unfused", action="store_true", help="step = the three separate operator launches")
+    ap.add_argument("--no-quant", action="store_true", help="skip the stage timings of the quantised format")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one GPU "
@@ -223,6 +224,43 @@ def main():
     val_us = event_time_us(torch, lambda: ops.value_spmv(rot(1), p, groups, out=o), n)
     sm_us = event_time_us(torch, lambda: ops.scale_softmax(s, D, out=p), n)
 
+    # quantised format (2- and 4-bit codes) on the same shape: producer once, then the key / value SpMVs with one
+    # row per query head through the C ABI
+    quant_us = {}
+    if not args.no_quant:
+        from mustafar_amd import compression_quant as cq
+        from mustafar_amd._lib import lib, check
+        Lh = lib()
+        Kd, Vd = make_kv(torch, dev, Bkv, L, D, gen)
+        Kd, Vd = ops.prune_rows(Kd.view(-1, D), kth).view(Bkv, L, D), ops.prune_rows(Vd.view(-1, D), kth).view(Bkv, L, D)
+        p1 = torch.softmax(torch.randn((Bq, L), generator=gen, device=dev), -1).half()
+        s1 = torch.empty((Bq, L), dtype=torch.float16, device=dev)
+        for bit in (2, 4):
+            kq = cq.convert_key_batched_quant(Kd, return_metadata=True, bit=bit)
+            vq = cq.convert_value_batched_quant(Vd, bit=bit)
+            st = torch.cuda.current_stream().cuda_stream
+            wsq = ops.workspace(dev, Lh.mstf_value_spmv_quant_workspace_bytes(D, L, Bq, groups, 1))
+
+            def qkey():
+                check(Lh.mstf_key_spmv_quant(st, kq[0].data_ptr(), kq[2].data_ptr(), kq[1].data_ptr(), None, None,
+                                             kq[5].data_ptr(), kq[6].data_ptr(), q2.data_ptr(), s1.data_ptr(), L, D, Bq,
+                                             groups, 1, bit, 32 // bit, 0), "mstf_key_spmv_quant")
+
+            def qval():
+                check(Lh.mstf_value_spmv_quant(st, vq[0].data_ptr(), vq[2].data_ptr(), vq[1].data_ptr(), None, None,
+                                               vq[5].data_ptr(), vq[6].data_ptr(), p1.data_ptr(), o2.data_ptr(), D, L, Bq,
+                                               groups, 1, bit, 32 // bit, 0, wsq.data_ptr(), wsq.numel()),
+                      "mstf_value_spmv_quant")
+
+            qkey(), qval()
+            nbytes = lambda t: sum(x.numel() * x.element_size() for x in (t[0], t[1], t[2], t[5], t[6]))
+            quant_us["%dbit" % bit] = {"key_spmv": round(event_time_us(torch, qkey, 30), 2),
+                                       "value_spmv": round(event_time_us(torch, qval, 30), 2),
+                                       "bytes_per_token_per_kv_head": {"key": round(nbytes(kq) / Bkv / L, 2),
+                                                                       "value": round(nbytes(vq) / Bkv / L, 2)}}
+            del kq, vq
+        del Kd, Vd
+
     # a copy of known size, so that a counter run of this same command can be calibrated (outside every timed region)
     cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
     cal_dst = torch.empty_like(cal_src)
@@ -272,6 +310,7 @@ def main():
         "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
                       "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
+        "quant_stages_us": quant_us,
         "hbm_gbs_on_compressed_bytes": {"fused_decode_attention": round(fused_alg / fused_us / 1e3, 1),
                                         "key_spmv": round(key_alg / key_us / 1e3, 1),
                                         "value_spmv": round(val_alg / val_us / 1e3, 1),

@@ -126,14 +126,35 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
         const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
 
+        // Bitmaps and tile offsets come in batches of 8 tiles through scalar loads, each requested one batch
+        // ahead; the chain runs across the stages and from the key tiles into the value tiles.
+        constexpr int kBatches = kSubTiles / 8, kSideBatches = D / 8;
+        Batch cur = load_batch(bmK, ixK);
+        auto stage_batches = [&](int n, uint32_t buf, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
+            const uint32_t rel = buf - cur.ov[0] * 4u;  // idx counts 4-byte units from the start of the head's values
+#pragma unroll
+            for (int g = 0; g < kBatches; g++) {
+                const int g1 = n * kBatches + g + 1;
+                Batch nxt = cur;
+                if (g1 < 2 * kSideBatches)
+                    nxt = g1 < kSideBatches ? prefetch_batch(bmK + 8 * g1, ixK + 8 * g1)
+                                            : prefetch_batch(bmV + 8 * (g1 - kSideBatches), ixV + 8 * (g1 - kSideBatches));
+                batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
+                cur = nxt;
+            }
+        };
+
 #pragma unroll
         for (int n = 0; n < kKeySubs + kValSubs; n++) {
             wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for n == 0)
+            // The buffer of sub-chunk n-1 is refilled now: every LDS read of that sub-chunk fed an MFMA that was
+            // issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would also
+            // drain the scalar prefetch of the coming batch and expose its round trip at every stage.)
+            __builtin_amdgcn_sched_barrier(0);
             if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
             const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
             if (n < kKeySubs) {
-                sub_accumulate<NM>(bm_of(n), ix_of(n), buf, zaddr, qrow + (uint32_t)n * kSubTiles * 2u,
-                                   (uint32_t)D * 8u, acc_k);
+                stage_batches(n, buf, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
             } else {
                 if (n == kKeySubs) {
                     // ---- softmax statistics of the block; lane 4b+j holds tokens 4b..4b+3 of head 4m+j
@@ -169,12 +190,13 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
                 f4_t tmp[NM];
 #pragma unroll
                 for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
-                sub_accumulate<NM>(bm_of(n), ix_of(n), buf, zaddr, wa, 4u * kPRow, tmp);
+                stage_batches(n, buf, wa, 4u * kPRow, tmp);
 #pragma unroll
                 for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
             }
-            wait_lgkm0();
+            __builtin_amdgcn_sched_barrier(0);
         }
+        wait_lgkm0();
     }
 
     // ---- workgroup combine: park (output[4*NM][D], max, sum) of every wavefront, then one thread per (head, channel)

@@ -177,25 +177,71 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float* sh)
     return r;
 }
 
+// One workgroup per row.  Rows of up to 256 * 8 * kSoftmaxPieces elements stay in registers between the three
+// passes (maximum, sum, normalise), so the scores are read from memory once; longer rows fall back to re-reading.
+constexpr int kSoftmaxPieces = 4;  // 16-byte pieces per thread: rows of up to 8192 elements
 __global__ __launch_bounds__(256) void scale_softmax_kernel(const _Float16* __restrict__ s, _Float16* p, int L,
                                                             int64_t s_stride, int64_t p_stride, float div)
 {
     __shared__ float sh[4];
     const _Float16* sr = s + (size_t)blockIdx.x * s_stride;
     _Float16* pr = p + (size_t)blockIdx.x * p_stride;
+    const int tid = (int)threadIdx.x;
+    const bool vec = (L % 8 == 0) && L <= 256 * 8 * kSoftmaxPieces && ((uintptr_t)sr % 16 == 0) && ((uintptr_t)pr % 16 == 0);
+    if (vec) {
+        typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+        float w[kSoftmaxPieces][8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxPieces; k++) {
+            const int i = (k * 256 + tid) * 8;
+            if (i < L) {
+                const h8_t v = *reinterpret_cast<const h8_t*>(sr + i);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    w[k][e] = (float)(_Float16)((float)v[e] / div);
+                    mx = fmaxf(mx, w[k][e]);
+                }
+            }
+        }
+        mx = block_reduce(mx, true, sh);
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < kSoftmaxPieces; k++) {
+            if ((k * 256 + tid) * 8 < L) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    w[k][e] = expf(w[k][e] - mx);
+                    sum += w[k][e];
+                }
+            }
+        }
+        sum = block_reduce(sum, false, sh);
+#pragma unroll
+        for (int k = 0; k < kSoftmaxPieces; k++) {
+            const int i = (k * 256 + tid) * 8;
+            if (i < L) {
+                h8_t o;
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[e] = (_Float16)(w[k][e] / sum);
+                *reinterpret_cast<h8_t*>(pr + i) = o;
+            }
+        }
+        return;
+    }
     float mx = -INFINITY;
-    for (int i = (int)threadIdx.x; i < L; i += 256) {
+    for (int i = tid; i < L; i += 256) {
         const float w = (float)(_Float16)((float)sr[i] / div);
         mx = fmaxf(mx, w);
     }
     mx = block_reduce(mx, true, sh);
     float sum = 0.f;
-    for (int i = (int)threadIdx.x; i < L; i += 256) {
+    for (int i = tid; i < L; i += 256) {
         const float w = (float)(_Float16)((float)sr[i] / div);
         sum += expf(w - mx);
     }
     sum = block_reduce(sum, false, sh);
-    for (int i = (int)threadIdx.x; i < L; i += 256) {
+    for (int i = tid; i < L; i += 256) {
         const float w = (float)(_Float16)((float)sr[i] / div);
         pr[i] = (_Float16)(expf(w - mx) / sum);
     }
