@@ -48,8 +48,11 @@ def append_compressed(old, new):
 
 
 class SparseKVCache:
-    def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256):
+    def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False):
+        """fused: the compressed part of a decode step is one launch (ops.decode_attention) whose (max, sum) joins
+        the dense window under one softmax, instead of the reference's key SpMV / softmax / value SpMV sequence."""
         self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
+        self.fused = fused
         self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
         self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
         self.k = self.v = None              # CompressedKV
@@ -73,6 +76,21 @@ class SparseKVCache:
         self.v_win = V[:, :, Lc:].contiguous().clone()
         self.compressed_length, self.kv_len = Lc, L
 
+    def _decode_fused(self, q, s_loc):
+        """One launch over the compressed tokens, then a log-sum-exp merge with the dense window."""
+        bs, n_q, _, D = q.shape
+        g = self.groups
+        lse = torch.empty((bs * n_q, 2), dtype=torch.float32, device=q.device)
+        o_c = ops.decode_attention(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), g, lse=lse)
+        m_c = lse[:, 0].view(bs, n_q, 1, 1)
+        l_c = lse[:, 1].view(bs, n_q, 1, 1)
+        w = (s_loc / ops.sqrt_head_dim(D)).float()        # fp16 division first, as for the compressed scores
+        M = torch.maximum(m_c, w.amax(-1, keepdim=True))
+        p = torch.exp(w - M)
+        a = l_c * torch.exp(m_c - M)
+        num = a * o_c.view(bs, n_q, 1, D).float() + torch.matmul(p, _repeat_kv(self.v_win, g).float())
+        return (num / (a + p.sum(-1, keepdim=True))).half()
+
     def decode(self, q, k_new, v_new):
         """q: [bs, n_q, 1, D]; k_new, v_new: [bs, n_kv, 1, D].  Returns the attention output [bs, n_q, 1, D]."""
         bs, n_q, _, D = q.shape
@@ -81,16 +99,19 @@ class SparseKVCache:
         self.k_win = torch.cat([self.k_win, k_new], dim=2)
         self.v_win = torch.cat([self.v_win, v_new], dim=2)
         s_loc = torch.matmul(q, _repeat_kv(self.k_win, g).transpose(2, 3))            # [bs, n_q, 1, Lw]
-        if Lc > 0:
+        if self.fused and Lc > 0:
+            out = self._decode_fused(q, s_loc)
+        elif Lc > 0:
             s_cmp = ops.key_spmv(self.k, q.reshape(bs * n_q, 1, D).contiguous(), g).view(bs, n_q, 1, Lc)
             s = torch.cat([s_cmp, s_loc], dim=-1)
         else:
             s = s_loc
-        p = ops.scale_softmax(s.contiguous(), D)
-        out = torch.matmul(p[..., Lc:], _repeat_kv(self.v_win, g))
-        if Lc > 0:
-            o_cmp = ops.value_spmv(self.v, p[..., :Lc].reshape(bs * n_q, 1, Lc).contiguous(), g)
-            out = out + o_cmp.view(bs, n_q, 1, D)
+        if not (self.fused and Lc > 0):
+            p = ops.scale_softmax(s.contiguous(), D)
+            out = torch.matmul(p[..., Lc:], _repeat_kv(self.v_win, g))
+            if Lc > 0:
+                o_cmp = ops.value_spmv(self.v, p[..., :Lc].reshape(bs * n_q, 1, Lc).contiguous(), g)
+                out = out + o_cmp.view(bs, n_q, 1, D)
         if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.k_win.shape[2] >= CHUNK:
             ck, cv = self._compress(self.k_win[:, :, :CHUNK].contiguous(), self.v_win[:, :, :CHUNK].contiguous())
             self.k = ck if self.k is None else append_compressed(self.k, ck)

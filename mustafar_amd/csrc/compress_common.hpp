@@ -1,13 +1,11 @@
-// Device helpers shared by the fp16 and the quantised compressors: the padded LDS slab of one
-// (KV head, 64-token block) unit, the per-row radix select and the tile bitmaps.
+// Device helpers shared by the fp16 and the quantised compressors: the staging of one
+// (KV head, 64-token block) unit through padded half-slabs in LDS, the per-row radix select and the tile bitmaps.
 #pragma once
 #include "common.hpp"
 
 namespace mstf {
 
 constexpr int kD = 128;                  // head_dim the slab layout is built for
-constexpr int kRowDw = kD / 2 + 1;       // dwords per LDS row: 64 of data + 1 of padding
-constexpr int kSlabDw = 64 * kRowDw;     // 16640 bytes
 
 // Half a slab: channels [64h, 64h+64) of the unit's 64 tokens.  Staging through half-slabs keeps the LDS of a
 // wavefront at 8.25 KB (19 wavefronts per CU instead of 9), the rows themselves live in registers.
@@ -17,26 +15,6 @@ constexpr int kHalfSlabDw = 64 * kHalfRowDw;   // 8448 bytes
 typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ us2_t as_us2(uint32_t x) { return __builtin_bit_cast(us2_t, x); }
 __device__ __forceinline__ uint32_t us2_u32(us2_t x) { return __builtin_bit_cast(uint32_t, x); }
-
-// Streams rows [row0, row0+64) of a [rows, 128] fp16 matrix into the padded LDS slab.
-// Rows >= rows_valid are filled with zeros.
-__device__ __forceinline__ void slab_load(const _Float16* x, int64_t row0, int64_t rows_valid, uint32_t* slab,
-                                          int lane)
-{
-    const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD);
-#pragma unroll
-    for (int j = 0; j < 16; j++) {
-        const int e = j * 64 + lane;  // 16-byte piece index inside the slab
-        const int row = e >> 4, c16 = e & 15;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + row < rows_valid) v = src[e];
-        uint32_t* d = slab + row * kRowDw + c16 * 4;
-        d[0] = v.x;
-        d[1] = v.y;
-        d[2] = v.z;
-        d[3] = v.w;
-    }
-}
 
 // Streams channels [64h, 64h+64) of rows [row0, row0+64) of a [rows, 128] fp16 matrix into the padded
 // half-slab (rows >= rows_valid as zeros); afterwards lane = token reads its own 32 dwords with row_of_lane.
@@ -170,20 +148,6 @@ __device__ __forceinline__ void unit_bitmaps(const uint32_t (&mag)[64], uint32_t
 // Keep threshold of this lane's row from its magnitudes (kth == 0: input already pruned, keep the non-zeros).
 __device__ __forceinline__ uint32_t threshold_of(const uint32_t (&mag)[64], int kth)
 {
-    uint32_t thr = 1u;
-    if (kth > 0) {
-        thr = select_kth(mag, kth);
-        if (thr == 0u) thr = 1u;  // zeros are never stored
-    }
-    return thr;
-}
-
-// Loads this lane's row magnitudes from the slab and returns the keep threshold
-// (kth == 0: input already pruned, keep the non-zeros).
-__device__ __forceinline__ uint32_t row_threshold(const uint32_t* slab, int lane, int kth, uint32_t (&mag)[64])
-{
-#pragma unroll
-    for (int j = 0; j < 64; j++) mag[j] = slab[lane * kRowDw + j] & 0x7FFF7FFFu;
     uint32_t thr = 1u;
     if (kth > 0) {
         thr = select_kth(mag, kth);

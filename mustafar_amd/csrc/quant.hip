@@ -25,19 +25,21 @@ __global__ __launch_bounds__(64) void quant_count_kernel(const _Float16* __restr
                                                          _Float16* __restrict__ scales, _Float16* __restrict__ zeros,
                                                          uint32_t* __restrict__ unit_tot)
 {
-    __shared__ uint32_t slab[kSlabDw];
+    __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int nblk = M / 64;
     const int unit = (int)blockIdx.x;
     const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
-    slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane);
-    __builtin_amdgcn_wave_barrier();
+    uint32_t r[64];  // this lane's token: 128 fp16 values
+    unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane, r);
 
     uint64_t bm[2];
     {
         uint32_t mag[64];
-        const uint32_t thr = row_threshold(slab, lane, kth, mag);
+#pragma unroll
+        for (int j = 0; j < 64; j++) mag[j] = r[j] & 0x7FFF7FFFu;
+        const uint32_t thr = threshold_of(mag, kth);
         unit_bitmaps<IS_VALUE>(mag, thr, lane, bm[0], bm[1]);
     }
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
@@ -47,17 +49,22 @@ __global__ __launch_bounds__(64) void quant_count_kernel(const _Float16* __restr
     uint32_t u[2];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        // element i of the tile: key -> (token i, channel h*64+lane); value -> (token lane, channel h*64+i)
+        // the half-slab of channels 64h.. back into LDS, so that lane = tile can walk its 64 elements:
+        // key -> (token i, channel 64h + lane); value -> (token lane, channel 64h + i)
+#pragma unroll
+        for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
+        __builtin_amdgcn_wave_barrier();
         float mn = INFINITY, mx = -INFINITY;
         const uint64_t m = bm[h];
         for (int i = 0; i < 64; i++) {
-            const int e = IS_VALUE ? (lane * (2 * kRowDw) + h * 64 + i) : (i * (2 * kRowDw) + h * 64 + lane);
+            const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
             const float v = (float)sh[e];
             if ((m >> (63 - i)) & 1ull) {
                 mn = fminf(mn, v);
                 mx = fmaxf(mx, v);
             }
         }
+        __builtin_amdgcn_wave_barrier();
         const uint32_t cnt = (uint32_t)__popcll(m);
         float scale = 1.f, zero = 0.f;
         if (cnt > 0) {
@@ -122,19 +129,20 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
                                                         const _Float16* __restrict__ zeros,
                                                         uint32_t* __restrict__ packed, uint64_t capacity_words)
 {
-    __shared__ uint32_t slab[kSlabDw];
+    __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int nblk = M / 64;
     const int unit = (int)blockIdx.x;
     const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
-    slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane);
-    __builtin_amdgcn_wave_barrier();
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
     const float maxq = (float)((1 << bit) - 1);
     const size_t tile0 = (size_t)b * T + (size_t)tb * kD;
-#pragma unroll
+#pragma unroll 1
     for (int h = 0; h < 2; h++) {
+        __builtin_amdgcn_wave_barrier();
+        half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, slab, lane);
+        __builtin_amdgcn_wave_barrier();
         const size_t ti = tile0 + (size_t)h * 64 + lane;
         const uint64_t m = bmp[ti];
         const uint64_t off = tile_off[ti];
@@ -147,7 +155,7 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
         uint32_t w = 0;
         for (int i = 0; i < 64; i++) {
             if (!((m >> (63 - i)) & 1ull)) continue;
-            const int e = IS_VALUE ? (lane * (2 * kRowDw) + h * 64 + i) : (i * (2 * kRowDw) + h * 64 + lane);
+            const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
             const float v = (float)sh[e];
             float q = floorf(v / sc + 0.5f) + zp;
             q = fminf(fmaxf(q, 0.f), maxq);

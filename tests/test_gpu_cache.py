@@ -16,7 +16,8 @@ def rel_rowmax(a, b):
     return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
-def test_prefill_decode_append_matches_one_shot_and_oracle():
+@pytest.mark.parametrize("fused", [False, True])
+def test_prefill_decode_append_matches_one_shot_and_oracle(fused):
     from mustafar_amd import ops
     from mustafar_amd.cache import SparseKVCache
     dev = torch.device("cuda:0")
@@ -28,7 +29,7 @@ def test_prefill_decode_append_matches_one_shot_and_oracle():
     Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
-    cache = SparseKVCache(g, D, 0.7, 0.7, res)
+    cache = SparseKVCache(g, D, 0.7, 0.7, res, fused=fused)
     cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
     assert cache.compressed_length == ((L0 - res) // 256) * 256 == 256
     checked = 0
