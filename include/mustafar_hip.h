@@ -76,6 +76,20 @@ int mstf_scatter_key_f16(void* stream, const mstf_half* x, int B, int M, int N, 
                          const uint32_t* idx, const uint32_t* nz_off, mstf_half* nz, uint64_t nz_capacity_halfs);
 int mstf_scatter_value_f16(void* stream, const mstf_half* x, int B, int M, int N, const uint64_t* bmp,
                            const uint32_t* idx, const uint32_t* nz_off, mstf_half* nz, uint64_t nz_capacity_halfs);
+/* Append to a pooled cache: the same pruning and compression of a chunk x[B, M, N] (the reference appends a
+ * 256-token chunk per head by re-concatenating every head's values, models/llama_mustafar_kernel.py:461-511),
+ * with the destination of the packed values chosen by the caller: head b's values are written at
+ * nz + 16 * dst_off[b] and must end at or before nz + 16 * dst_limit[b] (both in 16-byte units).  With one slab
+ * per head and dst_off[b] = slab start + idx_so_far[b][T] / 4 the cache grows in place; the format's nz_off[b]
+ * is the slab start.  bmp[B, M*N/64] and idx[B, M*N/64 + 1] receive the chunk's bitmaps and its offsets counted
+ * from the chunk's first value (add idx_so_far[b][T]).  A unit that would pass its head's limit is not written
+ * and *overflow (sticky, zeroed by the caller) is set to 1.  Workspace as for mstf_compress_*_f16. */
+int mstf_append_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp, uint32_t* idx,
+                        const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow,
+                        void* workspace, size_t workspace_bytes);
+int mstf_append_value_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp, uint32_t* idx,
+                          const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow,
+                          void* workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------------------ key SpMV (K1)
  * Replaces mustafar_key_formulation (kernel/kernel_wrapper/mustafar_wrapper.cu:19-133 ->

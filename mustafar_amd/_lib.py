@@ -28,6 +28,8 @@ SIGNATURES = {
     "mstf_compress_value_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _sz]),
     "mstf_scatter_key_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _u64]),
     "mstf_scatter_value_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _u64]),
+    "mstf_append_key_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "mstf_append_value_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "mstf_key_spmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     "mstf_value_spmv_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mstf_value_spmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz]),

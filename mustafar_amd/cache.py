@@ -11,9 +11,12 @@
 The appended cache is byte-identical to a one-shot compression of the same tokens (per head the new
 tiles, offsets and values follow the old ones, :461-511).
 """
+import math
+
 import torch
 
 from . import ops
+from ._lib import check, lib
 
 CHUNK = 256
 
@@ -47,18 +50,93 @@ def append_compressed(old, new):
                             total)
 
 
+class CompressedPool:
+    """One side (keys or values) of a compressed cache that grows in place.
+
+    Every head owns a slab of the packed-value pool (nz_off[b] = start of slab b, which the format allows); a chunk
+    is compressed straight to the end of each head's values by mstf_append_*_f16, so appending re-copies no packed
+    values, reads nothing back to the host and launches the same three kernels whatever the cache holds.  Only the
+    small per-tile arrays (bitmaps, offsets: 12 bytes per 64 elements) are re-concatenated, on the device.
+
+    slab_fraction: slab size relative to the dense size of max_tokens tokens (1.0 can never overflow; smaller
+    saves memory and is guarded by the sticky `overflow` flag, to be checked by the caller at a point where it
+    synchronises anyway)."""
+
+    def __init__(self, heads, head_dim, max_tokens, is_value, device, slab_fraction=1.0):
+        assert max_tokens % 64 == 0
+        self.heads, self.head_dim, self.is_value, self.max_tokens = heads, head_dim, is_value, max_tokens
+        slab16 = (int(math.ceil(max_tokens * head_dim * 2 * slab_fraction)) + 15) // 16
+        self.slab16 = slab16
+        self.nz = torch.zeros(heads * slab16 * 8, dtype=torch.float16, device=device)
+        self.nz_off = (torch.arange(heads, device=device, dtype=torch.int64) * slab16).to(torch.int32)
+        self.limit = (self.nz_off.to(torch.int64) + slab16).to(torch.int32)
+        self.bmp = torch.empty((heads, 0), dtype=torch.int64, device=device)
+        self.idx = torch.zeros((heads, 1), dtype=torch.int32, device=device)
+        self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
+        self.tokens = 0
+
+    def append(self, x, kth):
+        """x: [heads, M, head_dim] fp16, M % 64 == 0."""
+        B, M, N = x.shape
+        assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
+        x = x.contiguous()
+        L = lib()
+        Tc = M * N // 64
+        bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
+        idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
+        dst = self.nz_off + self.idx[:, -1] // 4          # 16-byte units; idx counts 4-byte units
+        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, M, N))
+        fn = L.mstf_append_value_f16 if self.is_value else L.mstf_append_key_f16
+        check(fn(torch.cuda.current_stream().cuda_stream, x.data_ptr(), B, M, N, int(kth), bmp_c.data_ptr(),
+                 idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(), self.overflow.data_ptr(),
+                 ws.data_ptr(), ws.numel()), "mstf_append_f16")
+        self.bmp = torch.cat([self.bmp, bmp_c], dim=1)
+        self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
+        self.tokens += M
+
+    def view(self):
+        """The cache as the operators take it (ops.key_spmv / value_spmv / decode_attention)."""
+        return ops.CompressedKV(self.bmp, self.idx, self.nz, self.nz_off, self.tokens, self.head_dim, self.is_value,
+                                None)
+
+    def head_values(self, b):
+        """Packed values of head b (a host read: for tests and debugging)."""
+        n = 2 * int(self.idx[b, -1])
+        start = 8 * int(self.nz_off[b])
+        return self.nz[start:start + n]
+
+
 class SparseKVCache:
-    def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False):
+    def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False,
+                 max_tokens=0):
         """fused: the compressed part of a decode step is one launch (ops.decode_attention) whose (max, sum) joins
-        the dense window under one softmax, instead of the reference's key SpMV / softmax / value SpMV sequence."""
+        the dense window under one softmax, instead of the reference's key SpMV / softmax / value SpMV sequence.
+        max_tokens > 0: the compressed part lives in pre-allocated pools (CompressedPool) and grows in place."""
         self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
         self.fused = fused
+        self.max_tokens = max_tokens
+        self.k_pool = self.v_pool = None
         self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
         self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
         self.k = self.v = None              # CompressedKV
         self.k_win = self.v_win = None      # [bs, n_kv, Lw, D] dense
         self.compressed_length = 0
         self.kv_len = 0
+
+    def _grow(self, K, V):
+        """Adds the tokens K, V [bs, n_kv, M, D] to the compressed part."""
+        bs, n_kv, M, D = K.shape
+        if self.max_tokens > 0:
+            if self.k_pool is None:
+                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, K.device)
+                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, K.device)
+            self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k)
+            self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v)
+            self.k, self.v = self.k_pool.view(), self.v_pool.view()
+            return
+        ck, cv = self._compress(K, V)
+        self.k = ck if self.k is None else append_compressed(self.k, ck)
+        self.v = cv if self.v is None else append_compressed(self.v, cv)
 
     def _compress(self, K, V):
         bs, n_kv, L, D = K.shape
@@ -71,7 +149,7 @@ class SparseKVCache:
         L = K.shape[2]
         Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
         if Lc > 0:
-            self.k, self.v = self._compress(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
+            self._grow(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
         self.k_win = K[:, :, Lc:].contiguous().clone()
         self.v_win = V[:, :, Lc:].contiguous().clone()
         self.compressed_length, self.kv_len = Lc, L
@@ -113,9 +191,7 @@ class SparseKVCache:
                 o_cmp = ops.value_spmv(self.v, p[..., :Lc].reshape(bs * n_q, 1, Lc).contiguous(), g)
                 out = out + o_cmp.view(bs, n_q, 1, D)
         if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.k_win.shape[2] >= CHUNK:
-            ck, cv = self._compress(self.k_win[:, :, :CHUNK].contiguous(), self.v_win[:, :, :CHUNK].contiguous())
-            self.k = ck if self.k is None else append_compressed(self.k, ck)
-            self.v = cv if self.v is None else append_compressed(self.v, cv)
+            self._grow(self.k_win[:, :, :CHUNK].contiguous(), self.v_win[:, :, :CHUNK].contiguous())
             self.k_win = self.k_win[:, :, CHUNK:].contiguous()
             self.v_win = self.v_win[:, :, CHUNK:].contiguous()
             self.compressed_length += CHUNK

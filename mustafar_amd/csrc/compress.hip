@@ -92,12 +92,16 @@ __global__ __launch_bounds__(1024) void scan_heads_kernel(const uint32_t* __rest
 // ------------------------------------------------------------------------------- scatter
 // grid = B * M/64 units, 64 threads.  bmp and nz_off are final; idx is final (ADD_BASE false) or still holds
 // the unit-local offsets of the count kernel, which are completed here with unit_base (ADD_BASE true).
+// head_limit (nullable): end of head b's slab in 16-byte units from nz; a unit whose values would pass it is
+// skipped and *overflow is set.
 template <bool IS_VALUE, bool ADD_BASE>
 __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, int M,
                                                               const uint64_t* __restrict__ bmp, uint32_t* idx,
                                                               const uint32_t* __restrict__ unit_base,
                                                               const uint32_t* __restrict__ nz_off,
-                                                              char* __restrict__ nz, uint64_t nz_capacity_halfs)
+                                                              char* __restrict__ nz, uint64_t nz_capacity_halfs,
+                                                              const uint32_t* __restrict__ head_limit,
+                                                              uint32_t* __restrict__ overflow)
 {
     // staging buffer of a half-slab, then image of that half's output (at most 64 tiles x 128 bytes);
     // the dword behind the image takes the writes of the lanes that keep nothing
@@ -130,6 +134,11 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
     const uint32_t mid = __builtin_amdgcn_readlane(iB, 0);
     const uint64_t head_half0 = 8ull * nz_off[b];
     if (head_half0 + 2ull * end > nz_capacity_halfs) return;  // would not fit: leave untouched (uniform)
+    if (head_limit && head_half0 + 2ull * end > 8ull * head_limit[b]) {
+        // the head's values would run past the end of its slab: nothing of this unit is written, the caller is told
+        if (lane == 0) atomicOr(overflow, 1u);
+        return;
+    }
 
     const uint32_t img = lds_addr(buf);
     const uint32_t dump = img + 64u * 128u;
@@ -244,7 +253,8 @@ static int scatter_impl(void* stream, const mstf_half* x, int B, int M, int N, c
     if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz_off, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
     hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, false>), dim3((unsigned)(B * (M / 64))), dim3(64), 0,
                        as_stream(stream), reinterpret_cast<const _Float16*>(x), M, bmp, const_cast<uint32_t*>(idx),
-                       (const uint32_t*)nullptr, nz_off, reinterpret_cast<char*>(nz), cap);
+                       (const uint32_t*)nullptr, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
+                       (uint32_t*)nullptr);
     return check_launch();
 }
 
@@ -278,7 +288,8 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     if (nz) {
         if (!aligned_to(nz, 16)) return MSTF_EALIGN;
         hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M,
-                           bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap);
+                           bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
+                           (uint32_t*)nullptr);
     } else {
         hipLaunchKernelGGL(finalize_idx_kernel, dim3((unsigned)(((size_t)nblk * kD + 255) / 256), (unsigned)B), dim3(256),
                            0, st, idx, unit_base, nblk, kD);
@@ -286,9 +297,57 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     return check_launch();
 }
 
+// Compresses a chunk and places head b's packed values at nz + 16 * dst_off[b] (limit: nz + 16 * dst_limit[b]).
+template <bool IS_VALUE>
+static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp, uint32_t* idx,
+                       const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow, void* ws,
+                       size_t ws_bytes)
+{
+    int rc = check_compress_args(x, B, M, N, kth);
+    if (rc != MSTF_OK) return rc;
+    if (!bmp || !idx || !dst_off || !dst_limit || !nz || !overflow) return MSTF_EINVAL;
+    if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(dst_off, 4) || !aligned_to(dst_limit, 4) ||
+        !aligned_to(nz, 16) || !aligned_to(overflow, 4))
+        return MSTF_EALIGN;
+    if (!ws || ws_bytes < compress_ws_bytes(B, M)) return MSTF_EWORKSPACE;
+    if (!aligned_to(ws, 256)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int nblk = M / 64;
+    const size_t ub = round_up((size_t)B * nblk * 4, 256);
+    uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
+    uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
+    uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
+    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
+    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bmp, idx,
+                       unit_tot);
+    if ((rc = check_launch()) != MSTF_OK) return rc;
+    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
+                       head_tot, nblk, kD);
+    if ((rc = check_launch()) != MSTF_OK) return rc;
+    hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bmp,
+                       idx, unit_base, dst_off, reinterpret_cast<char*>(nz), ~0ull, dst_limit, overflow);
+    return check_launch();
+}
+
 }  // namespace mstf
 
 using namespace mstf;
+
+extern "C" int mstf_append_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
+                                   uint32_t* idx, const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz,
+                                   uint32_t* overflow, void* workspace, size_t workspace_bytes)
+{
+    return append_impl<false>(stream, x, B, M, N, kth, bmp, idx, dst_off, dst_limit, nz, overflow, workspace,
+                              workspace_bytes);
+}
+
+extern "C" int mstf_append_value_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
+                                     uint32_t* idx, const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz,
+                                     uint32_t* overflow, void* workspace, size_t workspace_bytes)
+{
+    return append_impl<true>(stream, x, B, M, N, kth, bmp, idx, dst_off, dst_limit, nz, overflow, workspace,
+                             workspace_bytes);
+}
 
 extern "C" size_t mstf_compress_workspace_bytes(int B, int M, int N)
 {

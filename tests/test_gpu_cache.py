@@ -16,8 +16,8 @@ def rel_rowmax(a, b):
     return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
-@pytest.mark.parametrize("fused", [False, True])
-def test_prefill_decode_append_matches_one_shot_and_oracle(fused):
+@pytest.mark.parametrize("fused,pooled", [(False, False), (True, False), (True, True)])
+def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled):
     from mustafar_amd import ops
     from mustafar_amd.cache import SparseKVCache
     dev = torch.device("cuda:0")
@@ -29,7 +29,7 @@ def test_prefill_decode_append_matches_one_shot_and_oracle(fused):
     Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
-    cache = SparseKVCache(g, D, 0.7, 0.7, res, fused=fused)
+    cache = SparseKVCache(g, D, 0.7, 0.7, res, fused=fused, max_tokens=1024 if pooled else 0)
     cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
     assert cache.compressed_length == ((L0 - res) // 256) * 256 == 256
     checked = 0
@@ -48,18 +48,44 @@ def test_prefill_decode_append_matches_one_shot_and_oracle(fused):
     assert cache.kv_len == total and cache.compressed_length == 768      # two appends happened
     assert cache.k_win.shape[2] == total - 768
     assert checked >= 10
-    # incremental == one-shot, byte for byte
+    # incremental == one-shot, byte for byte (in a pooled cache every head's values sit in its own slab)
     Lc = cache.compressed_length
-    for side, is_value in ((cache.k, 0), (cache.v, 1)):
+    for side, pool, is_value in ((cache.k, cache.k_pool, 0), (cache.v, cache.v_pool, 1)):
         src = V if is_value else K
         rb, ri, rnz, roff = orc.compress(orc.prune_rows(np.ascontiguousarray(src[:, :Lc]), 89), is_value)
         assert np.array_equal(side.bmp.cpu().numpy(), rb)
         assert np.array_equal(side.idx.cpu().numpy(), ri)
-        assert np.array_equal(side.nz_off.cpu().numpy(), roff)
-        assert np.array_equal(side.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
-    one = ops.compress(Kt[:, :, :Lc].reshape(bs * n_kv, Lc, D).contiguous(), False, kth=89)
-    assert torch.equal(one.bmp, cache.k.bmp) and torch.equal(one.idx, cache.k.idx)
-    assert torch.equal(one.packed(), cache.k.packed())
+        if pooled:
+            assert int(pool.overflow) == 0
+            for b in range(bs * n_kv):
+                want = rnz[8 * int(roff[b]):8 * int(roff[b]) + 2 * int(ri[b, -1])]
+                assert np.array_equal(pool.head_values(b).cpu().numpy().view(np.uint16), want.view(np.uint16))
+        else:
+            assert np.array_equal(side.nz_off.cpu().numpy(), roff)
+            assert np.array_equal(side.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+    if not pooled:
+        one = ops.compress(Kt[:, :, :Lc].reshape(bs * n_kv, Lc, D).contiguous(), False, kth=89)
+        assert torch.equal(one.bmp, cache.k.bmp) and torch.equal(one.idx, cache.k.idx)
+        assert torch.equal(one.packed(), cache.k.packed())
+
+
+def test_pool_overflow_is_flagged_and_leaves_other_heads_alone():
+    from mustafar_amd.cache import CompressedPool
+    dev = torch.device("cuda:0")
+    heads, D = 3, 128
+    K, _ = orc.make_kv(9, heads, 256, D)
+    Kt = torch.from_numpy(K).to(dev)
+    pool = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)    # 30 % survive: 64 tokens fit, 256 do not
+    pool.append(Kt[:, :64], 89)
+    assert int(pool.overflow) == 0
+    before = pool.nz.clone()
+    pool.append(Kt[:, 64:256], 89)
+    assert int(pool.overflow) == 1
+    # what was there stays: the values of the first 64 tokens of every head
+    for b in range(heads):
+        n = 2 * int(pool.idx[b, 128])
+        s0 = 8 * int(pool.nz_off[b])
+        assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
 
 
 def test_short_prompt_stays_dense_until_first_chunk():
