@@ -147,6 +147,19 @@ int mstf_decode_attention_partial_f16(void* stream, const uint64_t* k_bmp, const
                                       int head_dim, int Bq, int groups, void* workspace, size_t workspace_bytes);
 int mstf_decode_attention_merge_f16(void* stream, const void* workspace, size_t workspace_bytes, mstf_half* out,
                                     float* lse_out, int tokens, int head_dim, int Bq, int groups);
+/* The whole attention of a decode step, compressed tokens and dense local window under one softmax
+ * (models/llama_mustafar_kernel.py:391-441: key SpMV | q.K_win^T, / sqrt(d), softmax, value SpMV + P_win.V_win):
+ * the fused kernel over the `tokens` compressed tokens, a dense kernel over the window, one merge.
+ * k_win, v_win: [Bq / groups][win_stride][head_dim] fp16, the first win_len tokens of every KV head valid (the new
+ * token included).  tokens may be 0 (nothing compressed yet; the compressed-side pointers are then ignored).
+ * Workspace: mstf_decode_attention_window_workspace_bytes(tokens, largest win_len, head_dim, Bq, groups). */
+size_t mstf_decode_attention_window_workspace_bytes(int tokens, int max_window, int head_dim, int Bq, int groups);
+int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                                     const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                                     const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q,
+                                     const mstf_half* k_win, const mstf_half* v_win, int win_len, int win_stride,
+                                     mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq, int groups,
+                                     void* workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),

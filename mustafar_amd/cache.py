@@ -108,12 +108,17 @@ class CompressedPool:
 
 class SparseKVCache:
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False,
-                 max_tokens=0):
+                 max_tokens=0, window_kernel=False):
         """fused: the compressed part of a decode step is one launch (ops.decode_attention) whose (max, sum) joins
         the dense window under one softmax, instead of the reference's key SpMV / softmax / value SpMV sequence.
-        max_tokens > 0: the compressed part lives in pre-allocated pools (CompressedPool) and grows in place."""
+        max_tokens > 0: the compressed part lives in pre-allocated pools (CompressedPool) and grows in place.
+        window_kernel: the dense window lives in a pre-allocated buffer and the whole attention of a step - compressed
+        tokens and window - is ops.decode_attention_window (three launches, no torch operators)."""
         self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
-        self.fused = fused
+        self.fused = fused or window_kernel
+        self.window_kernel = window_kernel
+        self._kbuf = self._vbuf = None      # [bs * n_kv, residual_length + CHUNK, D], first _wlen tokens valid
+        self._wlen = 0
         self.max_tokens = max_tokens
         self.k_pool = self.v_pool = None
         self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
@@ -150,9 +155,44 @@ class SparseKVCache:
         Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
         if Lc > 0:
             self._grow(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
+        self.compressed_length, self.kv_len = Lc, L
+        if self.window_kernel:
+            bs, n_kv, _, D = K.shape
+            cap = max(self.residual_length + CHUNK, L - Lc + 1)
+            self._kbuf = torch.empty((bs * n_kv, cap, D), dtype=torch.float16, device=K.device)
+            self._vbuf = torch.empty_like(self._kbuf)
+            self._wlen = L - Lc
+            self._kbuf[:, :self._wlen] = K[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
+            self._vbuf[:, :self._wlen] = V[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
+            self._shape = (bs, n_kv, D)
+            self._window_views()
+            return
         self.k_win = K[:, :, Lc:].contiguous().clone()
         self.v_win = V[:, :, Lc:].contiguous().clone()
-        self.compressed_length, self.kv_len = Lc, L
+
+    def _window_views(self):
+        bs, n_kv, D = self._shape
+        self.k_win = self._kbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
+        self.v_win = self._vbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
+
+    def _decode_window_kernel(self, q, k_new, v_new):
+        bs, n_q, _, D = q.shape
+        n_kv = self._shape[1]
+        self.kv_len += 1
+        self._kbuf[:, self._wlen] = k_new.reshape(bs * n_kv, D)
+        self._vbuf[:, self._wlen] = v_new.reshape(bs * n_kv, D)
+        self._wlen += 1
+        out = ops.decode_attention_window(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), self._kbuf, self._vbuf,
+                                          self._wlen, self.groups).view(bs, n_q, 1, D)
+        if (self.kv_len - self.residual_length - self.compressed_length) % CHUNK == 0 and self._wlen >= CHUNK:
+            self._grow(self._kbuf[:, :CHUNK].reshape(bs, n_kv, CHUNK, D), self._vbuf[:, :CHUNK].reshape(bs, n_kv, CHUNK, D))
+            rest = self._wlen - CHUNK
+            self._kbuf[:, :rest] = self._kbuf[:, CHUNK:self._wlen].clone()
+            self._vbuf[:, :rest] = self._vbuf[:, CHUNK:self._wlen].clone()
+            self._wlen = rest
+            self.compressed_length += CHUNK
+        self._window_views()
+        return out
 
     def _decode_fused(self, q, s_loc):
         """One launch over the compressed tokens, then a log-sum-exp merge with the dense window."""
@@ -171,6 +211,8 @@ class SparseKVCache:
 
     def decode(self, q, k_new, v_new):
         """q: [bs, n_q, 1, D]; k_new, v_new: [bs, n_kv, 1, D].  Returns the attention output [bs, n_q, 1, D]."""
+        if self.window_kernel:
+            return self._decode_window_kernel(q, k_new, v_new)
         bs, n_q, _, D = q.shape
         g, Lc = self.groups, self.compressed_length
         self.kv_len += 1

@@ -265,6 +265,94 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restri
     }
 }
 
+// Dense local window of the decode step (the tokens that are not compressed yet,
+// models/llama_mustafar_kernel.py:391-441): one wavefront per (KV head, 64-token block of the window) leaves the
+// same (max, sum, un-normalised output) triple as a split of the compressed tokens, in split slot split0 + block,
+// so that the merge kernel combines compressed tokens and window under one softmax.
+//   key phase   : lane = token reads its own row of k_win, fp32 dot products with the query rows (scalar loads);
+//   value phase : lane = channel pair, the 64 weights are broadcast one token at a time.
+// k_win, v_win: [Bkv][win_stride][D] fp16, the first win_len tokens of every head valid.  G4 = heads computed (>= groups).
+template <int G4>
+__global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __restrict__ k_win,
+                                                              const _Float16* __restrict__ v_win,
+                                                              const _Float16* __restrict__ q, float* __restrict__ part_o,
+                                                              float* __restrict__ part_ml, int win_len, int win_stride,
+                                                              int groups, int nsplit, int split0, float sqrt_d)
+{
+    constexpr int D = kFusedD;
+    const int lane = lane_id();
+    const int blk = (int)blockIdx.x, kv = (int)blockIdx.y;
+    const int tok = blk * 64 + lane;
+    const bool valid = tok < win_len;
+    int nt = win_len - blk * 64;
+    nt = nt > 64 ? 64 : nt;
+    const size_t head0 = (size_t)kv * win_stride;
+    // ---- scores of this lane's token for the G4 query heads
+    float s[G4];
+#pragma unroll
+    for (int h = 0; h < G4; h++) s[h] = 0.f;
+    const u32x4_t* krow = reinterpret_cast<const u32x4_t*>(k_win + (head0 + (valid ? tok : 0)) * D);
+    const uint32_t* qw = reinterpret_cast<const uint32_t*>(q + (size_t)kv * groups * D);  // wave-uniform
+#pragma unroll 4
+    for (int c = 0; c < D / 8; c++) {
+        const u32x4_t kk = krow[c];
+#pragma unroll
+        for (int h = 0; h < G4; h++) {
+            if (h < groups) {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    s[h] = __builtin_amdgcn_fdot2(as_h2(kk[e]), as_h2(qw[h * (D / 2) + c * 4 + e]), s[h], false);
+            }
+        }
+    }
+    // ---- block statistics and fp16 weights, as in the compressed path
+    uint32_t e16[G4];
+    float mrun[G4], lrun[G4];
+#pragma unroll
+    for (int h = 0; h < G4; h++) {
+        const _Float16 s16 = (_Float16)s[h];
+        const float w = valid ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
+        float mx = w;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const _Float16 eh = valid ? (_Float16)__expf(w - mx) : (_Float16)0.f;
+        float sum = (float)eh;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        mrun[h] = mx;
+        lrun[h] = sum;
+        e16[h] = (uint32_t)__builtin_bit_cast(uint16_t, eh);
+    }
+    // ---- value phase: lane owns channels 2*lane, 2*lane+1
+    float acc[G4][2];
+#pragma unroll
+    for (int h = 0; h < G4; h++) acc[h][0] = acc[h][1] = 0.f;
+    const uint32_t* vbase = reinterpret_cast<const uint32_t*>(v_win + (head0 + (size_t)blk * 64) * D) + lane;
+#pragma unroll 4
+    for (int t = 0; t < nt; t++) {
+        const h2_t vv = as_h2(vbase[(size_t)t * (D / 2)]);
+        const float v0 = (float)vv.x, v1 = (float)vv.y;
+#pragma unroll
+        for (int h = 0; h < G4; h++) {
+            const float pw = (float)as_h((uint16_t)__builtin_amdgcn_readlane(e16[h], t));
+            acc[h][0] += pw * v0;
+            acc[h][1] += pw * v1;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < G4; h++) {
+        if (h < groups) {
+            const size_t slot = ((size_t)kv * groups + h) * nsplit + split0 + blk;
+            part_o[slot * D + 2 * lane] = acc[h][0];
+            part_o[slot * D + 2 * lane + 1] = acc[h][1];
+            if (lane == 0) {
+                part_ml[slot * 2] = mrun[h];
+                part_ml[slot * 2 + 1] = lrun[h];
+            }
+        }
+    }
+}
+
 static int fused_nsplit(int tokens) { return (tokens / 64 + kFusedWaves - 1) / kFusedWaves; }
 
 }  // namespace mstf
@@ -299,11 +387,14 @@ static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, 
 static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
                          const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
                          const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
-                         int groups, void* workspace, int write_final)
+                         int groups, void* workspace, int write_final, int nsplit_total = 0)
 {
+    // nsplit_total: split slots per query row in the workspace (more than this launch fills when a dense window
+    // adds its own)
     const int Bkv = Bq / groups, nblk = tokens / 64, ns = fused_nsplit(tokens);
+    const int nst = nsplit_total > 0 ? nsplit_total : ns;
     float* part_o = reinterpret_cast<float*>(workspace);
-    float* part_ml = part_o + (size_t)Bq * ns * head_dim;
+    float* part_ml = part_o + (size_t)Bq * nst * head_dim;
     const dim3 grid((unsigned)ns, (unsigned)Bkv);
     const char* knz = reinterpret_cast<const char*>(k_nz);
     const char* vnz = reinterpret_cast<const char*>(v_nz);
@@ -312,11 +403,11 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     const float sq = sqrtf((float)head_dim);
     if (groups <= 4)
         hipLaunchKernelGGL(decode_attention_kernel<1>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
-                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, ns, write_final,
+                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst, write_final,
                            sq);
     else
         hipLaunchKernelGGL(decode_attention_kernel<2>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
-                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, ns, write_final,
+                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst, write_final,
                            sq);
     return check_launch();
 }
@@ -370,4 +461,65 @@ extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, co
     if (rc != MSTF_OK || write_final) return rc;
     return mstf_decode_attention_merge_f16(stream, workspace, workspace_bytes, out, lse_out, tokens, head_dim, Bq,
                                            groups);
+}
+
+static int window_blocks(int win_len) { return (win_len + 63) / 64; }
+
+extern "C" size_t mstf_decode_attention_window_workspace_bytes(int tokens, int max_window, int head_dim, int Bq,
+                                                               int groups)
+{
+    if (tokens < 0 || max_window <= 0 || head_dim != kFusedD || Bq <= 0 || groups <= 0 || tokens % 64 != 0 ||
+        Bq % groups != 0)
+        return 0;
+    const int nst = fused_nsplit(tokens) + window_blocks(max_window);
+    return round_up((size_t)Bq * nst * (head_dim + 2) * sizeof(float), 256);
+}
+
+extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                                const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
+                                                const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
+                                                const mstf_half* q, const mstf_half* k_win, const mstf_half* v_win,
+                                                int win_len, int win_stride, mstf_half* out, float* lse_out, int tokens,
+                                                int head_dim, int Bq, int groups, void* workspace,
+                                                size_t workspace_bytes)
+{
+    if (!q || !k_win || !v_win || !out) return MSTF_EINVAL;
+    if (tokens < 0 || win_len <= 0 || win_stride < win_len || Bq <= 0 || groups <= 0 || Bq % groups != 0)
+        return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (!aligned_to(q, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    const int ns = fused_nsplit(tokens), nwb = window_blocks(win_len), nst = ns + nwb;
+    const int Bkv = Bq / groups;
+    int rc;
+    if (tokens > 0) {
+        // the compressed tokens fill split slots 0 .. ns-1 of every row
+        rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, tokens, head_dim, Bq, groups,
+                          workspace, workspace_bytes);
+        if (rc != MSTF_OK) return rc;
+        rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, nullptr,
+                           tokens, head_dim, Bq, groups, workspace, 0, nst);
+        if (rc != MSTF_OK) return rc;
+    }
+    float* part_o = reinterpret_cast<float*>(workspace);
+    float* part_ml = part_o + (size_t)Bq * nst * head_dim;
+    const _Float16* kw = reinterpret_cast<const _Float16*>(k_win);
+    const _Float16* vw = reinterpret_cast<const _Float16*>(v_win);
+    const _Float16* qh = reinterpret_cast<const _Float16*>(q);
+    const float sq = sqrtf((float)head_dim);
+    const dim3 grid((unsigned)nwb, (unsigned)Bkv);
+    if (groups <= 4)
+        hipLaunchKernelGGL(window_attention_kernel<4>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
+                           win_len, win_stride, groups, nst, ns, sq);
+    else
+        hipLaunchKernelGGL(window_attention_kernel<8>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
+                           win_len, win_stride, groups, nst, ns, sq);
+    if ((rc = check_launch()) != MSTF_OK) return rc;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, as_stream(stream), part_o, part_ml,
+                       reinterpret_cast<_Float16*>(out), lse_out, nst, head_dim);
+    return check_launch();
 }

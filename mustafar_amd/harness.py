@@ -1,0 +1,234 @@
+"""Decode-loop harness: a random-init Llama-3 style decoder in plain PyTorch (library GEMMs, RMSNorm, RoPE, SDPA
+prefill) around the sparse KV cache, after the reference's benchmark/mem_spd_test.py:109-187 and
+benchmark/low_memory_generation.py: prompt -> prefill (the first Lc tokens are pruned and compressed per layer) ->
+greedy decode, reporting tokens/s and the share of the step spent in attention over the cache.
+
+The model is only the carrier of the measurement: weights are N(0, 0.02) and nothing is loaded from disk.
+`cache="sparse"` uses SparseKVCache (compressed tokens and window in three launches, pooled storage);
+`cache="dense_masked"` keeps the pruned tokens
+dense and attends with torch ops - the reference's own dense path (models/llama_mustafar_Kt_Mag_Vt_Mag.py:836-1026) -
+and is what the sparse run is compared against.
+
+    python -m mustafar_amd.harness --layers 32 --batch 16 --prompt 4096 --new-tokens 256
+"""
+import argparse
+import json
+import math
+import time
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .cache import CHUNK, SparseKVCache, _repeat_kv
+
+
+class Config:
+    def __init__(self, hidden=4096, layers=32, n_q=32, n_kv=8, head_dim=128, ffn=14336, vocab=128256,
+                 rope_theta=500000.0, rms_eps=1e-5):
+        self.hidden, self.layers, self.n_q, self.n_kv, self.head_dim = hidden, layers, n_q, n_kv, head_dim
+        self.ffn, self.vocab, self.rope_theta, self.rms_eps = ffn, vocab, rope_theta, rms_eps
+
+
+class DenseMaskedCache:
+    """Same state machine as SparseKVCache with the compressed range kept as pruned dense tensors."""
+
+    def __init__(self, groups, head_dim, k_sparsity, v_sparsity, residual_length):
+        self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
+        self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
+        self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
+        self.k = self.v = None
+        self.compressed_length = self.kv_len = 0
+
+    @staticmethod
+    def _prune(x, kth):
+        a = x.abs().float()
+        thr = torch.kthvalue(a, kth, dim=-1, keepdim=True).values
+        return torch.where(a >= thr, x, torch.zeros_like(x))
+
+    def prefill(self, K, V):
+        L = K.shape[2]
+        Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
+        self.k, self.v = K.clone(), V.clone()
+        if Lc > 0:
+            self.k[:, :, :Lc] = self._prune(K[:, :, :Lc], self.kth_k)
+            self.v[:, :, :Lc] = self._prune(V[:, :, :Lc], self.kth_v)
+        self.compressed_length, self.kv_len = Lc, L
+
+    def decode(self, q, k_new, v_new):
+        D, g = self.head_dim, self.groups
+        self.kv_len += 1
+        self.k = torch.cat([self.k, k_new], dim=2)
+        self.v = torch.cat([self.v, v_new], dim=2)
+        s = torch.matmul(q, _repeat_kv(self.k, g).transpose(2, 3))
+        p = torch.softmax((s / math.sqrt(D)).float(), -1).half()
+        out = torch.matmul(p, _repeat_kv(self.v, g))
+        Lc = self.compressed_length
+        if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.kv_len - Lc >= CHUNK:
+            self.k[:, :, Lc:Lc + CHUNK] = self._prune(self.k[:, :, Lc:Lc + CHUNK], self.kth_k)
+            self.v[:, :, Lc:Lc + CHUNK] = self._prune(self.v[:, :, Lc:Lc + CHUNK], self.kth_v)
+            self.compressed_length += CHUNK
+        return out
+
+
+def _rms_norm(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+
+
+def _rope(x, pos, theta):
+    """x: [bs, heads, L, D]; pos: [L] positions."""
+    D = x.shape[-1]
+    inv = 1.0 / (theta ** (torch.arange(0, D, 2, device=x.device, dtype=torch.float32) / D))
+    ang = pos.float()[:, None] * inv[None, :]
+    cos = torch.cat([ang.cos(), ang.cos()], -1).to(x.dtype)
+    sin = torch.cat([ang.sin(), ang.sin()], -1).to(x.dtype)
+    x1, x2 = x[..., : D // 2], x[..., D // 2:]
+    return x * cos + torch.cat([-x2, x1], -1) * sin
+
+
+class Decoder:
+    def __init__(self, cfg, device, seed=0, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=0):
+        self.cfg, self.dev = cfg, device
+        g = torch.Generator(device=device)
+        g.manual_seed(seed)
+
+        def w(*shape):
+            return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) * 0.02).half()
+
+        c = cfg
+        self.embed = w(c.vocab, c.hidden)
+        self.layers = []
+        for _ in range(c.layers):
+            self.layers.append({
+                "qkv": w((c.n_q + 2 * c.n_kv) * c.head_dim, c.hidden), "o": w(c.hidden, c.n_q * c.head_dim),
+                "gate_up": w(2 * c.ffn, c.hidden), "down": w(c.hidden, c.ffn),
+                "ln1": torch.ones(c.hidden, device=device, dtype=torch.float16),
+                "ln2": torch.ones(c.hidden, device=device, dtype=torch.float16)})
+        self.norm = torch.ones(c.hidden, device=device, dtype=torch.float16)
+        self.lm_head = w(c.vocab, c.hidden)
+        groups = c.n_q // c.n_kv
+        if cache == "sparse":
+            self.caches = [SparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length, fused=True,
+                                         max_tokens=max_tokens, window_kernel=True) for _ in range(c.layers)]
+        else:
+            self.caches = [DenseMaskedCache(groups, c.head_dim, sparsity, sparsity, residual_length)
+                           for _ in range(c.layers)]
+        self.attn_events = []   # (start, end) pairs around the cache's decode of every layer of timed steps
+
+    def _mlp(self, lw, x):
+        gu = F.linear(x, lw["gate_up"])
+        gate, up = gu.chunk(2, -1)
+        return F.linear(F.silu(gate) * up, lw["down"])
+
+    def _qkv(self, lw, x, pos):
+        c = self.cfg
+        bs, L, _ = x.shape
+        qkv = F.linear(x, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim).transpose(1, 2)
+        q, k, v = qkv[:, : c.n_q], qkv[:, c.n_q: c.n_q + c.n_kv], qkv[:, c.n_q + c.n_kv:]
+        return _rope(q, pos, c.rope_theta), _rope(k, pos, c.rope_theta).contiguous(), v.contiguous()
+
+    @torch.no_grad()
+    def prefill(self, ids, seq_chunk=4):
+        """ids: [bs, L].  Returns the logits of the last position; fills the caches."""
+        c = self.cfg
+        bs, L = ids.shape
+        pos = torch.arange(L, device=self.dev)
+        x = self.embed[ids]
+        for lw, cache in zip(self.layers, self.caches):
+            h = _rms_norm(x, lw["ln1"], c.rms_eps)
+            q, k, v = self._qkv(lw, h, pos)
+            outs = []
+            for b0 in range(0, bs, seq_chunk):   # bounded working set of the prefill attention
+                outs.append(F.scaled_dot_product_attention(q[b0:b0 + seq_chunk], k[b0:b0 + seq_chunk], v[b0:b0 + seq_chunk],
+                                                           is_causal=True, enable_gqa=True))
+            a = torch.cat(outs, 0).transpose(1, 2).reshape(bs, L, c.n_q * c.head_dim)
+            cache.prefill(k, v)
+            x = x + F.linear(a, lw["o"])
+            h = _rms_norm(x, lw["ln2"], c.rms_eps)
+            for b0 in range(0, bs, seq_chunk):
+                x[b0:b0 + seq_chunk] += self._mlp(lw, h[b0:b0 + seq_chunk])
+        return F.linear(_rms_norm(x[:, -1:], self.norm, c.rms_eps), self.lm_head)
+
+    @torch.no_grad()
+    def step(self, ids, position, timed=False):
+        """ids: [bs, 1] -> logits [bs, 1, vocab]."""
+        c = self.cfg
+        pos = torch.tensor([position], device=self.dev)
+        x = self.embed[ids]
+        for lw, cache in zip(self.layers, self.caches):
+            h = _rms_norm(x, lw["ln1"], c.rms_eps)
+            q, k, v = self._qkv(lw, h, pos)
+            if timed:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+            a = cache.decode(q.contiguous(), k, v)
+            if timed:
+                e1.record()
+                self.attn_events.append((e0, e1))
+            x = x + F.linear(a.transpose(1, 2).reshape(x.shape[0], 1, c.n_q * c.head_dim), lw["o"])
+            x = x + self._mlp(lw, _rms_norm(x, lw["ln2"], c.rms_eps))
+        return F.linear(_rms_norm(x, self.norm, c.rms_eps), self.lm_head)
+
+
+def generate(dec, prompt_ids, new_tokens, forced=None):
+    """Greedy decode (or teacher-forced with `forced` [bs, new_tokens]).  Returns (tokens, logits per step)."""
+    logits = dec.prefill(prompt_ids)
+    L = prompt_ids.shape[1]
+    toks, all_logits = [], []
+    for t in range(new_tokens):
+        nxt = logits[:, -1].argmax(-1, keepdim=True) if forced is None else forced[:, t:t + 1]
+        toks.append(nxt)
+        logits = dec.step(nxt, L + t)
+        all_logits.append(logits[:, 0].float())
+    return torch.cat(toks, 1), all_logits
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--prompt", type=int, default=4096)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--sparsity", type=float, default=0.7)
+    ap.add_argument("--residual", type=int, default=256)
+    ap.add_argument("--cache", default="sparse", choices=["sparse", "dense_masked"])
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    cfg = Config(layers=args.layers)
+    max_tokens = ((args.prompt + args.new_tokens + CHUNK - 1) // CHUNK) * CHUNK
+    dec = Decoder(cfg, dev, cache=args.cache, sparsity=args.sparsity, residual_length=args.residual, max_tokens=max_tokens)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    ids = torch.randint(0, cfg.vocab, (args.batch, args.prompt), generator=g, device=dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = dec.prefill(ids)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    nxt = logits[:, -1].argmax(-1, keepdim=True)
+    warm = min(8, args.new_tokens // 4)
+    for t in range(warm):
+        nxt = dec.step(nxt, args.prompt + t)[:, -1].argmax(-1, keepdim=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(warm, args.new_tokens):
+        nxt = dec.step(nxt, args.prompt + t, timed=True)[:, -1].argmax(-1, keepdim=True)
+    torch.cuda.synchronize()
+    t_dec = time.perf_counter() - t0
+    steps = args.new_tokens - warm
+    attn_ms = sum(a.elapsed_time(b) for a, b in dec.attn_events)
+    print(json.dumps({
+        "workload": "random-init Llama-3-8B shape, %d layers, batch %d, prompt %d, %d greedy tokens, residual %d, "
+                    "%d-token chunks, %.0f%% K/V sparsity, cache=%s (eager PyTorch around the cache operators)"
+                    % (args.layers, args.batch, args.prompt, args.new_tokens, args.residual, CHUNK,
+                       100 * args.sparsity, args.cache),
+        "prefill_s": round(t_prefill, 3), "decode_ms_per_step": round(1e3 * t_dec / steps, 3),
+        "tokens_per_s": round(args.batch * steps / t_dec, 1),
+        "attention_over_cache_ms_per_step": round(attn_ms / steps, 3),
+        "attention_share": round(attn_ms / (1e3 * t_dec), 4),
+        "compressed_tokens_at_end": dec.caches[0].compressed_length}))
+
+
+if __name__ == "__main__":
+    main()

@@ -16,8 +16,9 @@ def rel_rowmax(a, b):
     return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
-@pytest.mark.parametrize("fused,pooled", [(False, False), (True, False), (True, True)])
-def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled):
+@pytest.mark.parametrize("fused,pooled,window_kernel", [(False, False, False), (True, False, False), (True, True, False),
+                                                        (True, True, True)])
+def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled, window_kernel):
     from mustafar_amd import ops
     from mustafar_amd.cache import SparseKVCache
     dev = torch.device("cuda:0")
@@ -29,7 +30,8 @@ def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled):
     Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
-    cache = SparseKVCache(g, D, 0.7, 0.7, res, fused=fused, max_tokens=1024 if pooled else 0)
+    cache = SparseKVCache(g, D, 0.7, 0.7, res, fused=fused, max_tokens=1024 if pooled else 0,
+                          window_kernel=window_kernel)
     cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
     assert cache.compressed_length == ((L0 - res) // 256) * 256 == 256
     checked = 0
@@ -88,14 +90,15 @@ def test_pool_overflow_is_flagged_and_leaves_other_heads_alone():
         assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
 
 
-def test_short_prompt_stays_dense_until_first_chunk():
+@pytest.mark.parametrize("window_kernel", [False, True])
+def test_short_prompt_stays_dense_until_first_chunk(window_kernel):
     from mustafar_amd.cache import SparseKVCache
     dev = torch.device("cuda:0")
     bs, n_kv, g, D = 1, 2, 2, 128
     K, V = orc.make_kv(5, bs * n_kv, 300, D)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, 300, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, 300, D)
-    cache = SparseKVCache(g, D, 0.5, 0.5, 32)
+    cache = SparseKVCache(g, D, 0.5, 0.5, 32, window_kernel=window_kernel)
     cache.prefill(Kt[:, :, :200], Vt[:, :, :200])       # (200 - 32) // 256 == 0 -> nothing compressed
     assert cache.compressed_length == 0 and cache.k is None
     q = torch.randn((bs, n_kv * g, 1, D), device=dev, dtype=torch.float16)

@@ -1,0 +1,34 @@
+"""The decode-loop harness on a small model: the sparse cache (fused launch, pooled storage) against the dense masked
+cache with the same weights and the same forced tokens - the logits of every step agree, across a chunk append."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_sparse_cache_tracks_dense_masked_cache_in_the_decode_loop():
+    from mustafar_amd.harness import Config, Decoder, generate
+    dev = torch.device("cuda:0")
+    cfg = Config(hidden=512, layers=2, n_q=4, n_kv=2, head_dim=128, ffn=1024, vocab=1000)
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    bs, prompt, new = 2, 600, 180                      # Lc = 256 after prefill, one append at kv_len 768
+    ids = torch.randint(0, cfg.vocab, (bs, prompt), generator=g, device=dev)
+    ref = Decoder(cfg, dev, seed=11, cache="dense_masked")
+    toks, ref_logits = generate(ref, ids, new)
+    sp = Decoder(cfg, dev, seed=11, cache="sparse", max_tokens=1024)
+    toks2, sp_logits = generate(sp, ids, new, forced=toks)
+    assert sp.caches[0].compressed_length == ref.caches[0].compressed_length == 512
+    assert int(sp.caches[0].k_pool.overflow) == 0
+    worst = 0.0
+    for a, b in zip(sp_logits, ref_logits):
+        worst = max(worst, float((a - b).abs().max() / b.abs().max()))
+    assert worst < 1e-2, worst
+    # the greedy choice agrees wherever the reference's margin between its two best logits is not a rounding matter
+    agree = total = 0
+    for a, b in zip(sp_logits, ref_logits):
+        top2 = b.topk(2, -1).values
+        clear = (top2[:, 0] - top2[:, 1]) > 2e-2 * b.abs().max()
+        agree += int((a.argmax(-1) == b.argmax(-1))[clear].sum())
+        total += int(clear.sum())
+    assert total > 0 and agree == total
