@@ -76,6 +76,41 @@ def test_partial_then_merge_equals_fused():
     assert rel_rowmax(o.cpu().numpy(), host) < 1e-3
 
 
+@pytest.mark.parametrize("groups,Bkv,Lc,Lw", [(4, 2, 512, 300), (8, 1, 256, 64), (1, 3, 0, 257), (4, 2, 0, 1), (2, 2, 1024, 511)])
+def test_decode_attention_with_dense_window(groups, Bkv, Lc, Lw):
+    """Compressed tokens and dense window under one softmax against the oracle's dense masked attention over
+    [pruned compressed part | window]; Lc = 0 is the window alone."""
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    D = 128
+    Bq = Bkv * groups
+    kth = orc.kth_from_sparsity(0.7, D)
+    K, V = orc.make_kv(300 + Lc + Lw + groups, Bkv, Lc + Lw, D)
+    q = np.random.default_rng(Lw).standard_normal((Bq, D)).astype(np.float16)
+    Kf, Vf = K.copy(), V.copy()
+    ck = cv = None
+    if Lc > 0:
+        Kf[:, :Lc] = orc.prune_rows(np.ascontiguousarray(K[:, :Lc]), kth)
+        Vf[:, :Lc] = orc.prune_rows(np.ascontiguousarray(V[:, :Lc]), kth)
+        ck = ops.compress(torch.from_numpy(np.ascontiguousarray(K[:, :Lc])).to(dev), False, kth=kth)
+        cv = ops.compress(torch.from_numpy(np.ascontiguousarray(V[:, :Lc])).to(dev), True, kth=kth)
+    sc_ref, _, out_ref = orc.dense_masked_attention(q, Kf, Vf, groups)
+    cap = Lw + 37                                   # a buffer longer than the window, rows beyond it poisoned
+    kw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev)
+    vw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev)
+    kw[:, :Lw] = torch.from_numpy(np.ascontiguousarray(K[:, Lc:])).to(dev)
+    vw[:, :Lw] = torch.from_numpy(np.ascontiguousarray(V[:, Lc:])).to(dev)
+    lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
+    o = ops.decode_attention_window(ck, cv, torch.from_numpy(q).to(dev), kw, vw, Lw, groups, lse=lse)
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3
+    w = (sc_ref.astype(np.float32) / np.float32(np.sqrt(128.0))).astype(np.float16).astype(np.float32)
+    m_ref = w.max(-1)
+    got = lse.cpu().numpy()
+    assert np.abs(got[:, 0] - m_ref).max() <= 2e-2 * np.maximum(np.abs(m_ref).max(), 1)
+    l_ref = np.exp(w - m_ref[:, None]).sum(-1)
+    assert np.abs(got[:, 1] * np.exp(got[:, 0] - m_ref) - l_ref).max() <= 5e-3 * l_ref.max()
+
+
 def test_fused_rejects_bad_arguments():
     from mustafar_amd._lib import lib
     L = lib()
@@ -88,5 +123,9 @@ def test_fused_rejects_bad_arguments():
     assert L.mstf_decode_attention_f16(None, *args, 64, 128, 5, 4, a, 1 << 13) == -1
     assert L.mstf_decode_attention_workspace_bytes(4096, 128, 256, 4) == 256 * 8 * 130 * 4
     assert L.mstf_decode_attention_partial_f16(None, *args[:9], 64, 128, 4, 4, None, 0) == -4
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 0, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 9, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 8, 8, a, None, 64, 128, 4, 4, a, 16) == -4
+    assert L.mstf_decode_attention_window_workspace_bytes(4096, 512, 128, 256, 4) == 256 * 16 * 130 * 4
     assert L.mstf_decode_attention_merge_f16(None, a, 1 << 13, None, None, 64, 128, 4, 4) == -1
     assert L.mstf_decode_attention_merge_f16(None, a, 16, a, None, 64, 128, 4, 4) == -4
