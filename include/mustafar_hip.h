@@ -152,14 +152,18 @@ int mstf_decode_attention_merge_f16(void* stream, const void* workspace, size_t 
  * the fused kernel over the `tokens` compressed tokens, a dense kernel over the window, one merge.
  * k_win, v_win: [Bq / groups][win_stride][head_dim] fp16, the first win_len tokens of every KV head valid (the new
  * token included).  tokens may be 0 (nothing compressed yet; the compressed-side pointers are then ignored).
+ * win_len_dev (nullable): the valid length is read from device memory instead - min(*win_len_dev, win_len), at
+ * least 1 - and win_len only sizes the launch and the workspace; a call recorded into a HIP graph then replays
+ * with a window that grows between replays.
  * Workspace: mstf_decode_attention_window_workspace_bytes(tokens, largest win_len, head_dim, Bq, groups). */
 size_t mstf_decode_attention_window_workspace_bytes(int tokens, int max_window, int head_dim, int Bq, int groups);
 int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
                                      const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
                                      const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q,
-                                     const mstf_half* k_win, const mstf_half* v_win, int win_len, int win_stride,
-                                     mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq, int groups,
-                                     void* workspace, size_t workspace_bytes);
+                                     const mstf_half* k_win, const mstf_half* v_win, int win_len,
+                                     const int32_t* win_len_dev, int win_stride, mstf_half* out, float* lse_out,
+                                     int tokens, int head_dim, int Bq, int groups, void* workspace,
+                                     size_t workspace_bytes);
 
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),

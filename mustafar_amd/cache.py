@@ -158,10 +158,12 @@ class SparseKVCache:
         self.compressed_length, self.kv_len = Lc, L
         if self.window_kernel:
             bs, n_kv, _, D = K.shape
-            cap = max(self.residual_length + CHUNK, L - Lc + 1)
+            cap = max(self.residual_length + CHUNK, L - Lc)   # the window never holds more before a chunk leaves
             self._kbuf = torch.empty((bs * n_kv, cap, D), dtype=torch.float16, device=K.device)
             self._vbuf = torch.empty_like(self._kbuf)
             self._wlen = L - Lc
+            self._widx = torch.full((1,), self._wlen, dtype=torch.int64, device=K.device)       # next free row
+            self._wlen_dev = torch.full((1,), self._wlen, dtype=torch.int32, device=K.device)   # valid rows
             self._kbuf[:, :self._wlen] = K[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
             self._vbuf[:, :self._wlen] = V[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
             self._shape = (bs, n_kv, D)
@@ -175,23 +177,43 @@ class SparseKVCache:
         self.k_win = self._kbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
         self.v_win = self._vbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
 
-    def _decode_window_kernel(self, q, k_new, v_new):
+    def decode_device(self, q, k_new, v_new):
+        """The device work of a decode step in window_kernel mode: append the token to the window, attend.  Only
+        device memory changes (the window length is a device counter), so the call can be captured in a HIP graph and
+        replayed; the host-side bookkeeping of the step is advance()."""
         bs, n_q, _, D = q.shape
         n_kv = self._shape[1]
+        self._kbuf.index_copy_(1, self._widx, k_new.reshape(bs * n_kv, 1, D))
+        self._vbuf.index_copy_(1, self._widx, v_new.reshape(bs * n_kv, 1, D))
+        self._widx += 1
+        self._wlen_dev += 1
+        return ops.decode_attention_window(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), self._kbuf, self._vbuf,
+                                           self._kbuf.shape[1], self.groups, win_len_dev=self._wlen_dev).view(bs, n_q, 1, D)
+
+    def advance(self):
+        """Host-side bookkeeping after decode_device (or a replay of it): counts the token and, when the window holds
+        residual_length + 256 tokens, compresses its oldest 256.  Returns True when the compressed part grew (its
+        arrays moved: a captured graph must be captured again)."""
+        bs, n_kv, D = self._shape
         self.kv_len += 1
-        self._kbuf[:, self._wlen] = k_new.reshape(bs * n_kv, D)
-        self._vbuf[:, self._wlen] = v_new.reshape(bs * n_kv, D)
         self._wlen += 1
-        out = ops.decode_attention_window(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), self._kbuf, self._vbuf,
-                                          self._wlen, self.groups).view(bs, n_q, 1, D)
+        grew = False
         if (self.kv_len - self.residual_length - self.compressed_length) % CHUNK == 0 and self._wlen >= CHUNK:
             self._grow(self._kbuf[:, :CHUNK].reshape(bs, n_kv, CHUNK, D), self._vbuf[:, :CHUNK].reshape(bs, n_kv, CHUNK, D))
             rest = self._wlen - CHUNK
             self._kbuf[:, :rest] = self._kbuf[:, CHUNK:self._wlen].clone()
             self._vbuf[:, :rest] = self._vbuf[:, CHUNK:self._wlen].clone()
             self._wlen = rest
+            self._widx.fill_(rest)
+            self._wlen_dev.fill_(rest)
             self.compressed_length += CHUNK
+            grew = True
         self._window_views()
+        return grew
+
+    def _decode_window_kernel(self, q, k_new, v_new):
+        out = self.decode_device(q, k_new, v_new)
+        self.advance()
         return out
 
     def _decode_fused(self, q, s_loc):

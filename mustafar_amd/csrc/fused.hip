@@ -250,13 +250,18 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restri
 {
     const size_t row = blockIdx.x;
     const int c = (int)threadIdx.x;
+    const float* ml = part_ml + row * nsplit * 2;
+    const float* po = part_o + row * nsplit * D + c;
+    // the loads of a loop are independent of each other: unrolled, eight of them are in flight at a time
     float M = -INFINITY;
-    for (int s = 0; s < nsplit; s++) M = fmaxf(M, part_ml[(row * nsplit + s) * 2]);
+#pragma unroll 8
+    for (int s = 0; s < nsplit; s++) M = fmaxf(M, ml[s * 2]);
     float so = 0.f, sl = 0.f;
+#pragma unroll 8
     for (int s = 0; s < nsplit; s++) {
-        const float f = __expf(part_ml[(row * nsplit + s) * 2] - M);
-        so += f * part_o[(row * nsplit + s) * D + c];
-        sl += f * part_ml[(row * nsplit + s) * 2 + 1];
+        const float f = __expf(ml[s * 2] - M);
+        so += f * po[(size_t)s * D];
+        sl += f * ml[s * 2 + 1];
     }
     if (c < D) out[row * D + c] = (_Float16)(so / sl);
     if (lse_out && c == 0) {
@@ -269,85 +274,219 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restri
 // models/llama_mustafar_kernel.py:391-441): one wavefront per (KV head, 64-token block of the window) leaves the
 // same (max, sum, un-normalised output) triple as a split of the compressed tokens, in split slot split0 + block,
 // so that the merge kernel combines compressed tokens and window under one softmax.
-//   key phase   : lane = token reads its own row of k_win, fp32 dot products with the query rows (scalar loads);
-//   value phase : lane = channel pair, the 64 weights are broadcast one token at a time.
-// k_win, v_win: [Bkv][win_stride][D] fp16, the first win_len tokens of every head valid.  G4 = heads computed (>= groups).
-template <int G4>
-__global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __restrict__ k_win,
-                                                              const _Float16* __restrict__ v_win,
-                                                              const _Float16* __restrict__ q, float* __restrict__ part_o,
-                                                              float* __restrict__ part_ml, int win_len, int win_stride,
+// A dense block is handled as 128 full tiles of each format with the accumulation of the compressed path:
+//   key phase   : the K block [64 tokens][128] goes through registers into an LDS slab with a padded row stride, so
+//                 that lane = token reads column `channel` without bank conflicts (immediate offsets, no address
+//                 arithmetic); MFMA against the query rows as in the compressed path;
+//   value phase : the V block arrives by LDS-direct loads; lane = channel reads row `token`.
+// k_win, v_win: [Bkv][win_stride][D] fp16, the first win_len tokens of every head valid; rows beyond are never read.
+template <int NM>
+__global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __restrict__ k_win, const _Float16* v_win,
+                                                              const _Float16* q, float* __restrict__ part_o,
+                                                              float* __restrict__ part_ml, int win_len,
+                                                              const int* __restrict__ win_len_dev, int win_stride,
                                                               int groups, int nsplit, int split0, float sqrt_d)
 {
     constexpr int D = kFusedD;
+    constexpr int kKRow = D * 2 + 4;             // bytes per slab row: 256 of data + 4 of padding
+    constexpr int kKSlab = 64 * kKRow;
+    constexpr int kVBlk = 64 * D * 2;
+    constexpr int kZero = 128;                   // a row half of zeros for the tokens beyond the window
+    constexpr int kQLds = NM * 4 * D * 2;
+    constexpr int kPRow = 64 * 2;
+    constexpr int kPLds = NM * 4 * kPRow;
+    // one array on purpose (LDS-direct loads into several LDS objects make the compiler serialise them)
+    __shared__ __attribute__((aligned(16))) char lds[kKSlab + kVBlk + kZero + kQLds + kPLds];
     const int lane = lane_id();
     const int blk = (int)blockIdx.x, kv = (int)blockIdx.y;
-    const int tok = blk * 64 + lane;
-    const bool valid = tok < win_len;
-    int nt = win_len - blk * 64;
-    nt = nt > 64 ? 64 : nt;
-    const size_t head0 = (size_t)kv * win_stride;
-    // ---- scores of this lane's token for the G4 query heads
-    float s[G4];
+    const int j = lane & 3;
+    // the valid length may live in device memory (a captured graph replays with a growing window); the launch is
+    // then sized for the buffer and a block beyond the window leaves a neutral triple
+    if (win_len_dev) win_len = *win_len_dev < win_len ? *win_len_dev : win_len;
+    if (blk * 64 >= win_len) {
 #pragma unroll
-    for (int h = 0; h < G4; h++) s[h] = 0.f;
-    const u32x4_t* krow = reinterpret_cast<const u32x4_t*>(k_win + (head0 + (valid ? tok : 0)) * D);
-    const uint32_t* qw = reinterpret_cast<const uint32_t*>(q + (size_t)kv * groups * D);  // wave-uniform
-#pragma unroll 4
-    for (int c = 0; c < D / 8; c++) {
-        const u32x4_t kk = krow[c];
-#pragma unroll
-        for (int h = 0; h < G4; h++) {
+        for (int m = 0; m < NM; m++) {
+            const int h = 4 * m + j;
             if (h < groups) {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    s[h] = __builtin_amdgcn_fdot2(as_h2(kk[e]), as_h2(qw[h * (D / 2) + c * 4 + e]), s[h], false);
+                const size_t slot = ((size_t)kv * groups + h) * nsplit + split0 + blk;
+                *reinterpret_cast<f4_t*>(part_o + slot * D + (lane & ~3)) = f4_t{0.f, 0.f, 0.f, 0.f};
+                *reinterpret_cast<f4_t*>(part_o + slot * D + 64 + (lane & ~3)) = f4_t{0.f, 0.f, 0.f, 0.f};
+                if (lane < 4) {
+                    part_ml[slot * 2] = -INFINITY;
+                    part_ml[slot * 2 + 1] = 0.f;
+                }
             }
         }
+        return;
     }
-    // ---- block statistics and fp16 weights, as in the compressed path
-    uint32_t e16[G4];
-    float mrun[G4], lrun[G4];
+    int nt = win_len - blk * 64;
+    nt = nt > 64 ? 64 : nt;
+    char* kslab = lds;
+    char* vblk = lds + kKSlab;
+    char* zero = vblk + kVBlk;
+    char* ql = zero + kZero;
+    char* pl = ql + kQLds;
+    const size_t row0 = (size_t)kv * win_stride + (size_t)blk * 64;
+
+    // ---- staging: V rows and the query rows by LDS-direct loads, K rows through registers into the padded slab
+    {
+        const char* vsrc = reinterpret_cast<const char*>(v_win + row0 * D);
 #pragma unroll
-    for (int h = 0; h < G4; h++) {
-        const _Float16 s16 = (_Float16)s[h];
-        const float w = valid ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
-        float mx = w;
+        for (int i = 0; i < kVBlk / 1024; i++) {
+            const int row = i * 4 + (lane >> 4);  // 16 lanes per 256-byte row
+            if (row < nt) dma16(vsrc + (size_t)(i * 64 + lane) * 16, vblk + i * 1024);
+        }
+        const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
+        const uint32_t qbytes = (uint32_t)groups * D * 2u;
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        const _Float16 eh = valid ? (_Float16)__expf(w - mx) : (_Float16)0.f;
-        float sum = (float)eh;
+        for (int i = 0; i < (kQLds + 1023) / 1024; i++) {
+            const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+            if (o < qbytes) dma16(qsrc + o, ql + i * 1024);
+        }
+        if (lane < kZero / 4) reinterpret_cast<uint32_t*>(zero)[lane] = 0u;
+        // all sixteen row pieces are requested before any is stored (a load under a branch would be waited for on
+        // the spot): rows beyond the window re-read the last valid row and are cleared in registers
+        const u32x4_t* ksrc = reinterpret_cast<const u32x4_t*>(k_win + row0 * D);
+        u32x4_t kreg[16];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-        mrun[h] = mx;
-        lrun[h] = sum;
-        e16[h] = (uint32_t)__builtin_bit_cast(uint16_t, eh);
-    }
-    // ---- value phase: lane owns channels 2*lane, 2*lane+1
-    float acc[G4][2];
+        for (int i = 0; i < 16; i++) {
+            const int e = i * 64 + lane;  // 16-byte piece: row e / 16, piece e % 16
+            const int row = e >> 4, c16 = e & 15;
+            const int src_row = row < nt ? row : nt - 1;
+            kreg[i] = ksrc[src_row * 16 + c16];
+        }
 #pragma unroll
-    for (int h = 0; h < G4; h++) acc[h][0] = acc[h][1] = 0.f;
-    const uint32_t* vbase = reinterpret_cast<const uint32_t*>(v_win + (head0 + (size_t)blk * 64) * D) + lane;
-#pragma unroll 4
-    for (int t = 0; t < nt; t++) {
-        const h2_t vv = as_h2(vbase[(size_t)t * (D / 2)]);
-        const float v0 = (float)vv.x, v1 = (float)vv.y;
-#pragma unroll
-        for (int h = 0; h < G4; h++) {
-            const float pw = (float)as_h((uint16_t)__builtin_amdgcn_readlane(e16[h], t));
-            acc[h][0] += pw * v0;
-            acc[h][1] += pw * v1;
+        for (int i = 0; i < 16; i++) {
+            const int e = i * 64 + lane;
+            const int row = e >> 4, c16 = e & 15;
+            const uint32_t keep = row < nt ? 0xFFFFFFFFu : 0u;
+            uint32_t* d = reinterpret_cast<uint32_t*>(kslab + row * kKRow + c16 * 16);
+            d[0] = kreg[i][0] & keep;
+            d[1] = kreg[i][1] & keep;
+            d[2] = kreg[i][2] & keep;
+            d[3] = kreg[i][3] & keep;
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- key phase: tile c = channel c over the 64 tokens, lane = token
+    f4_t acc_k[NM];
 #pragma unroll
-    for (int h = 0; h < G4; h++) {
+    for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t kcol = lds_addr(kslab) + (uint32_t)lane * kKRow;
+    const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
+    // the gathers of the next eight channels are issued before the current eight are consumed: with one wavefront
+    // per SIMD nothing else would cover the LDS round trip
+    auto key_gather = [&](int c8, _Float16 (&h)[8], u32x4_t (&w)[NM]) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) h[i] = lds_load_h(kcol + (uint32_t)(c8 * 8 + i) * 2u);
+#pragma unroll
+        for (int m = 0; m < NM; m++)
+            w[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(qrow + (uint32_t)c8 * 16u + (uint32_t)m * (D * 8u));
+    };
+    {
+        _Float16 hc[8], hn[8];
+        u32x4_t wc[NM], wn[NM];
+        key_gather(0, hc, wc);
+#pragma unroll
+        for (int c8 = 0; c8 < D / 8; c8++) {
+            if (c8 + 1 < D / 8) key_gather(c8 + 1, hn, wn);
+            __builtin_amdgcn_sched_barrier(0);
+            const uint32_t v0 = pack_h2(hc[0], hc[1]), v1 = pack_h2(hc[2], hc[3]);
+            const uint32_t v2 = pack_h2(hc[4], hc[5]), v3 = pack_h2(hc[6], hc[7]);
+#pragma unroll
+            for (int m = 0; m < NM; m++) {
+                acc_k[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(wc[m][0], wc[m][1]), acc_k[m], 0, 0, 0);
+                acc_k[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(wc[m][2], wc[m][3]), acc_k[m], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; i++) hc[i] = hn[i];
+#pragma unroll
+            for (int m = 0; m < NM; m++) wc[m] = wn[m];
+        }
+    }
+    // ---- block statistics and fp16 weights; lane 4b+j holds tokens 4b..4b+3 of head 4m+j
+    float m_run[NM], l_run[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        float w[4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const _Float16 s16 = (_Float16)acc_k[m][r];
+            w[r] = ((lane & ~3) + r < nt) ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
+            mx = fmaxf(mx, w[r]);
+        }
+        mx = wave_max_same_column(mx);
+        float sum = 0.f;
+        h4_t e16;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float e = w[r] == -INFINITY ? 0.f : __expf(w[r] - mx);
+            e16[r] = (_Float16)e;
+            sum += (float)e16[r];
+        }
+        sum = wave_sum_same_column(sum);
+        m_run[m] = mx;
+        l_run[m] = sum;
+        *reinterpret_cast<h4_t*>(pl + (m * 4 + j) * kPRow + (lane & ~3) * 2) = e16;
+    }
+    // ---- value phase: tile (half, token) = 64 channels of one token, lane = channel of the half
+    f4_t acc_v[NM][2];
+    const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
+    const uint32_t vcol = lds_addr(vblk) + (uint32_t)lane * 2u;
+    const uint32_t zcol = lds_addr(zero) + (uint32_t)lane * 2u;
+    auto value_gather = [&](int g, _Float16 (&h)[8], u32x4_t (&w)[NM]) {  // g = half * 8 + group of eight tokens
+        const int half = g >> 3, t8 = g & 7;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int t = t8 * 8 + i;  // a token beyond the window reads zeros: its weight is 0 but its row is not staged
+            h[i] = lds_load_h(t < nt ? vcol + (uint32_t)(t * D * 2 + half * 128) : zcol);
+        }
+#pragma unroll
+        for (int m = 0; m < NM; m++)
+            w[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(prow + (uint32_t)t8 * 16u + (uint32_t)m * (4u * kPRow));
+    };
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc_v[m][0] = acc_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+    {
+        _Float16 hc[8], hn[8];
+        u32x4_t wc[NM], wn[NM];
+        value_gather(0, hc, wc);
+#pragma unroll
+        for (int g = 0; g < 16; g++) {
+            if (g + 1 < 16) value_gather(g + 1, hn, wn);
+            __builtin_amdgcn_sched_barrier(0);
+            const int half = g >> 3;
+            const uint32_t v0 = pack_h2(hc[0], hc[1]), v1 = pack_h2(hc[2], hc[3]);
+            const uint32_t v2 = pack_h2(hc[4], hc[5]), v3 = pack_h2(hc[6], hc[7]);
+#pragma unroll
+            for (int m = 0; m < NM; m++) {
+                acc_v[m][half] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(wc[m][0], wc[m][1]),
+                                                                    acc_v[m][half], 0, 0, 0);
+                acc_v[m][half] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(wc[m][2], wc[m][3]),
+                                                                    acc_v[m][half], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; i++) hc[i] = hn[i];
+#pragma unroll
+            for (int m = 0; m < NM; m++) wc[m] = wn[m];
+        }
+    }
+    // lane 4b+j holds channels 4b..4b+3 of both halves for head 4m+j
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const int h = 4 * m + j;
         if (h < groups) {
             const size_t slot = ((size_t)kv * groups + h) * nsplit + split0 + blk;
-            part_o[slot * D + 2 * lane] = acc[h][0];
-            part_o[slot * D + 2 * lane + 1] = acc[h][1];
-            if (lane == 0) {
-                part_ml[slot * 2] = mrun[h];
-                part_ml[slot * 2 + 1] = lrun[h];
+            *reinterpret_cast<f4_t*>(part_o + slot * D + (lane & ~3)) = acc_v[m][0];
+            *reinterpret_cast<f4_t*>(part_o + slot * D + 64 + (lane & ~3)) = acc_v[m][1];
+            if (lane < 4) {
+                part_ml[slot * 2] = m_run[m];
+                part_ml[slot * 2 + 1] = l_run[m];
             }
         }
     }
@@ -479,7 +618,8 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
                                                 const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
                                                 const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
                                                 const mstf_half* q, const mstf_half* k_win, const mstf_half* v_win,
-                                                int win_len, int win_stride, mstf_half* out, float* lse_out, int tokens,
+                                                int win_len, const int32_t* win_len_dev, int win_stride, mstf_half* out,
+                                                float* lse_out, int tokens,
                                                 int head_dim, int Bq, int groups, void* workspace,
                                                 size_t workspace_bytes)
 {
@@ -488,7 +628,7 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
         return MSTF_EINVAL;
     if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
     if (!aligned_to(q, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
-        (lse_out && !aligned_to(lse_out, 4)))
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)))
         return MSTF_EALIGN;
     const size_t need = mstf_decode_attention_window_workspace_bytes(tokens, win_len, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
@@ -513,11 +653,11 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
     const float sq = sqrtf((float)head_dim);
     const dim3 grid((unsigned)nwb, (unsigned)Bkv);
     if (groups <= 4)
-        hipLaunchKernelGGL(window_attention_kernel<4>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
-                           win_len, win_stride, groups, nst, ns, sq);
+        hipLaunchKernelGGL(window_attention_kernel<1>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
+                           win_len, win_len_dev, win_stride, groups, nst, ns, sq);
     else
-        hipLaunchKernelGGL(window_attention_kernel<8>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
-                           win_len, win_stride, groups, nst, ns, sq);
+        hipLaunchKernelGGL(window_attention_kernel<2>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
+                           win_len, win_len_dev, win_stride, groups, nst, ns, sq);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, as_stream(stream), part_o, part_ml,
                        reinterpret_cast<_Float16*>(out), lse_out, nst, head_dim);

@@ -153,8 +153,11 @@ class Decoder:
     @torch.no_grad()
     def step(self, ids, position, timed=False):
         """ids: [bs, 1] -> logits [bs, 1, vocab]."""
-        c = self.cfg
         pos = torch.tensor([position], device=self.dev)
+        return self._layers(ids, pos, timed, lambda cache, q, k, v: cache.decode(q, k, v))
+
+    def _layers(self, ids, pos, timed, attend):
+        c = self.cfg
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
@@ -162,13 +165,59 @@ class Decoder:
             if timed:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            a = cache.decode(q.contiguous(), k, v)
+            a = attend(cache, q.contiguous(), k, v)
             if timed:
                 e1.record()
                 self.attn_events.append((e0, e1))
             x = x + F.linear(a.transpose(1, 2).reshape(x.shape[0], 1, c.n_q * c.head_dim), lw["o"])
             x = x + self._mlp(lw, _rms_norm(x, lw["ln2"], c.rms_eps))
         return F.linear(_rms_norm(x, self.norm, c.rms_eps), self.lm_head)
+
+
+class GraphedGreedyLoop:
+    """Greedy decoding with the whole step - embedding to argmax - replayed from a HIP graph.
+
+    Everything that changes from step to step lives in device memory and is updated inside the graph: the token
+    ids, the position (RoPE), the window length and write index of every layer's cache.  The host only counts
+    (SparseKVCache.advance) and, every 256 tokens, lets the caches compress a chunk; the compressed arrays move
+    then, so the graph is captured again."""
+
+    def __init__(self, dec, first_ids, position):
+        self.dec = dec
+        self.ids = first_ids.clone()
+        self.pos = torch.tensor([position], device=dec.dev)
+        self.graph = None
+        self.captures = 0
+
+    @torch.no_grad()
+    def _device_step(self):
+        logits = self.dec._layers(self.ids, self.pos, False, lambda cache, q, k, v: cache.decode_device(q, k, v))
+        self.ids.copy_(logits[:, -1].argmax(-1, keepdim=True))
+        self.pos += 1
+
+    def _advance(self):
+        grew = False
+        for cache in self.dec.caches:
+            grew |= cache.advance()
+        if grew:
+            self.graph = None
+
+    def step(self):
+        """One token for every sequence; returns nothing (self.ids holds the new tokens on the device)."""
+        if self.graph is None:
+            # one eager step warms allocations up, then the next step is captured and replayed from then on
+            self._device_step()
+            self._advance()
+            if self.graph is None:
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self._device_step()
+                self.graph = g
+                self.captures += 1
+            return
+        self.graph.replay()
+        self._advance()
 
 
 def generate(dec, prompt_ids, new_tokens, forced=None):
@@ -193,6 +242,7 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.7)
     ap.add_argument("--residual", type=int, default=256)
     ap.add_argument("--cache", default="sparse", choices=["sparse", "dense_masked"])
+    ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph (sparse cache only)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = Config(layers=args.layers)
@@ -208,25 +258,41 @@ def main():
     t_prefill = time.perf_counter() - t0
     nxt = logits[:, -1].argmax(-1, keepdim=True)
     warm = min(8, args.new_tokens // 4)
-    for t in range(warm):
-        nxt = dec.step(nxt, args.prompt + t)[:, -1].argmax(-1, keepdim=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for t in range(warm, args.new_tokens):
-        nxt = dec.step(nxt, args.prompt + t, timed=True)[:, -1].argmax(-1, keepdim=True)
-    torch.cuda.synchronize()
-    t_dec = time.perf_counter() - t0
+    loop = None
+    if args.graph:
+        assert args.cache == "sparse"
+        loop = GraphedGreedyLoop(dec, nxt, args.prompt)
+        for t in range(warm):
+            loop.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for t in range(warm, args.new_tokens):
+            loop.step()
+        torch.cuda.synchronize()
+        t_dec = time.perf_counter() - t0
+    else:
+        for t in range(warm):
+            nxt = dec.step(nxt, args.prompt + t)[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for t in range(warm, args.new_tokens):
+            nxt = dec.step(nxt, args.prompt + t, timed=True)[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        t_dec = time.perf_counter() - t0
     steps = args.new_tokens - warm
     attn_ms = sum(a.elapsed_time(b) for a, b in dec.attn_events)
     print(json.dumps({
         "workload": "random-init Llama-3-8B shape, %d layers, batch %d, prompt %d, %d greedy tokens, residual %d, "
-                    "%d-token chunks, %.0f%% K/V sparsity, cache=%s (eager PyTorch around the cache operators)"
+                    "%d-token chunks, %.0f%% K/V sparsity, cache=%s (%s)"
                     % (args.layers, args.batch, args.prompt, args.new_tokens, args.residual, CHUNK,
-                       100 * args.sparsity, args.cache),
+                       100 * args.sparsity, args.cache,
+                       "decode step replayed from a HIP graph" if loop is not None
+                       else "eager PyTorch around the cache operators"),
         "prefill_s": round(t_prefill, 3), "decode_ms_per_step": round(1e3 * t_dec / steps, 3),
         "tokens_per_s": round(args.batch * steps / t_dec, 1),
-        "attention_over_cache_ms_per_step": round(attn_ms / steps, 3),
-        "attention_share": round(attn_ms / (1e3 * t_dec), 4),
+        "attention_over_cache_ms_per_step": round(attn_ms / steps, 3) if loop is None else None,
+        "attention_share": round(attn_ms / (1e3 * t_dec), 4) if loop is None else None,
+        "graph_captures": loop.captures if loop is not None else 0,
         "compressed_tokens_at_end": dec.caches[0].compressed_length}))
 
 

@@ -144,11 +144,12 @@ def decode_attention(ck, cv, q, groups, out=None, lse=None):
     return o
 
 
-def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, lse=None):
+def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, lse=None, win_len_dev=None):
     """Attention of one decode step over [compressed tokens | dense window] under one softmax, three launches.
 
     ck, cv: CompressedKV or None (nothing compressed yet); q: [Bq, D]; k_win, v_win: [Bkv, win_stride, D] fp16 with
-    the first win_len tokens valid."""
+    the first win_len tokens valid.  win_len_dev (int32 tensor of one element): the valid length is read on the
+    device and win_len is only its upper bound, so that the call can be captured in a HIP graph."""
     assert q.dtype == torch.float16 and q.is_contiguous()
     assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
     D = k_win.shape[-1]
@@ -159,6 +160,7 @@ def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, 
     ws = workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(tokens, int(win_len), D, Bq, groups))
     cp = [t.data_ptr() for t in (ck.bmp, ck.nz, ck.idx, ck.nz_off, cv.bmp, cv.nz, cv.idx, cv.nz_off)] if tokens else [None] * 8
     check(L.mstf_decode_attention_window_f16(_stream(), *cp, q.data_ptr(), k_win.data_ptr(), v_win.data_ptr(), int(win_len),
+                                             win_len_dev.data_ptr() if win_len_dev is not None else None,
                                              k_win.shape[1], o.data_ptr(), lse.data_ptr() if lse is not None else None,
                                              tokens, D, Bq, groups, ws.data_ptr(), ws.numel()),
           "mstf_decode_attention_window_f16")

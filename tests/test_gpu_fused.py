@@ -103,6 +103,10 @@ def test_decode_attention_with_dense_window(groups, Bkv, Lc, Lw):
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
     o = ops.decode_attention_window(ck, cv, torch.from_numpy(q).to(dev), kw, vw, Lw, groups, lse=lse)
     assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3
+    # the same with the length read on the device and the launch sized for the whole buffer
+    wl = torch.tensor([Lw], dtype=torch.int32, device=dev)
+    o_dev = ops.decode_attention_window(ck, cv, torch.from_numpy(q).to(dev), kw, vw, cap, groups, win_len_dev=wl)
+    assert torch.equal(o_dev, o)
     w = (sc_ref.astype(np.float32) / np.float32(np.sqrt(128.0))).astype(np.float16).astype(np.float32)
     m_ref = w.max(-1)
     got = lse.cpu().numpy()
@@ -123,9 +127,9 @@ def test_fused_rejects_bad_arguments():
     assert L.mstf_decode_attention_f16(None, *args, 64, 128, 5, 4, a, 1 << 13) == -1
     assert L.mstf_decode_attention_workspace_bytes(4096, 128, 256, 4) == 256 * 8 * 130 * 4
     assert L.mstf_decode_attention_partial_f16(None, *args[:9], 64, 128, 4, 4, None, 0) == -4
-    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 0, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
-    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 9, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
-    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 8, 8, a, None, 64, 128, 4, 4, a, 16) == -4
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 0, None, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 9, None, 8, a, None, 64, 128, 4, 4, a, 1 << 20) == -1
+    assert L.mstf_decode_attention_window_f16(None, *args[:9], a, a, 8, None, 8, a, None, 64, 128, 4, 4, a, 16) == -4
     assert L.mstf_decode_attention_window_workspace_bytes(4096, 512, 128, 256, 4) == 256 * 16 * 130 * 4
     assert L.mstf_decode_attention_merge_f16(None, a, 1 << 13, None, None, 64, 128, 4, 4) == -1
     assert L.mstf_decode_attention_merge_f16(None, a, 16, a, None, 64, 128, 4, 4) == -4
