@@ -252,10 +252,16 @@ def main():
                                                groups, 1, bit, 32 // bit, 0, wsq.data_ptr(), wsq.numel()),
                       "mstf_value_spmv_quant")
 
-            qkey(), qval()
+            from mustafar_amd import mustafar_package_quant as mpq
+
+            def qfused():
+                mpq.decode_attention_quant(kq, vq, q2, groups, bit, out=o2)
+
+            qkey(), qval(), qfused()
             nbytes = lambda t: sum(x.numel() * x.element_size() for x in (t[0], t[1], t[2], t[5], t[6]))
             quant_us["%dbit" % bit] = {"key_spmv": round(event_time_us(torch, qkey, 30), 2),
                                        "value_spmv": round(event_time_us(torch, qval, 30), 2),
+                                       "fused_decode_attention_incl_merge": round(event_time_us(torch, qfused, 30), 2),
                                        "bytes_per_token_per_kv_head": {"key": round(nbytes(kq) / Bkv / L, 2),
                                                                        "value": round(nbytes(vq) / Bkv / L, 2)}}
             del kq, vq

@@ -203,6 +203,15 @@ int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* pac
                           const mstf_half* zeros, const mstf_half* P, mstf_half* C, int M, int K, int Bq, int groups,
                           int n_rows, int bit, int capacity, int dequant_mode, void* workspace,
                           size_t workspace_bytes);
+/* The fused decode step of mstf_decode_attention_f16 over a quantised cache: key side and value side as produced by
+ * mstf_compress_{key,value}_quant (counts / units are not needed).  Workspace as for mstf_decode_attention_f16. */
+int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off,
+                                const mstf_half* k_scales, const mstf_half* k_zeros, const uint64_t* v_bmp,
+                                const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out, int tokens,
+                                int head_dim, int Bq, int groups, int bit, int capacity, int dequant_mode,
+                                void* workspace, size_t workspace_bytes);
+
 
 #ifdef __cplusplus
 }

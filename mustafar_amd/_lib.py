@@ -49,6 +49,7 @@ SIGNATURES = {
     "mstf_value_spmv_quant_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mstf_value_spmv_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _sz]),
+    "mstf_decode_attention_quant": (_i, [_vp] * 14 + [_i, _i, _i, _i, _i, _i, _i, _vp, _sz]),
 }
 
 

@@ -12,29 +12,9 @@
 // The wavefronts of a workgroup (consecutive token blocks of one KV head) then combine their
 // (max, sum, output) triples through LDS; token splits across workgroups are combined by a small
 // merge kernel.  Scores and probabilities never touch HBM.
-#include "spmv_common.hpp"
-#include "spmv_device.hpp"
+#include "fused_common.hpp"
 
 namespace mstf {
-
-constexpr int kFusedD = 128;
-constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
-constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
-constexpr int kFusedWaves = 8;
-
-__device__ __forceinline__ float wave_max_same_column(float v)
-{
-    // lanes 4b+j for b = 0..15 hold column j: combine over b with xor shuffles of 4, 8, 16, 32
-#pragma unroll
-    for (int o = 4; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-__device__ __forceinline__ float wave_sum_same_column(float v)
-{
-#pragma unroll
-    for (int o = 4; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
 
 // grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns token block
 // s*kFusedWaves + w.  NM = accumulator groups of four query heads (groups <= 4*NM).
@@ -157,31 +137,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
                 stage_batches(n, buf, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
             } else {
                 if (n == kKeySubs) {
-                    // ---- softmax statistics of the block; lane 4b+j holds tokens 4b..4b+3 of head 4m+j
-#pragma unroll
-                    for (int m = 0; m < NM; m++) {
-                        float w[4];
-                        float mx = -INFINITY;
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const _Float16 s16 = (_Float16)acc_k[m][r];
-                            w[r] = (float)(_Float16)((float)s16 / sqrt_d);
-                            mx = fmaxf(mx, w[r]);
-                        }
-                        mx = wave_max_same_column(mx);
-                        float sum = 0.f;
-                        h4_t e16;
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const float e = __expf(w[r] - mx);
-                            e16[r] = (_Float16)e;
-                            sum += (float)e16[r];  // the sum matches the fp16 weights that multiply V
-                        }
-                        sum = wave_sum_same_column(sum);
-                        m_run[m] = mx;
-                        l_run[m] = sum;
-                        *reinterpret_cast<h4_t*>(pl + (m * 4 + j) * kPRow + (lane & ~3) * 2) = e16;
-                    }
+                    block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
                 }
                 const int vs = n - kKeySubs;                      // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
                 constexpr int kSubsPerHalf = 64 / kSubTiles;
@@ -199,47 +155,8 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         wait_lgkm0();
     }
 
-    // ---- workgroup combine: park (output[4*NM][D], max, sum) of every wavefront, then one thread per (head, channel)
-    __syncthreads();
-    {
-        float* po = reinterpret_cast<float*>(my);
-#pragma unroll
-        for (int m = 0; m < NM; m++) {
-            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + (lane & ~3)) = acc_v[m][0];
-            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + 64 + (lane & ~3)) = acc_v[m][1];
-            if (lane < 4) {
-                po[NM * 4 * D + (m * 4 + j) * 2] = m_run[m];
-                po[NM * 4 * D + (m * 4 + j) * 2 + 1] = l_run[m];
-            }
-        }
-    }
-    __syncthreads();
-    for (int o = (int)threadIdx.x; o < groups * D; o += kFusedWaves * 64) {
-        const int h = o / D, c = o - h * D;
-        float M = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < kFusedWaves; w++)
-            M = fmaxf(M, reinterpret_cast<const float*>(lds[w])[NM * 4 * D + h * 2]);
-        float so = 0.f, sl = 0.f;
-#pragma unroll
-        for (int w = 0; w < kFusedWaves; w++) {
-            const float* pw = reinterpret_cast<const float*>(lds[w]);
-            const float mw = pw[NM * 4 * D + h * 2];
-            const float f = mw == -INFINITY ? 0.f : __expf(mw - M);
-            so += f * pw[h * D + c];
-            sl += f * pw[NM * 4 * D + h * 2 + 1];
-        }
-        const size_t row = (size_t)kv * groups + h;
-        if (write_final) {
-            out[row * D + c] = (_Float16)(so / sl);
-        } else {
-            part_o[(row * nsplit + split) * D + c] = so;
-            if (c == 0) {
-                part_ml[(row * nsplit + split) * 2] = M;
-                part_ml[(row * nsplit + split) * 2 + 1] = sl;
-            }
-        }
-    }
+    workgroup_combine<NM>(&lds[0][0], kWaveLds, wave, lane, acc_v, m_run, l_run, kv, groups, split, nsplit, write_final,
+                          out, part_o, part_ml);
 }
 
 // grid = Bq, 128 threads: log-sum-exp combine of the token splits.
@@ -407,32 +324,9 @@ __global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __
             for (int m = 0; m < NM; m++) wc[m] = wn[m];
         }
     }
-    // ---- block statistics and fp16 weights; lane 4b+j holds tokens 4b..4b+3 of head 4m+j
+    // ---- block statistics and fp16 weights; tokens beyond the window get weight 0
     float m_run[NM], l_run[NM];
-#pragma unroll
-    for (int m = 0; m < NM; m++) {
-        float w[4];
-        float mx = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const _Float16 s16 = (_Float16)acc_k[m][r];
-            w[r] = ((lane & ~3) + r < nt) ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
-            mx = fmaxf(mx, w[r]);
-        }
-        mx = wave_max_same_column(mx);
-        float sum = 0.f;
-        h4_t e16;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const float e = w[r] == -INFINITY ? 0.f : __expf(w[r] - mx);
-            e16[r] = (_Float16)e;
-            sum += (float)e16[r];
-        }
-        sum = wave_sum_same_column(sum);
-        m_run[m] = mx;
-        l_run[m] = sum;
-        *reinterpret_cast<h4_t*>(pl + (m * 4 + j) * kPRow + (lane & ~3) * 2) = e16;
-    }
+    block_softmax<NM>(acc_k, sqrt_d, nt, pl, lane, m_run, l_run);
     // ---- value phase: tile (half, token) = 64 channels of one token, lane = channel of the half
     f4_t acc_v[NM][2];
     const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
@@ -491,8 +385,6 @@ __global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __
         }
     }
 }
-
-static int fused_nsplit(int tokens) { return (tokens / 64 + kFusedWaves - 1) / kFusedWaves; }
 
 }  // namespace mstf
 

@@ -1,0 +1,121 @@
+// Pieces shared by the fused decode-attention kernels (fused.hip: fp16 format and dense window; fused_quant.hip:
+// quantised format): block softmax statistics, the workgroup combine and the layout of the split partials.
+#pragma once
+#include "spmv_common.hpp"
+#include "spmv_device.hpp"
+
+namespace mstf {
+
+constexpr int kFusedD = 128;
+constexpr int kFusedWaves = 8;    // token blocks (= wavefronts) per workgroup: 512 tokens per split
+constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
+constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
+
+static inline int fused_nsplit(int tokens) { return (tokens / 64 + kFusedWaves - 1) / kFusedWaves; }
+
+__device__ __forceinline__ float wave_max_same_column(float v)
+{
+    // lanes 4b+j for b = 0..15 hold column j: combine over b with xor shuffles of 4, 8, 16, 32
+#pragma unroll
+    for (int o = 4; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum_same_column(float v)
+{
+#pragma unroll
+    for (int o = 4; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Softmax statistics of one 64-token block from its scores; lane 4b+j holds tokens 4b..4b+3 of head 4m+j in acc_k[m].
+// Scores are rounded to fp16 and divided by sqrt(d) in fp16 (as the reference's glue does); the un-normalised
+// weights exp(w - max) go to LDS as fp16 rows of 64 tokens (the B operand of the value phase) and the block's
+// (max, sum of the fp16 weights) stay in m_run / l_run.  Tokens >= nt (nt < 64 only in a partial block) get weight 0.
+template <int NM>
+__device__ __forceinline__ void block_softmax(const f4_t (&acc_k)[NM], float sqrt_d, int nt, char* pl, int lane,
+                                              float (&m_run)[NM], float (&l_run)[NM])
+{
+    constexpr int kPRow = 64 * 2;
+    const int j = lane & 3;
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        float w[4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const _Float16 s16 = (_Float16)acc_k[m][r];
+            w[r] = ((lane & ~3) + r < nt) ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
+            mx = fmaxf(mx, w[r]);
+        }
+        mx = wave_max_same_column(mx);
+        float sum = 0.f;
+        h4_t e16;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float e = w[r] == -INFINITY ? 0.f : __expf(w[r] - mx);
+            e16[r] = (_Float16)e;
+            sum += (float)e16[r];  // the sum matches the fp16 weights that multiply V
+        }
+        sum = wave_sum_same_column(sum);
+        m_run[m] = mx;
+        l_run[m] = sum;
+        *reinterpret_cast<h4_t*>(pl + (m * 4 + j) * kPRow + (lane & ~3) * 2) = e16;
+    }
+}
+
+// Workgroup combine of the kFusedWaves blocks of a split: every wavefront parks (output[4*NM][D], max, sum) in its
+// own LDS area (`lds_base + wave * wave_stride`, at least NM*4*D*4 + 64 bytes), then one thread per (head, channel)
+// folds them and writes either the final fp16 output (write_final, one split only) or the split's partial:
+//   part_o[((kv*groups + h)*nsplit + split)*D + d] (un-normalised), part_ml[..][2] = (max, sum).
+// An inactive wavefront parks (-inf, 0, 0).
+template <int NM>
+__device__ __forceinline__ void workgroup_combine(char* lds_base, int wave_stride, int wave, int lane,
+                                                  const f4_t (&acc_v)[NM][2], const float (&m_run)[NM],
+                                                  const float (&l_run)[NM], int kv, int groups, int split, int nsplit,
+                                                  int write_final, _Float16* out, float* part_o, float* part_ml)
+{
+    constexpr int D = kFusedD;
+    const int j = lane & 3;
+    __syncthreads();
+    {
+        float* po = reinterpret_cast<float*>(lds_base + wave * wave_stride);
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + (lane & ~3)) = acc_v[m][0];
+            *reinterpret_cast<f4_t*>(po + (m * 4 + j) * D + 64 + (lane & ~3)) = acc_v[m][1];
+            if (lane < 4) {
+                po[NM * 4 * D + (m * 4 + j) * 2] = m_run[m];
+                po[NM * 4 * D + (m * 4 + j) * 2 + 1] = l_run[m];
+            }
+        }
+    }
+    __syncthreads();
+    for (int o = (int)threadIdx.x; o < groups * D; o += kFusedWaves * 64) {
+        const int h = o / D, c = o - h * D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; w++)
+            M = fmaxf(M, reinterpret_cast<const float*>(lds_base + w * wave_stride)[NM * 4 * D + h * 2]);
+        float so = 0.f, sl = 0.f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; w++) {
+            const float* pw = reinterpret_cast<const float*>(lds_base + w * wave_stride);
+            const float mw = pw[NM * 4 * D + h * 2];
+            const float f = mw == -INFINITY ? 0.f : __expf(mw - M);
+            so += f * pw[h * D + c];
+            sl += f * pw[NM * 4 * D + h * 2 + 1];
+        }
+        const size_t row = (size_t)kv * groups + h;
+        if (write_final) {
+            out[row * D + c] = (_Float16)(so / sl);
+        } else {
+            part_o[(row * nsplit + split) * D + c] = so;
+            if (c == 0) {
+                part_ml[(row * nsplit + split) * 2] = M;
+                part_ml[(row * nsplit + split) * 2 + 1] = sl;
+            }
+        }
+    }
+}
+
+}  // namespace mstf

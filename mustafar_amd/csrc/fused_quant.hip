@@ -1,0 +1,241 @@
+// Fused sparse decode attention over the quantised format: key SpMV -> scale + softmax -> value SpMV in one
+// launch, with the work decomposition, softmax and combine of the fp16 kernel (fused.hip) and the staged
+// dequantisation of the quantised SpMVs (quant_spmv.hip).
+//
+// One wavefront owns one (KV head, 64-token block): four stages of 32 key tiles, then four stages of 32 value
+// tiles.  A stage's packed words and metadata arrive by LDS-direct loads one stage ahead (double buffers); the
+// stage is dequantised into the wavefront's fp16 tile image and expanded from there.
+#include "fused_common.hpp"
+#include "quant_device.hpp"
+
+namespace mstf {
+
+#pragma clang fp contract(off)
+
+// One side (keys or values) of a quantised cache; `off_dma` is `off` again, kept apart so that `off` stays a
+// pointer that never reaches an LDS-direct load and is read with scalar loads.
+struct QSide {
+    const uint64_t* bmp;
+    const uint32_t* packed;
+    const uint32_t* off;
+    const uint32_t* off_dma;
+    const uint16_t* scales;
+    const uint16_t* zeros;
+};
+
+// grid = (token splits, KV heads), kFusedWaves wavefronts; see decode_attention_kernel.
+template <int NM, int BIT>
+__global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kernel(
+    const uint64_t* __restrict__ k_bmp, const uint32_t* k_packed, const uint32_t* __restrict__ k_off,
+    const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros, const uint64_t* __restrict__ v_bmp,
+    const uint32_t* v_packed, const uint32_t* __restrict__ v_off, const uint32_t* v_off_dma, const uint16_t* v_scales,
+    const uint16_t* v_zeros, const _Float16* q, _Float16* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int Lc, int groups, int nblk, int nsplit, int write_final, float sqrt_d, int mode)
+{
+    using F = QFmt<BIT>;
+    constexpr int D = kFusedD;
+    constexpr int kQLds = NM * 4 * D * 2;
+    constexpr int kPRow = 64 * 2;
+    constexpr int kPLds = NM * 4 * kPRow;
+    constexpr int kStage = q_lds_bytes<BIT>();  // image, zero slot, two word buffers, two metadata buffers
+    constexpr int kNeed = kStage + kQLds + kPLds;
+    constexpr int kPark = NM * 4 * D * 4 + 64;
+    constexpr int kWaveLds = kNeed > kPark ? kNeed : kPark;
+    // one array on purpose (LDS-direct loads into several LDS objects make the compiler serialise them)
+    __shared__ __attribute__((aligned(16))) char lds_all[kFusedWaves * kWaveLds];
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int split = (int)blockIdx.x;
+    const int kv = (int)blockIdx.y;
+    const int tb = split * kFusedWaves + wave;
+    const bool active = tb < nblk;  // wave-uniform
+    const int j = lane & 3;
+    const size_t T = (size_t)Lc * D / 64;
+    char* my = lds_all + wave * kWaveLds;
+    char* wordbuf = my + kImgBytes + 16;
+    char* metabuf = wordbuf + 2 * F::kWordBuf;
+    char* ql = my + kStage;
+    char* pl = ql + kQLds;
+    const uint32_t lbase = lds_addr(my);
+    const uint32_t zaddr = lbase + kImgBytes;
+
+    f4_t acc_v[NM][2];
+    float m_run[NM], l_run[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        acc_v[m][0] = f4_t{0.f, 0.f, 0.f, 0.f};
+        acc_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+        m_run[m] = -INFINITY;
+        l_run[m] = 0.f;
+    }
+
+    if (active) {
+        const size_t tile0 = (size_t)kv * T + (size_t)tb * D;  // tile_off / scales / zeros / bmp are flat over [Bkv, T]
+        const QSide K = {k_bmp + tile0, k_packed, k_off + tile0, k_off_dma + tile0, k_scales + tile0, k_zeros + tile0};
+        const QSide V = {v_bmp + tile0, v_packed, v_off + tile0, v_off_dma + tile0, v_scales + tile0, v_zeros + tile0};
+        if (lane < 4) reinterpret_cast<uint32_t*>(my + kImgBytes)[lane] = 0u;
+        // word offsets at the stage boundaries of both sides by one vector load (lanes 0.. keys, 16.. values); the
+        // block's last stage ends where its last tile's words end
+        uint32_t bnd = 0u;
+        if (lane < kKeySubs) bnd = K.off[lane * kSubTiles];
+        else if (lane >= 16 && lane < 16 + kValSubs) bnd = V.off[(lane - 16) * kSubTiles];
+        auto words_of = [](uint64_t bm) {
+            return ((uint32_t)__builtin_popcountll(bm) + (uint32_t)F::kCap - 1u) >> F::kCapShift;
+        };
+        const uint32_t endK = K.off[D - 1] + words_of(K.bmp[D - 1]);
+        const uint32_t endV = V.off[D - 1] + words_of(V.bmp[D - 1]);
+        auto start_of = [&](int n) -> uint32_t {
+            return __builtin_amdgcn_readlane(bnd, n < kKeySubs ? n : 16 + n - kKeySubs);
+        };
+        auto end_of = [&](int n) -> uint32_t {
+            if (n == kKeySubs - 1) return endK;
+            if (n == kKeySubs + kValSubs - 1) return endV;
+            return start_of(n + 1);
+        };
+        auto issue = [&](int n) {
+            const QSide& S = n < kKeySubs ? K : V;
+            const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
+            const uint32_t s = start_of(n);
+            uint32_t nw = end_of(n) - s;
+            nw = nw > (uint32_t)F::kWordsMax ? (uint32_t)F::kWordsMax : nw;  // never true for a well-formed cache
+            char* wb = wordbuf + (n & 1) * F::kWordBuf;
+#pragma unroll
+            for (int i = 0; i < F::kWordsMax / 64; i++) {
+                const uint32_t o = (uint32_t)(i * 64 + lane);
+                if (o < nw) dma4(S.packed + s + o, wb + i * 256);
+            }
+            // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane)
+            const void* src = lane < 32 ? (const void*)(S.off_dma + t + lane)
+                                        : lane < 48 ? (const void*)(reinterpret_cast<const uint32_t*>(S.scales + t) + (lane - 32))
+                                                    : (const void*)(reinterpret_cast<const uint32_t*>(S.zeros + t) + (lane - 48));
+            dma4(src, metabuf + (n & 1) * kMetaBytes);
+            // pulls the stage's bitmaps into L2 ahead of the scalar loads of the expansion
+            uint2 b = make_uint2(0u, 0u);
+            if (lane < kSubTiles) b = *reinterpret_cast<const uint2*>(S.bmp + t + lane);
+            return b;
+        };
+
+        // the query rows of this KV head: groups x D fp16, contiguous
+        {
+            const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
+            const uint32_t qbytes = (uint32_t)groups * D * 2u;
+#pragma unroll
+            for (int i = 0; i < (kQLds + 1023) / 1024; i++) {
+                const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
+                if (o < qbytes) dma16(qsrc + o, ql + i * 1024);
+            }
+        }
+        uint2 touch = issue(0);
+
+        f4_t acc_k[NM];
+#pragma unroll
+        for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+        const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
+        const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
+
+        auto stage = [&](int n, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
+            const QSide& S = n < kKeySubs ? K : V;
+            const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
+            dequant_stage<BIT>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
+                               lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), lane, mode);
+            const uint64_t* bm = S.bmp + t;
+            u32x16_t cur = load_bitmaps(bm);
+#pragma unroll
+            for (int g = 0; g < kSubTiles / 8; g++) {
+                u32x16_t nxt = cur;
+                if (g + 1 < kSubTiles / 8) nxt = prefetch_bitmaps(bm + 8 * (g + 1));
+                batch_accumulate_img<NM>(cur, lbase + (uint32_t)g * 1024u, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
+                cur = nxt;
+            }
+        };
+
+#pragma unroll
+        for (int n = 0; n < kKeySubs + kValSubs; n++) {
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
+            if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
+            if (n < kKeySubs) {
+                stage(n, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
+            } else {
+                if (n == kKeySubs) block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
+                const int vs = n - kKeySubs;  // value stage: half = vs / 2, tokens (vs % 2) * 32..
+                constexpr int kSubsPerHalf = 64 / kSubTiles;
+                const int half = vs / kSubsPerHalf;
+                f4_t tmp[NM];
+#pragma unroll
+                for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
+                stage(n, prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u, 4u * kPRow, tmp);
+#pragma unroll
+                for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
+            }
+            wait_lgkm0();  // every read of the image and of the staged buffers is done before they are rewritten
+        }
+    }
+    workgroup_combine<NM>(lds_all, kWaveLds, wave, lane, acc_v, m_run, l_run, kv, groups, split, nsplit, write_final, out,
+                          part_o, part_ml);
+}
+
+template <int NM, int BIT>
+static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                const uint32_t* k_off, const uint16_t* k_scales, const uint16_t* k_zeros,
+                                const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_off,
+                                const uint16_t* v_scales, const uint16_t* v_zeros, const _Float16* q, _Float16* out,
+                                float* part_o, float* part_ml, int tokens, int groups, int ns, int write_final, float sq,
+                                int mode)
+{
+    hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, k_packed, k_off,
+                       k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q, out, part_o, part_ml,
+                       tokens, groups, tokens / 64, ns, write_final, sq, mode);
+}
+
+}  // namespace mstf
+
+using namespace mstf;
+
+extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                           const uint32_t* k_tile_off, const mstf_half* k_scales,
+                                           const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
+                                           const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                           const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out,
+                                           int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
+                                           int dequant_mode, void* workspace, size_t workspace_bytes)
+{
+    if (!k_bmp || !k_packed || !k_tile_off || !k_scales || !k_zeros || !v_bmp || !v_packed || !v_tile_off || !v_scales ||
+        !v_zeros || !q || !out)
+        return MSTF_EINVAL;
+    if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
+    if (dequant_mode != 0 && dequant_mode != 1) return MSTF_EINVAL;
+    if (bit != 2 && bit != 4 && bit != 8) return MSTF_EUNSUPPORTED;
+    if (capacity != 32 / bit) return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (!aligned_to(k_bmp, 8) || !aligned_to(v_bmp, 8) || !aligned_to(k_packed, 4) || !aligned_to(v_packed, 4) ||
+        !aligned_to(k_tile_off, 4) || !aligned_to(v_tile_off, 4) || !aligned_to(k_scales, 4) || !aligned_to(v_scales, 4) ||
+        !aligned_to(k_zeros, 4) || !aligned_to(v_zeros, 4) || !aligned_to(q, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int Bkv = Bq / groups, ns = fused_nsplit(tokens);
+    float* part_o = reinterpret_cast<float*>(workspace);
+    float* part_ml = part_o + (size_t)Bq * ns * head_dim;
+    // with one split and no (max, sum) requested the kernel writes the final output itself
+    const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
+    const dim3 grid((unsigned)ns, (unsigned)Bkv);
+    const _Float16* qh = reinterpret_cast<const _Float16*>(q);
+    _Float16* oh = reinterpret_cast<_Float16*>(out);
+    const float sq = sqrtf((float)head_dim);
+#define MSTF_FQ(NMV, BITV)                                                                                              \
+    launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, \
+                                   v_scales, v_zeros, qh, oh, part_o, part_ml, tokens, groups, ns, write_final, sq,     \
+                                   dequant_mode)
+    if (groups <= 4) {
+        if (bit == 2) MSTF_FQ(1, 2); else if (bit == 4) MSTF_FQ(1, 4); else MSTF_FQ(1, 8);
+    } else {
+        if (bit == 2) MSTF_FQ(2, 2); else if (bit == 4) MSTF_FQ(2, 4); else MSTF_FQ(2, 8);
+    }
+#undef MSTF_FQ
+    int rc = check_launch();
+    if (rc != MSTF_OK || write_final) return rc;
+    return mstf_decode_attention_merge_f16(stream, workspace, workspace_bytes, out, lse_out, tokens, head_dim, Bq, groups);
+}

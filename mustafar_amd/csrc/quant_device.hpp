@@ -1,0 +1,142 @@
+// Device-side building blocks of the quantised consumers (quant_spmv.hip, fused_quant.hip): staging sizes,
+// dequantisation of a staged run of tiles into an fp16 tile image in LDS, expansion of that image.
+#pragma once
+#include "spmv_device.hpp"
+
+namespace mstf {
+
+#pragma clang fp contract(off)
+
+template <int BIT>
+struct QFmt {
+    static constexpr int kCap = 32 / BIT;                       // codes per packed word
+    static constexpr int kCapShift = BIT == 2 ? 4 : (BIT == 4 ? 3 : 2);
+    static constexpr int kSlots = 64 / kCap;                    // words of a full tile = lanes per tile in a pass
+    static constexpr int kTilesPerPass = 64 / kSlots;
+    static constexpr int kPasses = kSubTiles / kTilesPerPass;
+    static constexpr int kWordsMax = kSubTiles * kSlots;        // words of a stage, every tile full
+    static constexpr int kWordBuf = kWordsMax * 4 + 64;         // + room for the lanes past a tile's last word
+};
+constexpr int kImgBytes = kSubTiles * 128;   // fp16 image of a stage: 64 slots per tile
+constexpr int kMetaBytes = 256;              // 32 word offsets, 32 scales, 32 zero-points
+template <int BIT>
+constexpr int q_lds_bytes()
+{
+    return kImgBytes + 16 + 2 * QFmt<BIT>::kWordBuf + 2 * kMetaBytes;
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits) { return (float)as_h((uint16_t)bits); }
+
+// The literal arithmetic of the two dequantisation modes for one code.
+__device__ __forceinline__ _Float16 dequant_exact(uint32_t q, uint32_t scale_bits, uint32_t zero_bits, int mode)
+{
+    if (mode == 1) {
+        const _Float16 d = (_Float16)(int)q - as_h((uint16_t)zero_bits);  // fp16 arithmetic, rounded after each step
+        return d * as_h((uint16_t)scale_bits);
+    }
+    return (_Float16)(((float)q - half_bits_to_float(zero_bits)) * half_bits_to_float(scale_bits));
+}
+
+// fp16x2 ( (q_lo - zero) * scale, (q_hi - zero) * scale ) from two codes held in bytes 0 and 2 of `codes`.
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, h2_t neg_bias, h2_t scale2)
+{
+    const h2_t x = as_h2(codes | 0x64006400u);  // (1024 + q_lo, 1024 + q_hi)
+    return as_u32((x + neg_bias) * scale2);
+}
+
+// One stage: every lane owns one packed word (tile = lane / kSlots of the pass, word = lane % kSlots) and
+// writes that word's values to the tile image.  Lanes past a tile's last word decode whatever follows in
+// the staged buffer into image slots no rank ever points to.
+//   meta  : LDS address of the staged metadata; words: LDS address of the staged words, word 0 = `start_word`
+template <int BIT>
+__device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uint32_t img, uint32_t start_word, int lane,
+                                              int mode)
+{
+    using F = QFmt<BIT>;
+#pragma unroll
+    for (int p = 0; p < F::kPasses; p++) {
+        const uint32_t tl = (uint32_t)(p * F::kTilesPerPass + lane / F::kSlots);
+        const uint32_t slot = (uint32_t)(lane % F::kSlots);
+        const uint32_t off = lds_load_u32(meta + tl * 4u);
+        const uint32_t sc = lds_load_u16(meta + 128u + tl * 2u);
+        const uint32_t zp = lds_load_u16(meta + 192u + tl * 2u);
+        const uint32_t w = lds_load_u32(words + (off - start_word + slot) * 4u);
+        const uint32_t dst = img + tl * 128u + slot * (uint32_t)(F::kCap * 2);
+        if ((zp & 0x7fffu) <= 0x6400u) {
+            const _Float16 nb = (_Float16)(-1024.0f) - as_h((uint16_t)zp);  // exact: |zero| <= 1024
+            const _Float16 sh = as_h((uint16_t)sc);
+            const h2_t neg_bias = {nb, nb};
+            const h2_t scale2 = {sh, sh};
+            if (BIT == 2) {
+                // E[k % 4] holds code k in byte k / 4
+                const uint32_t e0 = w & 0x03030303u, e1 = (w >> 2) & 0x03030303u;
+                const uint32_t e2 = (w >> 4) & 0x03030303u, e3 = (w >> 6) & 0x03030303u;
+                u32x4_t lo, hi;
+                lo[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), neg_bias, scale2);  // codes 0, 1
+                lo[1] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c040c00u), neg_bias, scale2);  // codes 2, 3
+                lo[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), neg_bias, scale2);
+                lo[3] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c050c01u), neg_bias, scale2);
+                hi[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), neg_bias, scale2);
+                hi[1] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c060c02u), neg_bias, scale2);
+                hi[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), neg_bias, scale2);
+                hi[3] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c070c03u), neg_bias, scale2);
+                *(MSTF_LDS u32x4_t*)(uintptr_t)dst = lo;
+                *(MSTF_LDS u32x4_t*)(uintptr_t)(dst + 16u) = hi;
+            } else if (BIT == 4) {
+                // e0 holds codes 0, 2, 4, 6 in its bytes, e1 codes 1, 3, 5, 7
+                const uint32_t e0 = w & 0x0f0f0f0fu, e1 = (w >> 4) & 0x0f0f0f0fu;
+                u32x4_t v;
+                v[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), neg_bias, scale2);
+                v[1] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), neg_bias, scale2);
+                v[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), neg_bias, scale2);
+                v[3] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), neg_bias, scale2);
+                *(MSTF_LDS u32x4_t*)(uintptr_t)dst = v;
+            } else {
+                u32x2_t v;
+                v[0] = dequant_pair(__builtin_amdgcn_perm(w, w, 0x0c010c00u), neg_bias, scale2);
+                v[1] = dequant_pair(__builtin_amdgcn_perm(w, w, 0x0c030c02u), neg_bias, scale2);
+                *(MSTF_LDS u32x2_t*)(uintptr_t)dst = v;
+            }
+        } else {
+#pragma unroll 1
+            for (int k = 0; k < F::kCap; k++) {
+                const uint32_t q = (w >> (k * BIT)) & ((1u << BIT) - 1u);
+                *(MSTF_LDS _Float16*)(uintptr_t)(dst + 2u * (uint32_t)k) = dequant_exact(q, sc, zp, mode);
+            }
+        }
+    }
+}
+
+// Expands 8 tiles of the image and accumulates them (see batch_accumulate for the MFMA layout).
+//   mv   : the 8 bitmaps;  base0: LDS address of the first tile's image slots
+template <int NM>
+__device__ __forceinline__ void batch_accumulate_img(const u32x16_t& mv, uint32_t base0, uint32_t zaddr, uint32_t waddr,
+                                                     uint32_t wgroup, f4_t (&acc)[NM])
+{
+    uint32_t a[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(mv[2 * i], mv[2 * i + 1]), base0 + (uint32_t)i * 128u, zaddr);
+    _Float16 h[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
+    const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
+    const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
+        const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
+    }
+}
+
+__device__ __forceinline__ u32x16_t load_bitmaps(const uint64_t* bm) { return *reinterpret_cast<const u32x16_a4*>(bm); }
+__device__ __forceinline__ u32x16_t prefetch_bitmaps(const uint64_t* bm)
+{
+    __builtin_amdgcn_sched_barrier(0);
+    const u32x16_t v = load_bitmaps(bm);
+    __builtin_amdgcn_sched_barrier(0);
+    return v;
+}
+
+}  // namespace mstf

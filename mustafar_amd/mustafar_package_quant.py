@@ -109,6 +109,32 @@ def mustafar_value_formulation_quant_decode_n1(bmp, NZ_quant, tile_offsets, tile
                   "mustafar_value_formulation_quant_decode_n1")
 
 
+def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, dequant_mode=0, out=None, lse=None):
+    """One launch for key SpMV -> / sqrt(d) -> softmax -> value SpMV over a quantised cache (no counterpart in the
+    reference, which runs the three steps separately).
+
+    key_side, value_side: (bitmaps, tile_offsets, packed, scales, zeros) as convert_*_batched_quant return them
+    (7-tuples with counts and units are accepted); q: [Bq, 128] fp16 -> [Bq, 128] fp16.  lse (optional fp32 [Bq, 2])
+    receives (max, sum) of every row."""
+    def five(side):
+        return side if len(side) == 5 else (side[0], side[1], side[2], side[5], side[6])
+    kb, ko, kp, ks, kz = five(key_side)
+    vb, vo, vp, vs, vz = five(value_side)
+    D = q.shape[-1]
+    Bq = q.numel() // D
+    tokens = kb.shape[1] * 64 // D
+    L = lib()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    ws = ops.workspace(q.device, L.mstf_decode_attention_workspace_bytes(tokens, D, Bq, num_key_value_groups))
+    check(L.mstf_decode_attention_quant(torch.cuda.current_stream().cuda_stream, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(),
+                                        ks.data_ptr(), kz.data_ptr(), vb.data_ptr(), vp.data_ptr(), vo.data_ptr(),
+                                        vs.data_ptr(), vz.data_ptr(), q.contiguous().data_ptr(), o.data_ptr(),
+                                        lse.data_ptr() if lse is not None else None, tokens, D, Bq,
+                                        int(num_key_value_groups), int(bit), 32 // int(bit), int(dequant_mode),
+                                        ws.data_ptr(), ws.numel()), "mstf_decode_attention_quant")
+    return o
+
+
 # aliases the reference exports for its model code (pybind_quant.cpp:96-176)
 mustafar_quant_sparse_forward = mustafar_key_formulation_quant
 mustafar_quant_sparse_forward_meta = mustafar_key_formulation_quant_meta

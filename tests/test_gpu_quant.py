@@ -201,6 +201,42 @@ def test_quant_dequantised_values_bit_exact(bit, dequant_mode):
                             assert np.array_equal(got & ((got != 0x8000) * 0xFFFF), want & ((want != 0x8000) * 0xFFFF))
 
 
+@pytest.mark.parametrize("bit", [2, 4, 8])
+@pytest.mark.parametrize("groups,Bkv,Lc", [(4, 2, 1024), (8, 1, 576), (1, 3, 64)])
+def test_fused_quant_decode_attention(bit, groups, Bkv, Lc):
+    """The one-launch path against dense masked attention on the dequantised cache (1e-2) and against the
+    three-launch quantised path (same dequantised values, so only the softmax rounding differs)."""
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    from mustafar_amd import ops
+    D = 128
+    Bq = Bkv * groups
+    Kp, Vp = pruned(90 + bit + Lc, Bkv, Lc)
+    kq = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
+    vq = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    kr = [t.cpu().numpy() for t in kq]
+    vr = [t.cpu().numpy() for t in vq]
+    Kd = np.stack([orc.decode_quant(kr[0], kr[2], kr[1], kr[5], kr[6], b, Lc, D, 0, bit) for b in range(Bkv)])
+    Vd = np.stack([orc.decode_quant(vr[0], vr[2], vr[1], vr[5], vr[6], b, Lc, D, 1, bit) for b in range(Bkv)])
+    q = np.random.default_rng(bit + Lc).standard_normal((Bq, D)).astype(np.float16)
+    _, _, out_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
+    lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev())
+    o = mpq.decode_attention_quant(kq, vq, to_gpu(q), groups, bit, lse=lse)
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3      # the cache is the same dequantised one: fp16 accuracy
+    o2 = mpq.decode_attention_quant(kq, vq, to_gpu(q), groups, bit)
+    assert torch.equal(o, o2) or rel_rowmax(o2.cpu().numpy(), o.cpu().numpy()) < 1e-3
+    # three-launch path
+    qp = np.zeros((Bq, 8, D), np.float16)
+    qp[:, 0] = q
+    s = mpq.mustafar_key_formulation_quant_meta(kq[0], kq[2], kq[1], kq[3], kq[4], kq[5], kq[6], to_gpu(qp), Lc, D, Bq,
+                                                groups, bit, 32 // bit)[:, 0].contiguous()
+    p = ops.scale_softmax(s, D)
+    o3 = mpq.mustafar_value_formulation_quant_decode_n1(vq[0], vq[2], vq[1], vq[3], vq[4], vq[5], vq[6], p, None, D, Lc,
+                                                        Bq, groups, bit, 32 // bit)
+    assert rel_rowmax(o.cpu().numpy(), o3.cpu().numpy()) < 2e-3
+
+
 def test_quant_c_abi_rejects_bad_arguments():
     from mustafar_amd._lib import lib
     L = lib()
