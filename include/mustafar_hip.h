@@ -138,9 +138,12 @@ int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_ha
                               size_t workspace_bytes);
 /* The two phases of mstf_decode_attention_f16 as separate calls, for a caller that shards the cached
  * tokens (each shard runs `partial` on its tokens, the (max, sum, output) triples are then combined).
- * partial: per 512-token split s and query row: workspace = float part_o[Bq][ns][head_dim] followed by
- *   float part_ml[Bq][ns][2] = (max, sum of exp(w - max)), part_o un-normalised; ns = ceil(tokens / 512).
+ * partial: per token split s and query row: workspace = float part_o[Bq][ns][head_dim] followed by
+ *   float part_ml[Bq][ns][2] = (max, sum of exp(w - max)), part_o un-normalised;
+ *   ns = mstf_decode_attention_splits(tokens, head_dim, Bq, groups) <= ceil(tokens / 512): a split covers 512
+ *   tokens while every 64-token block can have a resident wavefront of its own, a multiple of that beyond.
  * merge: log-sum-exp combine of the ns splits into out (fp16) and, if given, lse_out. */
+int mstf_decode_attention_splits(int tokens, int head_dim, int Bq, int groups);
 int mstf_decode_attention_partial_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
                                       const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
                                       const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q, int tokens,

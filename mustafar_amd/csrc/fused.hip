@@ -16,17 +16,21 @@
 
 namespace mstf {
 
-// grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns token block
-// s*kFusedWaves + w.  NM = accumulator groups of four query heads (groups <= 4*NM).
+// grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns the bpw consecutive token
+// blocks (s*kFusedWaves + w)*bpw ...  NM = accumulator groups of four query heads (groups <= 4*NM).
+// MULTI = false: bpw is 1.  MULTI = true: the wavefront walks its blocks one after the other - the first value
+// stream, the boundaries and the first scalar batch of the coming block are requested while the current block is
+// still being decompressed, so only the first block of a wavefront waits for memory - and folds every block's
+// (max, sum, output) into running ones before the workgroup combine.
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
-template <int NM>
+template <int NM, bool MULTI>
 __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
     const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
     _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int Lc, int groups, int nblk,
-    int nsplit, int write_final, float sqrt_d)
+    int nsplit, int write_final, float sqrt_d, int bpw)
 {
     constexpr int D = kFusedD;
     constexpr int kQLds = NM * 4 * D * 2;          // query rows [4*NM][D] fp16
@@ -35,13 +39,17 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
     constexpr int kNeed = kNzLds + kQLds + kPLds;
     constexpr int kPark = NM * 4 * D * 4 + 64;     // per-wave (output, max, sum) parked for the workgroup combine
     constexpr int kWaveLds = kNeed > kPark ? kNeed : kPark;
+    constexpr int kStages = kKeySubs + kValSubs;
+    static_assert(kStages % 2 == 0, "the first stage of the coming block lands in buffer 0");
     __shared__ __attribute__((aligned(16))) char lds[kFusedWaves][kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
     const int split = (int)blockIdx.x;
     const int kv = (int)blockIdx.y;
-    const int tb = split * kFusedWaves + wave;
-    const bool active = tb < nblk;  // wave-uniform
+    const int tb = (split * kFusedWaves + wave) * (MULTI ? bpw : 1);  // first token block of this wavefront
+    int nb = nblk - tb;                                                // its blocks (wave-uniform)
+    if (MULTI) nb = nb > bpw ? bpw : nb;
+    const bool active = nb > 0;
     const int j = lane & 3;
     const size_t T = (size_t)Lc * D / 64;
     char* my = lds[wave];
@@ -69,23 +77,35 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         const char* nzV = v_nz + (size_t)v_nz_off[kv] * 16u;
         if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
 
-        // sub-chunk n of the walk: n < kKeySubs -> key tiles n*32.., else value tiles (n-kKeySubs)*32..
+        // sub-chunk n of a block's walk: n < kKeySubs -> key tiles n*32.., else value tiles (n-kKeySubs)*32..
         auto bm_of = [&](int n) { return n < kKeySubs ? bmK + n * kSubTiles : bmV + (n - kKeySubs) * kSubTiles; };
         auto ix_of = [&](int n) { return n < kKeySubs ? ixK + n * kSubTiles : ixV + (n - kKeySubs) * kSubTiles; };
         auto nz_of = [&](int n) { return n < kKeySubs ? nzK : nzV; };
-        // idx at the boundaries of all sub-chunks, fetched by one vector load (lanes 0.. hold the key
+        // idx at the boundaries of all sub-chunks of a block, fetched by one vector load (lanes 0.. hold the key
         // boundaries, lanes 16.. the value boundaries): no stage then waits for a scalar load from HBM
         // before it can issue its value stream
         static_assert(kKeySubs < 16 && kValSubs < 48, "boundary lanes");
-        uint32_t bnd = 0u;
-        if (lane <= kKeySubs) bnd = ixK[lane * kSubTiles];
-        else if (lane >= 16 && lane <= 16 + kValSubs) bnd = ixV[(lane - 16) * kSubTiles];
+        auto boundaries = [&](const uint32_t* ik, const uint32_t* iv) {
+            uint32_t b = 0u;
+            if (lane <= kKeySubs) b = ik[lane * kSubTiles];
+            else if (lane >= 16 && lane <= 16 + kValSubs) b = iv[(lane - 16) * kSubTiles];
+            return b;
+        };
+        uint32_t bnd = boundaries(ixK, ixV);
+        uint32_t bnd_next = bnd;  // MULTI: boundaries of the coming block
         auto issue = [&](int n) {
             const int bl = n < kKeySubs ? n : 16 + n - kKeySubs;
             const uint32_t s0 = __builtin_amdgcn_readlane(bnd, bl);
             const uint32_t s1 = __builtin_amdgcn_readlane(bnd, bl + 1);
             sub_issue(nz_of(n) + (size_t)s0 * 4u, sub_bytes(s0, s1), my + (n & 1) * kSubBytes, lane);
             return touch_sub(bm_of(n), ix_of(n), lane);
+        };
+        // first key sub-chunk of the coming block (adv = D tiles ahead; adv = 0 and no bytes after the last block)
+        auto issue_coming = [&](int adv) {
+            const uint32_t s0 = __builtin_amdgcn_readlane(bnd_next, 0);
+            const uint32_t s1 = __builtin_amdgcn_readlane(bnd_next, 1);
+            sub_issue(nzK + (size_t)s0 * 4u, adv ? sub_bytes(s0, s1) : 0u, my, lane);
+            return touch_sub(bmK + adv, ixK + adv, lane);
         };
 
         // the query rows of this KV head: groups x D fp16, contiguous
@@ -100,17 +120,15 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         }
         Touch touch = issue(0);
 
-        f4_t acc_k[NM];
-#pragma unroll
-        for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
         const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
         const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
 
         // Bitmaps and tile offsets come in batches of 8 tiles through scalar loads, each requested one batch
-        // ahead; the chain runs across the stages and from the key tiles into the value tiles.
+        // ahead; the chain runs across the stages, from the key tiles into the value tiles and (MULTI) into the
+        // coming block.
         constexpr int kBatches = kSubTiles / 8, kSideBatches = D / 8;
         Batch cur = load_batch(bmK, ixK);
-        auto stage_batches = [&](int n, uint32_t buf, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
+        auto stage_batches = [&](int n, uint32_t buf, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM], int adv) {
             const uint32_t rel = buf - cur.ov[0] * 4u;  // idx counts 4-byte units from the start of the head's values
 #pragma unroll
             for (int g = 0; g < kBatches; g++) {
@@ -119,39 +137,85 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
                 if (g1 < 2 * kSideBatches)
                     nxt = g1 < kSideBatches ? prefetch_batch(bmK + 8 * g1, ixK + 8 * g1)
                                             : prefetch_batch(bmV + 8 * (g1 - kSideBatches), ixV + 8 * (g1 - kSideBatches));
+                else if (MULTI)
+                    nxt = prefetch_batch(bmK + adv, ixK + adv);
                 batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
                 cur = nxt;
             }
         };
 
+#pragma unroll 1
+        for (int r = 0; r < (MULTI ? nb : 1); r++) {
+            const int adv = (MULTI && r + 1 < nb) ? D : 0;  // tiles to the coming block of this wavefront
+            f4_t acc_k[NM], blk_v[NM][2];
+            float m_blk[NM], l_blk[NM];
 #pragma unroll
-        for (int n = 0; n < kKeySubs + kValSubs; n++) {
-            wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for n == 0)
-            // The buffer of sub-chunk n-1 is refilled now: every LDS read of that sub-chunk fed an MFMA that was
-            // issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would also
-            // drain the scalar prefetch of the coming batch and expose its round trip at every stage.)
-            __builtin_amdgcn_sched_barrier(0);
-            if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
-            const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
-            if (n < kKeySubs) {
-                stage_batches(n, buf, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
-            } else {
-                if (n == kKeySubs) {
-                    block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
-                }
-                const int vs = n - kKeySubs;                      // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
-                constexpr int kSubsPerHalf = 64 / kSubTiles;
-                const int half = vs / kSubsPerHalf;
-                const uint32_t wa = prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u;
-                f4_t tmp[NM];
-#pragma unroll
-                for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
-                stage_batches(n, buf, wa, 4u * kPRow, tmp);
-#pragma unroll
-                for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
+            for (int m = 0; m < NM; m++) {
+                acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+                blk_v[m][0] = f4_t{0.f, 0.f, 0.f, 0.f};
+                blk_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
             }
-            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int n = 0; n < kStages; n++) {
+                wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for the first one)
+                // The buffer of sub-chunk n-1 is refilled now: every LDS read of that sub-chunk fed an MFMA that was
+                // issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would also
+                // drain the scalar prefetch of the coming batch and expose its round trip at every stage.)
+                __builtin_amdgcn_sched_barrier(0);
+                if (n + 1 < kStages) touch = issue(n + 1);
+                else if (MULTI) touch = issue_coming(adv);
+                const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
+                if (n < kKeySubs) {
+                    stage_batches(n, buf, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k, adv);
+                } else {
+                    if (n == kKeySubs) {
+                        block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_blk, l_blk);
+                        // its latency is covered by the value phase; the wait of the next stage completes it
+                        if (MULTI) bnd_next = boundaries(ixK + adv, ixV + adv);
+                    }
+                    const int vs = n - kKeySubs;                  // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
+                    constexpr int kSubsPerHalf = 64 / kSubTiles;
+                    const int half = vs / kSubsPerHalf;
+                    const uint32_t wa = prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u;
+                    f4_t tmp[NM];
+#pragma unroll
+                    for (int m = 0; m < NM; m++) tmp[m] = blk_v[m][half];
+                    stage_batches(n, buf, wa, 4u * kPRow, tmp, adv);
+#pragma unroll
+                    for (int m = 0; m < NM; m++) blk_v[m][half] = tmp[m];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (!MULTI) {
+#pragma unroll
+                for (int m = 0; m < NM; m++) {
+                    acc_v[m][0] = blk_v[m][0];
+                    acc_v[m][1] = blk_v[m][1];
+                    m_run[m] = m_blk[m];
+                    l_run[m] = l_blk[m];
+                }
+            } else {
+                // fold the block into the running triple of this wavefront (lane 4b+j: head 4m+j in every register)
+#pragma unroll
+                for (int m = 0; m < NM; m++) {
+                    const float mn = fmaxf(m_run[m], m_blk[m]);
+                    const float fa = m_run[m] == -INFINITY ? 0.f : __expf(m_run[m] - mn);
+                    const float fb = m_blk[m] == -INFINITY ? 0.f : __expf(m_blk[m] - mn);
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+#pragma unroll
+                        for (int c = 0; c < 4; c++) acc_v[m][h][c] = acc_v[m][h][c] * fa + blk_v[m][h][c] * fb;
+                    l_run[m] = l_run[m] * fa + l_blk[m] * fb;
+                    m_run[m] = mn;
+                }
+                bmK += adv;
+                ixK += adv;
+                bmV += adv;
+                ixV += adv;
+                bnd = bnd_next;
+            }
         }
+        wait_vm0();
         wait_lgkm0();
     }
 
@@ -415,14 +479,15 @@ static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, 
     return MSTF_OK;
 }
 
+// Launches the fp16 kernel over the compressed tokens; returns through *ns_out the split slots it fills
+// (slots 0 .. ns-1 of every query row; nsplit_total slots per row when a dense window adds its own behind them).
 static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
                          const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
                          const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
                          int groups, void* workspace, int write_final, int nsplit_total = 0)
 {
-    // nsplit_total: split slots per query row in the workspace (more than this launch fills when a dense window
-    // adds its own)
-    const int Bkv = Bq / groups, nblk = tokens / 64, ns = fused_nsplit(tokens);
+    const int Bkv = Bq / groups, nblk = tokens / 64;
+    const int bpw = fused_blocks_per_wave(tokens, Bkv), ns = fused_nsplit(tokens, bpw);
     const int nst = nsplit_total > 0 ? nsplit_total : ns;
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * nst * head_dim;
@@ -432,15 +497,39 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
     _Float16* oh = reinterpret_cast<_Float16*>(out);
     const float sq = sqrtf((float)head_dim);
-    if (groups <= 4)
-        hipLaunchKernelGGL(decode_attention_kernel<1>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
-                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst, write_final,
-                           sq);
-    else
-        hipLaunchKernelGGL(decode_attention_kernel<2>, grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, k_nz_off,
-                           v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst, write_final,
-                           sq);
+#define MSTF_FD(NMV, MULTIV)                                                                                         \
+    hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, \
+                       k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst,     \
+                       write_final, sq, bpw)
+    if (groups <= 4) {
+        if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
+    } else {
+        if (bpw == 1) MSTF_FD(2, false); else MSTF_FD(2, true);
+    }
+#undef MSTF_FD
     return check_launch();
+}
+
+// Merge of ns split slots per query row (layout of the partial entry point); shared with the quantised kernel.
+int mstf::merge_splits(hipStream_t st, const void* workspace, mstf_half* out, float* lse_out, int ns, int head_dim,
+                       int Bq)
+{
+    const float* part_o = reinterpret_cast<const float*>(workspace);
+    const float* part_ml = part_o + (size_t)Bq * ns * head_dim;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, st, part_o, part_ml,
+                       reinterpret_cast<_Float16*>(out), lse_out, ns, head_dim);
+    return check_launch();
+}
+
+static int splits_of(int tokens, int Bq, int groups)
+{
+    return fused_nsplit(tokens, fused_blocks_per_wave(tokens, Bq / groups));
+}
+
+extern "C" int mstf_decode_attention_splits(int tokens, int head_dim, int Bq, int groups)
+{
+    if (tokens <= 0 || head_dim != kFusedD || Bq <= 0 || groups <= 0 || tokens % 64 != 0 || Bq % groups != 0) return 0;
+    return splits_of(tokens, Bq, groups);
 }
 
 extern "C" int mstf_decode_attention_partial_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
@@ -466,12 +555,7 @@ extern "C" int mstf_decode_attention_merge_f16(void* stream, const void* workspa
     const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16) || !aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
-    const int ns = fused_nsplit(tokens);
-    const float* part_o = reinterpret_cast<const float*>(workspace);
-    const float* part_ml = part_o + (size_t)Bq * ns * head_dim;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, as_stream(stream), part_o, part_ml,
-                       reinterpret_cast<_Float16*>(out), lse_out, ns, head_dim);
-    return check_launch();
+    return merge_splits(as_stream(stream), workspace, out, lse_out, splits_of(tokens, Bq, groups), head_dim, Bq);
 }
 
 extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
@@ -486,7 +570,7 @@ extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, co
     if (rc != MSTF_OK) return rc;
     if (!aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
     // with one split and no (max, sum) requested the kernel writes the final output itself
-    const int write_final = (fused_nsplit(tokens) == 1 && !lse_out) ? 1 : 0;
+    const int write_final = (splits_of(tokens, Bq, groups) == 1 && !lse_out) ? 1 : 0;
     rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, out, tokens,
                        head_dim, Bq, groups, workspace, write_final);
     if (rc != MSTF_OK || write_final) return rc;
@@ -525,7 +609,7 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
     const size_t need = mstf_decode_attention_window_workspace_bytes(tokens, win_len, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
-    const int ns = fused_nsplit(tokens), nwb = window_blocks(win_len), nst = ns + nwb;
+    const int ns = tokens > 0 ? splits_of(tokens, Bq, groups) : 0, nwb = window_blocks(win_len), nst = ns + nwb;
     const int Bkv = Bq / groups;
     int rc;
     if (tokens > 0) {

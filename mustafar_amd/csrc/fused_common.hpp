@@ -11,7 +11,27 @@ constexpr int kFusedWaves = 8;    // token blocks (= wavefronts) per workgroup: 
 constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
 constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
 
-static inline int fused_nsplit(int tokens) { return (tokens / 64 + kFusedWaves - 1) / kFusedWaves; }
+constexpr int kFusedResident = 4096;  // wavefronts of the fused kernel the 256 CUs hold at once (16 per CU)
+constexpr int kFusedMaxBpw = 8;
+
+// Token blocks one wavefront of the fp16 kernel walks: 1 while every block can have a resident wavefront of its
+// own; beyond that the blocks are spread over one chip-filling set of wavefronts, so that only a wavefront's first
+// block waits for memory.
+static inline int fused_blocks_per_wave(int tokens, int Bkv)
+{
+    const long long blocks = (long long)Bkv * (tokens / 64);
+    const long long r = (blocks + kFusedResident - 1) / kFusedResident;
+    return r < 1 ? 1 : (r > kFusedMaxBpw ? kFusedMaxBpw : (int)r);
+}
+// Split slots (= workgroups) per KV head: kFusedWaves * bpw token blocks each.
+static inline int fused_nsplit(int tokens, int bpw = 1)
+{
+    return (tokens / 64 + kFusedWaves * bpw - 1) / (kFusedWaves * bpw);
+}
+
+// Launches the merge of ns split slots per query row out of a workspace in the layout of the fused kernels
+// (defined beside the merge kernel).
+int merge_splits(hipStream_t st, const void* workspace, mstf_half* out, float* lse_out, int ns, int head_dim, int Bq);
 
 __device__ __forceinline__ float wave_max_same_column(float v)
 {

@@ -237,5 +237,5 @@ extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, 
 #undef MSTF_FQ
     int rc = check_launch();
     if (rc != MSTF_OK || write_final) return rc;
-    return mstf_decode_attention_merge_f16(stream, workspace, workspace_bytes, out, lse_out, tokens, head_dim, Bq, groups);
+    return merge_splits(st, workspace, out, lse_out, ns, head_dim, Bq);
 }

@@ -83,15 +83,16 @@ def test_format_invariants_and_checksums(data, is_value):
     assert int((nz != 0).sum()) == int(pop.sum())
 
 
-def dense_masked_attention(q, Kp, Vp):
+def dense_masked_attention(q, Kp, Vp, groups=GROUPS):
     """The reference's dense path on pruned tensors (models/llama_mustafar_Kt_Mag_Vt_Mag.py:836-1026): fp16 scores with
     fp32 accumulation, / sqrt(d) in fp16, fp32 softmax rounded to fp16, fp32-accumulated P.V rounded to fp16."""
-    qh = q.view(BKV, GROUPS, D).float()
+    bkv, length = Kp.shape[0], Kp.shape[1]
+    qh = q.view(bkv, groups, D).float()
     s = torch.einsum("bgd,bld->bgl", qh, Kp.float()).half()
     w = (s / math.sqrt(D)).float()
     p = torch.softmax(w, -1).half()
     o = torch.einsum("bgl,bld->bgd", p.float(), Vp.float()).half()
-    return s.view(-1, L), p.view(-1, L), o.view(-1, D)
+    return s.view(-1, length), p.view(-1, length), o.view(-1, D)
 
 
 def rel_rowmax(a, b):
@@ -124,6 +125,42 @@ def test_decode_attention_full_size(data):
     # linearity of the value product in the probabilities: P -> 0.5 P halves the output exactly (power of two)
     o_half = ops.value_spmv(cv, (p * 0.5).contiguous(), GROUPS)
     assert torch.equal(o_half.float() * 2, o.float()) or rel_rowmax(o_half[:, 0] * 2, o[:, 0]) < 1e-3
+
+
+@pytest.mark.parametrize("bkv,blocks,groups", [(140, 31, 4), (150, 56, 2), (40, 112, 8), (600, 64, 1)])
+def test_decode_attention_many_blocks(bkv, blocks, groups):
+    """More 64-token blocks than resident wavefronts: every wavefront of the fused kernel walks several blocks
+    (2, 3, 2 and 8 here, with a ragged last wavefront in the first two) and folds them before the workgroup combine."""
+    from mustafar_amd import ops
+    from mustafar_amd._lib import lib
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(bkv * 1000 + blocks)
+    length = blocks * 64
+    K = torch.randn((bkv, length, D), generator=g, device=dev).half()
+    V = torch.randn((bkv, length, D), generator=g, device=dev).half()
+    K[:, :, 9] *= 8
+    q = torch.randn((bkv * groups, D), generator=g, device=dev).half()
+    Bq = bkv * groups
+    ns = lib().mstf_decode_attention_splits(length, D, Bq, groups)
+    assert 0 < ns < (blocks + 7) // 8 or blocks <= 8
+    s_ref, _, o_ref = dense_masked_attention(q, torch_prune(K, KTH), torch_prune(V, KTH), groups)
+    ck = ops.compress(K, False, kth=KTH)
+    cv = ops.compress(V, True, kth=KTH)
+    lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
+    o = ops.decode_attention(ck, cv, q, groups, lse=lse)
+    assert rel_rowmax(o, o_ref) < 2e-3
+    w = (s_ref / math.sqrt(D)).float()
+    m_ref = w.amax(-1)
+    assert float((lse[:, 0] - m_ref).abs().max()) <= 2e-2 * max(float(m_ref.abs().max()), 1.0)
+    l_ref = torch.exp(w - m_ref[:, None]).sum(-1)
+    assert float((lse[:, 1] * torch.exp(lse[:, 0] - m_ref) - l_ref).abs().max()) <= 5e-3 * float(l_ref.max())
+    o2 = ops.decode_attention(ck, cv, q, groups)            # route without (max, sum) output
+    assert rel_rowmax(o2, o_ref) < 2e-3
+    # the three-launch path on the same cache
+    p = ops.scale_softmax(ops.key_spmv(ck, q.view(Bq, 1, D), groups), D)
+    o3 = ops.value_spmv(cv, p, groups)
+    assert rel_rowmax(o, o3[:, 0]) < 2e-3
 
 
 def test_compress_twice_is_idempotent(data):

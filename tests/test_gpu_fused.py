@@ -66,7 +66,9 @@ def test_partial_then_merge_equals_fused():
     o2 = ops.decode_attention_merge(ws, Lc, D, Bq, groups, lse=lse2)
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
     # the splits themselves: (max, sum, un-normalised output) of every 512-token range, combined on the host
-    ns = (Lc // 64 + 7) // 8
+    from mustafar_amd._lib import lib
+    ns = lib().mstf_decode_attention_splits(Lc, D, Bq, groups)
+    assert ns == (Lc // 64 + 7) // 8   # few blocks: 512 tokens per split
     raw = ws[: Bq * ns * (D + 2) * 4].view(torch.float32).cpu().numpy()
     po = raw[: Bq * ns * D].reshape(Bq, ns, D).astype(np.float64)
     ml = raw[Bq * ns * D:].reshape(Bq, ns, 2).astype(np.float64)
