@@ -19,37 +19,47 @@
 namespace mstf {
 
 // ------------------------------------------------------------------------------- count
-// grid = B * M/64 units, 64 threads.  Writes bmp, unit-local exclusive offsets into idx[b][t]
-// and the unit total into unit_tot[b][tokblk].
+// grid = ceil(units / upw) with units = B * M/64, 64 threads: the wavefront owns upw consecutive units and has
+// the rows of the coming one in flight while it selects and packs the current one.  Writes bmp, unit-local
+// exclusive offsets into idx[b][t] and the unit total into unit_tot[b][tokblk].
 template <bool IS_VALUE>
 __global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __restrict__ x, int M, int kth,
                                                             uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
-                                                            uint32_t* __restrict__ unit_tot)
+                                                            uint32_t* __restrict__ unit_tot, int units, int upw)
 {
     __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int nblk = M / 64;
-    const int unit = (int)blockIdx.x;
-    const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
-    uint32_t mag[64];
-    unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane, mag);
+    const int unit0 = (int)blockIdx.x * upw;
+    int n = units - unit0;
+    n = n > upw ? upw : n;
+    UnitRaw raw;
+    unit_fetch(x, (int64_t)unit0 * 64, lane, raw);  // units are contiguous: unit u = rows [64u, 64u + 64) of [B*M, 128]
+#pragma unroll 1
+    for (int u = 0; u < n; u++) {
+        const int unit = unit0 + u;
+        const int b = unit / nblk, tb = unit - b * nblk;
+        uint32_t mag[64];
+        unit_rows_from(raw, slab, lane, mag);
+        if (u + 1 < n) unit_fetch(x, (int64_t)(unit + 1) * 64, lane, raw);
 #pragma unroll
-    for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
-    const uint32_t thr = threshold_of(mag, kth);
-    uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
-    unit_bitmaps<IS_VALUE>(mag, thr, lane, bmA, bmB);
-    uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
-    bo[lane] = bmA;
-    bo[64 + lane] = bmB;
-    const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
-    uint32_t totA, totB;
-    const uint32_t eA = wave_excl_scan(cA, lane, totA);
-    const uint32_t eB = wave_excl_scan(cB, lane, totB);
-    uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
-    io[lane] = eA;
-    io[64 + lane] = totA + eB;
-    if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
+        for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
+        const uint32_t thr = threshold_of(mag, kth);
+        uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
+        unit_bitmaps<IS_VALUE>(mag, thr, lane, bmA, bmB);
+        uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
+        bo[lane] = bmA;
+        bo[64 + lane] = bmB;
+        const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
+        uint32_t totA, totB;
+        const uint32_t eA = wave_excl_scan(cA, lane, totA);
+        const uint32_t eB = wave_excl_scan(cB, lane, totB);
+        uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
+        io[lane] = eA;
+        io[64 + lane] = totA + eB;
+        if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
+    }
 }
 
 // ------------------------------------------------------------------------------- scans
@@ -258,6 +268,18 @@ static int scatter_impl(void* stream, const mstf_half* x, int B, int M, int N, c
     return check_launch();
 }
 
+// Units per wavefront of the count kernel: two once that still fills the chip (its loads then overlap its
+// arithmetic), one for small inputs.
+template <bool IS_VALUE>
+static void launch_count(hipStream_t st, const _Float16* xh, int B, int M, int kth, uint64_t* bmp, uint32_t* idx,
+                         uint32_t* unit_tot)
+{
+    const int units = B * (M / 64);
+    const int upw = units >= 4096 ? 2 : 1;
+    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)((units + upw - 1) / upw)), dim3(64), 0, st, xh,
+                       M, kth, bmp, idx, unit_tot, units, upw);
+}
+
 template <bool IS_VALUE>
 static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp, uint32_t* idx,
                          uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz, uint64_t cap, void* ws,
@@ -277,8 +299,7 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
     uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
-    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bmp, idx,
-                       unit_tot);
+    launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
                        head_tot, nblk, kD);
@@ -318,8 +339,7 @@ static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, in
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
     uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
-    hipLaunchKernelGGL(compress_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bmp, idx,
-                       unit_tot);
+    launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
                        head_tot, nblk, kD);

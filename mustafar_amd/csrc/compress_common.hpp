@@ -55,6 +55,43 @@ __device__ __forceinline__ void unit_rows(const _Float16* x, int64_t row0, int64
     }
 }
 
+// The same in two steps, for a wavefront that requests its next unit while it works on the current one:
+// unit_fetch leaves the 16 KB of a whole unit (64 full rows from row0, all valid) in the registers of the
+// wavefront, unit_rows_from turns them into the lane's row.
+struct UnitRaw {
+    uint4 v[2][8];
+};
+__device__ __forceinline__ void unit_fetch(const _Float16* x, int64_t row0, int lane, UnitRaw& raw)
+{
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD) + h * 8;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = j * 64 + lane;
+            raw.v[h][j] = src[(e >> 3) * 16 + (e & 7)];
+        }
+    }
+}
+__device__ __forceinline__ void unit_rows_from(const UnitRaw& raw, uint32_t* slab, int lane, uint32_t (&r)[64])
+{
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = j * 64 + lane;
+            uint32_t* d = slab + (e >> 3) * kHalfRowDw + (e & 7) * 4;
+            d[0] = raw.v[h][j].x;
+            d[1] = raw.v[h][j].y;
+            d[2] = raw.v[h][j].z;
+            d[3] = raw.v[h][j].w;
+        }
+        __builtin_amdgcn_wave_barrier();
+        row_of_lane(slab, lane, r, 32 * h);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // kth-th smallest (1-based) of the 128 fp16 magnitudes of this lane's row.
 // mag[j] holds two 15-bit magnitudes.  Greedy MSB-first: the answer is the largest c with
 // #(mag < c) < kth.  The count comes from sums of absolute differences, one v_sad_u16 per register:
@@ -103,6 +140,13 @@ __device__ __forceinline__ uint32_t padded_units(uint64_t bm)
 }
 
 
+// dst with lane LANE (a constant) replaced by the wave-uniform value v.
+__device__ __forceinline__ uint32_t write_lane(uint32_t v, int lane_const, uint32_t dst)
+{
+    asm("v_writelane_b32 %0, %1, %2" : "+v"(dst) : "s"(v), "n"(lane_const));
+    return dst;
+}
+
 // Keep decision of one unit, as tile bitmaps (MSB-first).  Lane l returns the bitmaps of tiles
 // l (bmA) and 64+l (bmB) of the unit:
 //   key   : tile c = channel c over the 64 tokens        (ballot across lane = token)
@@ -115,22 +159,29 @@ __device__ __forceinline__ void unit_bitmaps(const uint32_t (&mag)[64], uint32_t
 {
     const us2_t t2 = as_us2(thr | (thr << 16));
     if (!IS_VALUE) {
-        bmA = 0;
-        bmB = 0;
+        // one 16-bit compare per channel; the wave-wide result goes into the lane that owns the tile with two
+        // v_writelane (the lane index is a compile-time constant)
+        uint32_t aLo = 0u, aHi = 0u, bLo = 0u, bHi = 0u;
+        const uint16_t t16 = (uint16_t)thr;
 #pragma unroll
         for (int j = 0; j < 64; j++) {
-            const uint32_t d = us2_u32(as_us2(mag[j]) - t2);  // bit 15 / 31 set <=> pruned
-            const uint64_t k0 = __builtin_bitreverse64(__ballot((d & 0x8000u) == 0u));
-            const uint64_t k1 = __builtin_bitreverse64(__ballot((d & 0x80000000u) == 0u));
-            const int c0 = 2 * j, c1 = 2 * j + 1;
-            if (c0 < 64) {
-                bmA = (lane == c0) ? k0 : bmA;
-                bmA = (lane == c1) ? k1 : bmA;
+            const uint64_t k0 = __builtin_bitreverse64(__ballot((uint16_t)mag[j] >= t16));
+            const uint64_t k1 = __builtin_bitreverse64(__ballot((uint16_t)(mag[j] >> 16) >= t16));
+            const int c0 = (2 * j) & 63, c1 = (2 * j + 1) & 63;
+            if (j < 32) {
+                aLo = write_lane((uint32_t)k0, c0, aLo);
+                aHi = write_lane((uint32_t)(k0 >> 32), c0, aHi);
+                aLo = write_lane((uint32_t)k1, c1, aLo);
+                aHi = write_lane((uint32_t)(k1 >> 32), c1, aHi);
             } else {
-                bmB = (lane == c0 - 64) ? k0 : bmB;
-                bmB = (lane == c1 - 64) ? k1 : bmB;
+                bLo = write_lane((uint32_t)k0, c0, bLo);
+                bHi = write_lane((uint32_t)(k0 >> 32), c0, bHi);
+                bLo = write_lane((uint32_t)k1, c1, bLo);
+                bHi = write_lane((uint32_t)(k1 >> 32), c1, bHi);
             }
         }
+        bmA = u64_of(aLo, aHi);
+        bmB = u64_of(bLo, bHi);
     } else {
         uint32_t w[4] = {0u, 0u, 0u, 0u};  // [half0 hi, half0 lo, half1 hi, half1 lo]
 #pragma unroll
