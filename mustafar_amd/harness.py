@@ -72,19 +72,23 @@ class DenseMaskedCache:
 
 
 def _rms_norm(x, w, eps):
-    xf = x.float()
-    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+    return F.rms_norm(x, (x.shape[-1],), w, eps)
 
 
-def _rope(x, pos, theta):
-    """x: [bs, heads, L, D]; pos: [L] positions."""
-    D = x.shape[-1]
-    inv = 1.0 / (theta ** (torch.arange(0, D, 2, device=x.device, dtype=torch.float32) / D))
+def _rope_tables(pos, D, theta, dtype):
+    """cos and signed sin of the rotary embedding for positions pos [L]: [L, D] each, sin negated in the first half,
+    so that x * cos + roll(x, D/2) * sin_signed == x * cos + rotate_half(x) * sin product by product."""
+    inv = 1.0 / (theta ** (torch.arange(0, D, 2, device=pos.device, dtype=torch.float32) / D))
     ang = pos.float()[:, None] * inv[None, :]
-    cos = torch.cat([ang.cos(), ang.cos()], -1).to(x.dtype)
-    sin = torch.cat([ang.sin(), ang.sin()], -1).to(x.dtype)
-    x1, x2 = x[..., : D // 2], x[..., D // 2:]
-    return x * cos + torch.cat([-x2, x1], -1) * sin
+    cos = torch.cat([ang.cos(), ang.cos()], -1).to(dtype)
+    sin = torch.cat([-ang.sin(), ang.sin()], -1).to(dtype)
+    return cos, sin
+
+
+def _rope(x, tables):
+    """x: [bs, heads, L, D]; tables from _rope_tables for the L positions."""
+    cos, sin = tables
+    return x * cos + torch.roll(x, x.shape[-1] // 2, -1) * sin
 
 
 class Decoder:
@@ -121,23 +125,24 @@ class Decoder:
         gate, up = gu.chunk(2, -1)
         return F.linear(F.silu(gate) * up, lw["down"])
 
-    def _qkv(self, lw, x, pos):
+    def _qkv(self, lw, x, tables):
         c = self.cfg
         bs, L, _ = x.shape
         qkv = F.linear(x, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim).transpose(1, 2)
-        q, k, v = qkv[:, : c.n_q], qkv[:, c.n_q: c.n_q + c.n_kv], qkv[:, c.n_q + c.n_kv:]
-        return _rope(q, pos, c.rope_theta), _rope(k, pos, c.rope_theta).contiguous(), v.contiguous()
+        qk = _rope(qkv[:, : c.n_q + c.n_kv], tables)   # query and key heads in one pass; contiguous [bs, heads, L, D]
+        return qk[:, : c.n_q], qk[:, c.n_q:], qkv[:, c.n_q + c.n_kv:].contiguous()
 
     @torch.no_grad()
     def prefill(self, ids, seq_chunk=4):
         """ids: [bs, L].  Returns the logits of the last position; fills the caches."""
         c = self.cfg
         bs, L = ids.shape
-        pos = torch.arange(L, device=self.dev)
+        tables = _rope_tables(torch.arange(L, device=self.dev), c.head_dim, c.rope_theta, torch.float16)
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            q, k, v = self._qkv(lw, h, pos)
+            q, k, v = self._qkv(lw, h, tables)
+            k = k.contiguous()
             outs = []
             for b0 in range(0, bs, seq_chunk):   # bounded working set of the prefill attention
                 outs.append(F.scaled_dot_product_attention(q[b0:b0 + seq_chunk], k[b0:b0 + seq_chunk], v[b0:b0 + seq_chunk],
@@ -158,10 +163,11 @@ class Decoder:
 
     def _layers(self, ids, pos, timed, attend):
         c = self.cfg
+        tables = _rope_tables(pos, c.head_dim, c.rope_theta, torch.float16)   # once per step, shared by the layers
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            q, k, v = self._qkv(lw, h, pos)
+            q, k, v = self._qkv(lw, h, tables)
             if timed:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
