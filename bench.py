@@ -12,6 +12,7 @@ reads come from HBM, not from the 256 MB Infinity Cache.  Prints exactly one JSO
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -102,6 +103,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
     ap.add_argument("--unfused", action="store_true", help="step = the three separate operator launches")
     ap.add_argument("--no-quant", action="store_true", help="skip the stage timings of the quantised format")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 attention timed beside the sparse path")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one GPU "
@@ -124,6 +126,7 @@ def main():
 
     # ---- build the rotating compressed caches (also times the fused prune+compress kernels)
     caches = []
+    dense = []   # the same tokens uncompressed, for the dense fp16 attention timed beside the sparse path
     t_ck = t_cv = 0.0
     for i in range(args.caches):
         K, V = make_kv(torch, dev, Bkv, L, D, gen)
@@ -132,6 +135,8 @@ def main():
             ops.compress(K, False, kth=kth, capacity_halfs=cap)  # warm-up (module load)
         t_ck += event_time_us(torch, lambda: caches.append([ops.compress(K, False, kth=kth, capacity_halfs=cap)]), 1)
         t_cv += event_time_us(torch, lambda: caches[-1].append(ops.compress(V, True, kth=kth, capacity_halfs=cap)), 1)
+        if not args.no_dense:
+            dense.append((K.view(bs, nkv, L, D), V.view(bs, nkv, L, D)))
         del K, V
     t_ck /= args.caches
     t_cv /= args.caches
@@ -223,6 +228,40 @@ def main():
     key_us = event_time_us(torch, lambda: ops.key_spmv(rot(0), q, groups, out=s), n)
     val_us = event_time_us(torch, lambda: ops.value_spmv(rot(1), p, groups, out=o), n)
     sm_us = event_time_us(torch, lambda: ops.scale_softmax(s, D, out=p), n)
+
+    # dense fp16 decode attention over the same (unpruned) tokens with library operators, cold caches rotated alike:
+    # what the sparse path has to beat.  "matmul" batches the query heads of a KV head into one product, so K and V
+    # are read once per KV head as in the sparse kernels; "sdpa" is torch's fused attention operator.
+    dense_us = None
+    if dense:
+        import torch.nn.functional as F
+        q5 = q.view(bs, nkv, groups, D)
+        q4 = q.view(bs, nq, 1, D)
+
+        def dense_matmul(i):
+            Kd, Vd = dense[i]
+            w = torch.matmul(q5, Kd.transpose(2, 3)) / math.sqrt(D)
+            return torch.matmul(torch.softmax(w, -1, dtype=torch.float32).half(), Vd)
+
+        def dense_sdpa(i):
+            Kd, Vd = dense[i]
+            return F.scaled_dot_product_attention(q4, Kd, Vd, enable_gqa=True)
+
+        def ring_time_us(fn):
+            """One step on each rotating cache captured into one HIP graph (as the sparse step is), replayed."""
+            for i in range(args.caches):
+                fn(i)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(args.caches):
+                    fn(i)
+            g.replay()
+            reps = max(n // args.caches, 5)
+            return event_time_us(torch, g.replay, reps) / args.caches
+
+        dense_us = {"matmul_softmax_matmul": round(ring_time_us(dense_matmul), 2),
+                    "sdpa": round(ring_time_us(dense_sdpa), 2), "bytes": int(2 * Bkv * L * D * 2)}
 
     # quantised format (2- and 4-bit codes) on the same shape: producer once, then the key / value SpMVs with one
     # row per query head through the C ABI
@@ -317,6 +356,7 @@ def main():
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
                       "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
         "quant_stages_us": quant_us,
+        "dense_fp16_attention_us": dense_us,
         "hbm_gbs_on_compressed_bytes": {"fused_decode_attention": round(fused_alg / fused_us / 1e3, 1),
                                         "key_spmv": round(key_alg / key_us / 1e3, 1),
                                         "value_spmv": round(val_alg / val_us / 1e3, 1),
