@@ -1,0 +1,77 @@
+"""The HIP path, through the C ABI, against the committed known-answer fixtures (tests/golden/*.npz): bit-exact for
+pruned rows, bitmaps, offsets and packed values (fp16 and quantised), 2e-3 / 1e-2 for the attention results."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def load(name):
+    return np.load(os.path.join(GOLDEN, name), allow_pickle=False)
+
+
+def gpu_f16(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.float16)).to("cuda:0")
+
+
+def bits(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+def rel_rowmax(a, b):
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
+
+
+@pytest.mark.parametrize("fused_prune", [True, False])
+def test_compress_reproduces_the_fixture(fused_prune):
+    from mustafar_amd import ops
+    g = load("kat_fp16.npz")
+    kth = int(g["kth"])
+    for src, pruned, pre, is_value in (("K", "Kp", "k", False), ("V", "Vp", "v", True)):
+        x = gpu_f16(g[src])
+        xp = ops.prune_rows(x.view(-1, 128), kth).view(x.shape)
+        assert np.array_equal(bits(xp), g[pruned])
+        c = ops.compress(x, is_value, kth=kth) if fused_prune else ops.compress(gpu_f16(g[pruned]), is_value, kth=0)
+        assert np.array_equal(c.bmp.cpu().numpy(), g[pre + "_bmp"])
+        assert np.array_equal(c.idx.cpu().numpy(), g[pre + "_idx"])
+        assert np.array_equal(c.nz_off.cpu().numpy(), g[pre + "_nz_off"])
+        assert np.array_equal(bits(c.packed()), g[pre + "_nz"])
+
+
+def test_attention_reproduces_the_fixture():
+    from mustafar_amd import ops
+    g = load("kat_attention.npz")
+    kth, groups = int(g["kth"]), int(g["groups"])
+    q = gpu_f16(g["q"])
+    Bq, D = q.shape
+    want_s, want_p, want_o = (g[n].view(np.float16) for n in ("scores", "probs", "out"))
+    ck = ops.compress(gpu_f16(g["K"]), False, kth=kth)
+    cv = ops.compress(gpu_f16(g["V"]), True, kth=kth)
+    s = ops.key_spmv(ck, q.view(Bq, 1, D), groups)
+    assert rel_rowmax(s[:, 0].cpu().numpy(), want_s) < 2e-3
+    p = ops.scale_softmax(s, D)
+    assert rel_rowmax(p[:, 0].cpu().numpy(), want_p) < 2e-3
+    o = ops.value_spmv(cv, p, groups)
+    assert rel_rowmax(o[:, 0].cpu().numpy(), want_o) < 2e-3
+    assert rel_rowmax(ops.decode_attention(ck, cv, q, groups).cpu().numpy(), want_o) < 2e-3
+
+
+@pytest.mark.parametrize("bit", [2, 4])
+def test_quant_producer_reproduces_the_fixture(bit):
+    from mustafar_amd import compression_quant as cq
+    g, want = load("kat_fp16.npz"), load("kat_quant.npz")
+    names = ["bmp", "tile_off", "packed", "counts", "units", "scales", "zeros"]
+    for pruned, pre, is_value in (("Kp", "k", False), ("Vp", "v", True)):
+        x = gpu_f16(g[pruned])
+        got = cq.convert_value_batched_quant(x, bit=bit) if is_value else \
+            cq.convert_key_batched_quant(x, return_metadata=True, bit=bit)
+        for name, t in zip(names, got):
+            a = t.cpu().numpy()
+            a = a.view(np.uint16) if a.dtype == np.float16 else a
+            assert np.array_equal(a, want["%s%d_%s" % (pre, bit, name)]), name
