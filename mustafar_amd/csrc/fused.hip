@@ -223,29 +223,46 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
                           out, part_o, part_ml);
 }
 
-// grid = Bq, 128 threads: log-sum-exp combine of the token splits.
+// grid = Bq, 128 threads: log-sum-exp combine of the token splits.  The splits are taken eight at a time: the
+// (max, sum) pairs and the partial outputs of a group are requested together, so a group costs one memory round
+// trip, and the groups are folded into running (max, output, sum) values.
 __global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restrict__ part_o,
                                                            const float* __restrict__ part_ml,
                                                            _Float16* __restrict__ out, float* __restrict__ lse_out,
                                                            int nsplit, int D)
 {
+    constexpr int G = 8;
     const size_t row = blockIdx.x;
-    const int c = (int)threadIdx.x;
-    const float* ml = part_ml + row * nsplit * 2;
+    const int c = (int)threadIdx.x < D ? (int)threadIdx.x : D - 1;
+    const float2* ml = reinterpret_cast<const float2*>(part_ml) + row * nsplit;
     const float* po = part_o + row * nsplit * D + c;
-    // the loads of a loop are independent of each other: unrolled, eight of them are in flight at a time
-    float M = -INFINITY;
-#pragma unroll 8
-    for (int s = 0; s < nsplit; s++) M = fmaxf(M, ml[s * 2]);
-    float so = 0.f, sl = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < nsplit; s++) {
-        const float f = __expf(ml[s * 2] - M);
-        so += f * po[(size_t)s * D];
-        sl += f * ml[s * 2 + 1];
+    float M = -INFINITY, so = 0.f, sl = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += G) {
+        float2 m[G];
+        float o[G];
+#pragma unroll
+        for (int u = 0; u < G; u++) {
+            const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;  // clamped: the loads stay unconditional
+            m[u] = ml[s];
+            o[u] = po[(size_t)s * D];
+        }
+        float gm = M;
+#pragma unroll
+        for (int u = 0; u < G; u++)
+            if (s0 + u < nsplit) gm = fmaxf(gm, m[u].x);
+        const float fr = M == -INFINITY ? 0.f : __expf(M - gm);
+        so *= fr;
+        sl *= fr;
+#pragma unroll
+        for (int u = 0; u < G; u++) {
+            const float f = (s0 + u < nsplit && m[u].x != -INFINITY) ? __expf(m[u].x - gm) : 0.f;
+            so += f * o[u];
+            sl += f * m[u].y;
+        }
+        M = gm;
     }
-    if (c < D) out[row * D + c] = (_Float16)(so / sl);
-    if (lse_out && c == 0) {
+    if ((int)threadIdx.x < D) out[row * D + c] = (_Float16)(so / sl);
+    if (lse_out && threadIdx.x == 0) {
         lse_out[row * 2] = M;
         lse_out[row * 2 + 1] = sl;
     }
