@@ -121,13 +121,26 @@ class Decoder:
         self.attn_events = []   # (start, end) pairs around the cache's decode of every layer of timed steps
 
     def _mlp(self, lw, x):
-        gu = F.linear(x, lw["gate_up"])
-        gate, up = gu.chunk(2, -1)
+        # two products over the halves of the stacked weight: both results are contiguous, so the activation and
+        # the gating run as vectorised elementwise kernels
+        ffn = self.cfg.ffn
+        gate, up = F.linear(x, lw["gate_up"][:ffn]), F.linear(x, lw["gate_up"][ffn:])
         return F.linear(F.silu(gate) * up, lw["down"])
 
     def _qkv(self, lw, x, tables):
         c = self.cfg
         bs, L, _ = x.shape
+        if L == 1:
+            # decode step: one contiguous pass over all heads; the value heads go through with cos = 1, sin = 0
+            cos, sin = tables
+            H = c.n_q + 2 * c.n_kv
+            if cos.shape[0] != H:
+                one = torch.ones((c.n_kv, c.head_dim), dtype=cos.dtype, device=cos.device)
+                cos = torch.cat([cos.expand(c.n_q + c.n_kv, -1), one], 0)
+                sin = torch.cat([sin.expand(c.n_q + c.n_kv, -1), torch.zeros_like(one)], 0)
+                tables[0], tables[1] = cos, sin        # built by the first layer of the step, reused by the others
+            qkv = _rope(F.linear(x, lw["qkv"]).view(bs, H, c.head_dim), (cos, sin)).unsqueeze(2)
+            return qkv[:, : c.n_q], qkv[:, c.n_q: c.n_q + c.n_kv], qkv[:, c.n_q + c.n_kv:]
         qkv = F.linear(x, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim).transpose(1, 2)
         qk = _rope(qkv[:, : c.n_q + c.n_kv], tables)   # query and key heads in one pass; contiguous [bs, heads, L, D]
         return qk[:, : c.n_q], qk[:, c.n_q:], qkv[:, c.n_q + c.n_kv:].contiguous()
@@ -163,7 +176,7 @@ class Decoder:
 
     def _layers(self, ids, pos, timed, attend):
         c = self.cfg
-        tables = _rope_tables(pos, c.head_dim, c.rope_theta, torch.float16)   # once per step, shared by the layers
+        tables = list(_rope_tables(pos, c.head_dim, c.rope_theta, torch.float16))   # once per step, shared by the layers
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
