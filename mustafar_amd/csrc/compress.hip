@@ -8,7 +8,7 @@
 //
 //   count kernel   : row threshold by a 15-step radix select on the fp16 magnitudes, bitmaps by ballot
 //                    (key) or in-lane packing (value), padded counts and their prefix inside the unit.
-//   scan kernels   : unit totals -> unit bases per head, head totals -> nz_off.
+//   scan kernel    : unit totals -> unit bases per head and, summed over the earlier heads, nz_off.
 //   scatter kernel : re-reads the slab and compacts the survivors, half a unit (64 tiles) at a time,
 //                    into an LDS image of the output that reuses the staging buffer - key: one
 //                    rank-addressed 2-byte write per tile straight from the registers; value: every lane
@@ -23,7 +23,7 @@ namespace mstf {
 // the rows of the coming one in flight while it selects and packs the current one.  Writes bmp, unit-local
 // exclusive offsets into idx[b][t] and the unit total into unit_tot[b][tokblk].
 template <bool IS_VALUE>
-__global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __restrict__ x, int M, int kth,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void compress_count_kernel(const _Float16* __restrict__ x, int M, int kth,
                                                             uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
                                                             uint32_t* __restrict__ unit_tot, int units, int upw)
 {
@@ -45,9 +45,8 @@ __global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __re
         if (u + 1 < n) unit_fetch(x, (int64_t)(unit + 1) * 64, lane, raw);
 #pragma unroll
         for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
-        const uint32_t thr = threshold_of(mag, kth);
         uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
-        unit_bitmaps<IS_VALUE>(mag, thr, lane, bmA, bmB);
+        unit_keep<IS_VALUE>(mag, kth, lane, bmA, bmB);
         uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
         bo[lane] = bmA;
         bo[64 + lane] = bmB;
@@ -63,20 +62,38 @@ __global__ __launch_bounds__(64) void compress_count_kernel(const _Float16* __re
 }
 
 // ------------------------------------------------------------------------------- scans
-// grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base, idx[b][T] = head total,
-// head_tot[b] = head total (4-byte units).
+// grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base, idx[b][T] = head total.
+// With nz_off given (the compress entry points) the workgroup also adds up the unit totals of all earlier heads:
+// nz_off[b] = that sum / 4 (16-byte units), and the last head's workgroup writes the grand total in fp16 values.
+// Every workgroup re-reads at most B * nblk small numbers, which spares a launch for the scan over heads.
 __global__ __launch_bounds__(256) void scan_units_kernel(const uint32_t* __restrict__ unit_tot,
                                                          uint32_t* __restrict__ unit_base, uint32_t* __restrict__ idx,
-                                                         uint32_t* __restrict__ head_tot, int nblk, int tiles_per_unit)
+                                                         uint32_t* __restrict__ nz_off,
+                                                         uint64_t* __restrict__ total_halfs, int nblk,
+                                                         int tiles_per_unit)
 {
     extern __shared__ uint32_t base[];  // nblk entries
+    __shared__ uint64_t wsum[4];
     const int b = (int)blockIdx.x;
     const int tid = (int)threadIdx.x;
     const uint32_t total = units_scan(unit_tot + (size_t)b * nblk, base, nblk);
     for (int i = tid; i < nblk; i += 256) unit_base[(size_t)b * nblk + i] = base[i];
-    if (tid == 0) {
-        idx[(size_t)b * ((size_t)nblk * tiles_per_unit + 1) + (size_t)nblk * tiles_per_unit] = total;
-        head_tot[b] = total;
+    if (tid == 0) idx[(size_t)b * ((size_t)nblk * tiles_per_unit + 1) + (size_t)nblk * tiles_per_unit] = total;
+    if (nz_off) {
+        uint64_t mine = 0;
+        const size_t before = (size_t)b * nblk;
+        // the loads of a pass are independent: unrolled, eight of them are in flight at a time
+#pragma unroll 8
+        for (size_t i = tid; i < before; i += 256) mine += unit_tot[i];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+        if ((tid & 63) == 0) wsum[tid >> 6] = mine;
+        __syncthreads();
+        if (tid == 0) {
+            const uint64_t pre = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+            nz_off[b] = (uint32_t)(pre >> 2);
+            if (b == (int)gridDim.x - 1) *total_halfs = 2ull * (pre + total);
+        }
     }
 }
 
@@ -89,14 +106,6 @@ __global__ __launch_bounds__(256) void finalize_idx_kernel(uint32_t* __restrict_
     const size_t T = (size_t)nblk * tiles_per_unit;
     const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (t < T) idx[(size_t)b * (T + 1) + t] += unit_base[(size_t)b * nblk + t / tiles_per_unit];
-}
-
-// one workgroup: nz_off[b] = (sum of earlier head totals) / 4 (16-byte units); total in fp16 values.
-__global__ __launch_bounds__(1024) void scan_heads_kernel(const uint32_t* __restrict__ head_tot,
-                                                          uint32_t* __restrict__ nz_off,
-                                                          uint64_t* __restrict__ total_halfs, int B)
-{
-    heads_scan(head_tot, nz_off, total_halfs, B, 2, 2ull);
 }
 
 // ------------------------------------------------------------------------------- scatter
@@ -201,7 +210,7 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 
 // ------------------------------------------------------------------------------- dense prune
 // y = x * (|x| >= kth-th smallest |x| of the row); 64 rows per wavefront.
-__global__ __launch_bounds__(64) void prune_rows_kernel(const _Float16* __restrict__ x, _Float16* y, int64_t rows,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void prune_rows_kernel(const _Float16* __restrict__ x, _Float16* y, int64_t rows,
                                                         int kth)
 {
     __shared__ uint32_t slab[kHalfSlabDw];
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(64) void prune_rows_kernel(const _Float16* __restri
 }
 
 // ------------------------------------------------------------------------------- host
-// workspace: unit totals, unit bases (both [B][M/64]), head totals [B]
+// workspace: unit totals, unit bases (both [B][M/64]) and a spare row of B words
 static size_t compress_ws_bytes(int B, int M)
 {
     return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
@@ -297,14 +306,11 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
-    uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
-                       head_tot, nblk, kD);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(scan_heads_kernel, dim3(1), dim3(1024), 0, st, head_tot, nz_off, total_halfs, B);
+                       nz_off, total_halfs, nblk, kD);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     if (nz) {
         if (!aligned_to(nz, 16)) return MSTF_EALIGN;
@@ -337,12 +343,11 @@ static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, in
     const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
-    uint32_t* head_tot = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
-                       head_tot, nblk, kD);
+                       (uint32_t*)nullptr, (uint64_t*)nullptr, nblk, kD);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bmp,
                        idx, unit_base, dst_off, reinterpret_cast<char*>(nz), ~0ull, dst_limit, overflow);

@@ -19,7 +19,7 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits) { return (flo
 // grid = B * M/64 units, 64 threads.  Lane l owns tiles l and 64+l of the unit: bitmap, raw count,
 // units, scale, zero; tile_off gets the unit-local exclusive word offset, unit_tot the unit total.
 template <bool IS_VALUE>
-__global__ __launch_bounds__(64) void quant_count_kernel(const _Float16* __restrict__ x, int M, int kth, int bit,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void quant_count_kernel(const _Float16* __restrict__ x, int M, int kth, int bit,
                                                          uint64_t* __restrict__ bmp, uint32_t* __restrict__ counts,
                                                          uint32_t* __restrict__ units, uint32_t* __restrict__ tile_off,
                                                          _Float16* __restrict__ scales, _Float16* __restrict__ zeros,
@@ -39,8 +39,7 @@ __global__ __launch_bounds__(64) void quant_count_kernel(const _Float16* __restr
         uint32_t mag[64];
 #pragma unroll
         for (int j = 0; j < 64; j++) mag[j] = r[j] & 0x7FFF7FFFu;
-        const uint32_t thr = threshold_of(mag, kth);
-        unit_bitmaps<IS_VALUE>(mag, thr, lane, bm[0], bm[1]);
+        unit_keep<IS_VALUE>(mag, kth, lane, bm[0], bm[1]);
     }
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
     const int cap = 32 / bit;
