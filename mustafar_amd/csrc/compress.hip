@@ -82,9 +82,17 @@ __global__ __launch_bounds__(256) void scan_units_kernel(const uint32_t* __restr
     if (nz_off) {
         uint64_t mine = 0;
         const size_t before = (size_t)b * nblk;
-        // the loads of a pass are independent: unrolled, eight of them are in flight at a time
-#pragma unroll 8
-        for (size_t i = tid; i < before; i += 256) mine += unit_tot[i];
+        // 16-byte loads, four of them in flight per thread (unit_tot is 256-byte aligned)
+        const uint4* ut4 = reinterpret_cast<const uint4*>(unit_tot);
+        const size_t n4 = before / 4;
+        for (size_t i = tid; i < n4; i += 1024) {
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = i + 256 * u < n4 ? ut4[i + 256 * u] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+            for (int u = 0; u < 4; u++) mine += (uint64_t)v[u].x + v[u].y + v[u].z + v[u].w;
+        }
+        if (tid < (int)(before - 4 * n4)) mine += unit_tot[4 * n4 + tid];
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
         if ((tid & 63) == 0) wsum[tid >> 6] = mine;

@@ -123,20 +123,22 @@ __device__ __forceinline__ Batch prefetch_batch(const uint64_t* bm, const uint32
 }
 
 // One staged sub-chunk (kSubTiles tiles).
+//   cur    : bitmaps and offsets of its first 8 tiles, already requested; on return those of the first 8 tiles at
+//            (bm_next, ix_next) - the coming sub-chunk - so that the chain of scalar requests, each one batch ahead,
+//            runs across sub-chunks
 //   bm, ix : the sub-chunk's bitmaps and tile offsets (wave-uniform pointers)
 //   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
 //   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
 template <int NM>
-__device__ __forceinline__ void sub_accumulate(const uint64_t* bm, const uint32_t* ix, uint32_t buf, uint32_t zaddr,
-                                               uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
+__device__ __forceinline__ void sub_accumulate(Batch& cur, const uint64_t* bm, const uint32_t* ix,
+                                               const uint64_t* bm_next, const uint32_t* ix_next, uint32_t buf,
+                                               uint32_t zaddr, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
 {
     constexpr int G = kSubTiles / 8;
-    Batch cur = load_batch(bm, ix);
     const uint32_t rel = buf - cur.ov[0] * 4u;
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        Batch nxt = cur;
-        if (g + 1 < G) nxt = prefetch_batch(bm + 8 * (g + 1), ix + 8 * (g + 1));
+        const Batch nxt = g + 1 < G ? prefetch_batch(bm + 8 * (g + 1), ix + 8 * (g + 1)) : prefetch_batch(bm_next, ix_next);
         batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
         cur = nxt;
     }
@@ -192,8 +194,13 @@ __device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stag
     Touch touch = touch_sub(bmk + t_cur, ixk + t_cur, lane);
     size_t t_nxt = nsubs > 1 ? tile_of(1) : t_cur;
     uint32_t s_nxt = ixk[t_nxt], e_nxt = ixk[t_nxt + kSubTiles];
+    Batch cur = load_batch(bmk + t_cur, ixk + t_cur);
     for (int n = 0; n < nsubs; n++) {
         wait_vm0_keep(touch);  // sub-chunk n (values, weights) has landed
+        // Buffer (n+1)&1 is refilled now.  Its last reader was sub-chunk n-1, and every LDS read of that sub-chunk
+        // fed an MFMA issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would
+        // also drain the scalar request for the coming batch and expose its round trip at every sub-chunk.)
+        __builtin_amdgcn_sched_barrier(0);
         if (n + 1 < nsubs) {
             sub_issue(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), my + ((n + 1) & 1) * kSubBytes, lane);
             stage_w(n + 1);
@@ -206,10 +213,11 @@ __device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stag
             s_nxt = ixk[t_nxt];
             e_nxt = ixk[t_nxt + kSubTiles];
         }
-        sub_accumulate<NM>(bmk + t_now, ixk + t_now, lbase + (uint32_t)(n & 1) * kSubBytes, zaddr, waddr_of(n), wgroup,
-                           acc);
-        wait_lgkm0();  // all LDS reads of buffer n&1 are done before it is refilled
+        sub_accumulate<NM>(cur, bmk + t_now, ixk + t_now, bmk + t_cur, ixk + t_cur, lbase + (uint32_t)(n & 1) * kSubBytes,
+                           zaddr, waddr_of(n), wgroup, acc);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    wait_lgkm0();
 }
 
 }  // namespace mstf
