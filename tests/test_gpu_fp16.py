@@ -250,3 +250,31 @@ def test_c_abi_rejects_bad_arguments():
                                    tot.data_ptr(), None, 0, None, 0) == -4
     assert b"workspace" in L.mstf_strerror(-4)
     torch.cuda.synchronize()
+
+
+def test_config0_shape_against_oracle():
+    """The reference's CPU-runnable case: batch 1, 32 heads (MHA), head_dim 128, 4096 tokens, K with 4 outlier
+    channels per head, 70 % pruning on K and V, one query token.  Formats bit-exact against the oracle at the full
+    size; raw scores, probabilities and attention output against its dense masked attention."""
+    from mustafar_amd import ops
+    heads, L, D, groups = 32, 4096, 128, 1
+    kth = orc.kth_from_sparsity(0.7, D)
+    K, V = orc.make_kv(0, heads, L, D)
+    q = np.random.default_rng(1).standard_normal((heads, D)).astype(np.float16)
+    Kp, Vp = orc.prune_rows(K, kth), orc.prune_rows(V, kth)
+    s_ref, p_ref, o_ref = orc.dense_masked_attention(q, Kp, Vp, groups)
+    ck = ops.compress(to_gpu(K), False, kth=kth)
+    cv = ops.compress(to_gpu(V), True, kth=kth)
+    for c, xp, is_value in ((ck, Kp, 0), (cv, Vp, 1)):
+        rb, ri, rnz, roff = orc.compress(xp, is_value)
+        assert np.array_equal(c.bmp.cpu().numpy(), rb) and np.array_equal(c.idx.cpu().numpy(), ri)
+        assert np.array_equal(c.nz_off.cpu().numpy(), roff)
+        assert np.array_equal(c.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+    qg = to_gpu(q)
+    s = ops.key_spmv(ck, qg.view(heads, 1, D), groups)
+    assert rel_rowmax(s.cpu().numpy()[:, 0], s_ref) < RTOL
+    p = ops.scale_softmax(s, D)
+    assert rel_rowmax(p.cpu().numpy()[:, 0], p_ref) < RTOL
+    o = ops.value_spmv(cv, p, groups)
+    assert rel_rowmax(o.cpu().numpy()[:, 0], o_ref) < RTOL
+    assert rel_rowmax(ops.decode_attention(ck, cv, qg, groups).cpu().numpy(), o_ref) < RTOL
