@@ -135,6 +135,21 @@ def main():
             ops.compress(K, False, kth=kth, capacity_halfs=cap)  # warm-up (module load)
         t_ck += event_time_us(torch, lambda: caches.append([ops.compress(K, False, kth=kth, capacity_halfs=cap)]), 1)
         t_cv += event_time_us(torch, lambda: caches[-1].append(ops.compress(V, True, kth=kth, capacity_halfs=cap)), 1)
+        if i == args.caches - 1:
+            # GPU time of the compressors without the launch gaps of the Python calls: one capture, replayed
+            try:
+                def graphed_us(x, is_value):
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        keep = ops.compress(x, is_value, kth=kth, capacity_halfs=cap)
+                    g.replay()
+                    t = event_time_us(torch, g.replay, 5)
+                    del keep
+                    return t
+                tg_ck, tg_cv = graphed_us(K, False), graphed_us(V, True)
+            except Exception as e:  # pragma: no cover - reported as null in the JSON line
+                print("compress graph capture failed (%s)" % e, file=sys.stderr)
+                tg_ck = tg_cv = None
         if not args.no_dense:
             dense.append((K.view(bs, nkv, L, D), V.view(bs, nkv, L, D)))
         del K, V
@@ -355,6 +370,15 @@ def main():
         "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
                       "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
+        # the compressors alone (configs[2] reports them): GPU time from a replayed capture, bytes read (dense fp16
+        # context) and written (bitmaps + offsets + packed values), and the resulting rate
+        "compress": {
+            "key": {"us": None if tg_ck is None else round(tg_ck, 1), "read_bytes": int(Bkv * L * D * 2),
+                    "written_bytes": int(kbytes),
+                    "gbs": None if tg_ck is None else round((Bkv * L * D * 2 + kbytes) / tg_ck / 1e3, 1)},
+            "value": {"us": None if tg_cv is None else round(tg_cv, 1), "read_bytes": int(Bkv * L * D * 2),
+                      "written_bytes": int(vbytes),
+                      "gbs": None if tg_cv is None else round((Bkv * L * D * 2 + vbytes) / tg_cv / 1e3, 1)}},
         "quant_stages_us": quant_us,
         "dense_fp16_attention_us": dense_us,
         "hbm_gbs_on_compressed_bytes": {"fused_decode_attention": round(fused_alg / fused_us / 1e3, 1),
