@@ -116,6 +116,47 @@ __global__ __launch_bounds__(256) void finalize_idx_kernel(uint32_t* __restrict_
     if (t < T) idx[(size_t)b * (T + 1) + t] += unit_base[(size_t)b * nblk + t / tiles_per_unit];
 }
 
+// Compacts half a unit (64 tiles) into the LDS image at `img` and streams it to dst.
+//   v      : this lane's token, channels 64h .. 64h+63 (raw fp16 pairs)
+//   bm_l   : bitmap of tile 64h + lane;  ix_l: its final offset (4-byte units);  s_h: offset of the half's first tile
+//   bytes  : packed size of the half;  dump: LDS address that takes the writes of the lanes that keep nothing
+template <bool IS_VALUE>
+__device__ __forceinline__ void scatter_half(const uint32_t (&v)[32], uint64_t bm_l, uint32_t ix_l, uint32_t s_h,
+                                             uint32_t bytes, uint32_t img, uint32_t dump, char* dst, int lane)
+{
+    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+        *(MSTF_LDS u32x4_t*)(uintptr_t)(img + o) = u32x4_t{0u, 0u, 0u, 0u};  // the padding stays +0.0
+    if (!IS_VALUE) {
+        // tile c = channel 64h + c over the 64 tokens: lane = token writes its element at the tile's rank
+#pragma unroll
+        for (int c = 0; c < 64; c++) {
+            const uint64_t m = lanes_of(u64_of(__builtin_amdgcn_readlane((uint32_t)bm_l, c),
+                                               __builtin_amdgcn_readlane((uint32_t)(bm_l >> 32), c)));
+            const uint32_t off = img + (__builtin_amdgcn_readlane(ix_l, c) - s_h) * 4u;
+            const uint32_t a = select_lane(m, rank_below(m) * 2u + off, dump);
+            const uint32_t w = v[c >> 1];
+            *(MSTF_LDS uint16_t*)(uintptr_t)a = (uint16_t)((c & 1) ? (w >> 16) : w);
+        }
+    } else {
+        // tile (h, token = lane): the lane walks its own 64 channels, MSB of the bitmap first
+        uint32_t a = img + (ix_l - s_h) * 4u;
+        const uint32_t hi = (uint32_t)(bm_l >> 32), lo = (uint32_t)bm_l;
+#pragma unroll
+        for (int i = 0; i < 64; i++) {
+            const uint32_t word = i < 32 ? hi : lo;
+            const int32_t keep = (int32_t)(word << (i & 31)) >> 31;  // -1 when channel i is kept
+            const uint32_t w = v[i >> 1];
+            *(MSTF_LDS uint16_t*)(uintptr_t)((a & (uint32_t)keep) | (dump & ~(uint32_t)keep)) =
+                (uint16_t)((i & 1) ? (w >> 16) : w);
+            a -= 2 * keep;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+        *reinterpret_cast<u32x4_t*>(dst + o) = *(MSTF_LDS const u32x4_t*)(uintptr_t)(img + o);
+    __builtin_amdgcn_wave_barrier();
+}
+
 // ------------------------------------------------------------------------------- scatter
 // grid = B * M/64 units, 64 threads.  bmp and nz_off are final; idx is final (ADD_BASE false) or still holds
 // the unit-local offsets of the count kernel, which are completed here with unit_base (ADD_BASE true).
@@ -179,39 +220,8 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
         __builtin_amdgcn_wave_barrier();
         row_of_lane(buf, lane, v, 0);
         __builtin_amdgcn_wave_barrier();
-        for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
-            *(MSTF_LDS u32x4_t*)(uintptr_t)(img + o) = u32x4_t{0u, 0u, 0u, 0u};  // the padding stays +0.0
-        const uint64_t bm_l = h == 0 ? bmA : bmB;
-        const uint32_t ix_l = h == 0 ? iA : iB;
-        if (!IS_VALUE) {
-            // tile c = channel 64h + c over the 64 tokens: lane = token writes its element at the tile's rank
-#pragma unroll
-            for (int c = 0; c < 64; c++) {
-                const uint64_t m = lanes_of(u64_of(__builtin_amdgcn_readlane((uint32_t)bm_l, c),
-                                                   __builtin_amdgcn_readlane((uint32_t)(bm_l >> 32), c)));
-                const uint32_t off = img + (__builtin_amdgcn_readlane(ix_l, c) - s_h) * 4u;
-                const uint32_t a = select_lane(m, rank_below(m) * 2u + off, dump);
-                const uint32_t w = v[c >> 1];
-                *(MSTF_LDS uint16_t*)(uintptr_t)a = (uint16_t)((c & 1) ? (w >> 16) : w);
-            }
-        } else {
-            // tile (h, token = lane): the lane walks its own 64 channels, MSB of the bitmap first
-            uint32_t a = img + (ix_l - s_h) * 4u;
-            const uint32_t hi = (uint32_t)(bm_l >> 32), lo = (uint32_t)bm_l;
-#pragma unroll
-            for (int i = 0; i < 64; i++) {
-                const uint32_t word = i < 32 ? hi : lo;
-                const int32_t keep = (int32_t)(word << (i & 31)) >> 31;  // -1 when channel i is kept
-                const uint32_t w = v[i >> 1];
-                *(MSTF_LDS uint16_t*)(uintptr_t)((a & (uint32_t)keep) | (dump & ~(uint32_t)keep)) =
-                    (uint16_t)((i & 1) ? (w >> 16) : w);
-                a -= 2 * keep;
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        char* dst = nz + (head_half0 + 2ull * s_h) * 2ull;
-        for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
-            *reinterpret_cast<u32x4_t*>(dst + o) = *(MSTF_LDS const u32x4_t*)(uintptr_t)(img + o);
+        scatter_half<IS_VALUE>(v, h == 0 ? bmA : bmB, h == 0 ? iA : iB, s_h, bytes, img, dump,
+                               nz + (head_half0 + 2ull * s_h) * 2ull, lane);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -311,10 +321,10 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     if (!aligned_to(ws, 256)) return MSTF_EALIGN;
     hipStream_t st = as_stream(stream);
     const int nblk = M / 64;
+    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
-    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
