@@ -38,15 +38,27 @@ __device__ __forceinline__ void dma4(const void* src, void* dst_wave_uniform)
 }
 
 // Streams `bytes` (a multiple of 16, <= kSubBytes) into LDS: piece i of lane l lands at dst + (i*64 + l)*16.
+// The lane's source address is formed once; the 1 KB pieces differ only in the instruction's immediate offset
+// (which moves the global and the LDS address alike).  Whole pieces need no lane predicate, only the last,
+// partial one does - so a sub-chunk costs two or three vector instructions besides the loads themselves.
 __device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char* dst, int lane)
 {
-#pragma unroll
-    for (int i = 0; i < kSubBytes / 1024; i++) {
-        if ((uint32_t)(i * 1024) < bytes) {
-            const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
-            if (o < bytes) dma16(src + o, dst + i * 1024);
-        }
+    const char* mine = src + (uint32_t)lane * 16u;
+    const uint32_t whole = bytes >> 10, rest = bytes & 1023u;  // wave-uniform
+#define MSTF_PIECE(I)                                                                                              \
+    if ((uint32_t)(I) < whole) {                                                                                   \
+        __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)mine, (MSTF_LDS void*)dst, 16, (I) * 1024, 0);  \
+    } else if ((uint32_t)(I) == whole && (uint32_t)lane * 16u < rest) {                                            \
+        __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)mine, (MSTF_LDS void*)dst, 16, (I) * 1024, 0);  \
     }
+    static_assert(kSubBytes / 1024 == 4 || kSubBytes / 1024 == 2, "pieces per sub-chunk");
+    MSTF_PIECE(0)
+    MSTF_PIECE(1)
+    if (kSubBytes / 1024 == 4) {
+        MSTF_PIECE(2)
+        MSTF_PIECE(3)
+    }
+#undef MSTF_PIECE
 }
 
 // LDS byte address of D[t][lane] for one tile (the zero slot when the lane's element is absent).
