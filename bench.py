@@ -60,7 +60,7 @@ def event_time_us(torch, fn, iters):
 
 def cpu_baseline(args, bs, nkv, groups, L, D, kth):
     """The oracle's dense masked attention (prune -> q.K^T -> /sqrt(d) -> fp32 softmax -> P.V) on the
-    host cores, on a bounded sample: the full layer shape at a reduced batch."""
+    host cores, on a bounded sample: the layer shape at up to --cpu-batch batch entries, repeated for about 10 s."""
     import numpy as np
     from oracle import oracle as orc
     sample_bs = max(1, min(bs, args.cpu_batch))
@@ -72,7 +72,7 @@ def cpu_baseline(args, bs, nkv, groups, L, D, kth):
     t_prune = time.perf_counter() - t0
     orc.dense_masked_attention(q, Kp, Vp, groups)  # warm-up
     reps, t_att = 0, 0.0
-    while reps < 3 or (t_att < 10.0 and reps < 50):
+    while reps < 3 or (t_att < 10.0 and reps < 1000):
         t0 = time.perf_counter()
         orc.dense_masked_attention(q, Kp, Vp, groups)
         t_att += time.perf_counter() - t0
@@ -98,7 +98,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--caches", type=int, default=6, help="distinct compressed caches rotated between steps")
-    ap.add_argument("--cpu-batch", type=int, default=2, help="batch entries in the CPU-baseline sample")
+    ap.add_argument("--cpu-batch", type=int, default=8, help="batch entries in the CPU-baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
     ap.add_argument("--unfused", action="store_true", help="step = the three separate operator launches")
