@@ -66,3 +66,38 @@ def test_random_case(seed):
     scale = max(np.abs(o_ref.astype(np.float64)).max(), 1e-30)
     assert np.abs(o.cpu().numpy().astype(np.float64) - o_ref).max() < 2e-3 * scale
     assert np.abs(o3.cpu().numpy()[:, 0].astype(np.float64) - o_ref).max() < 2e-3 * scale
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_case_quantised(seed):
+    """The quantised producer bit-exact against the oracle, and the one-launch quantised attention against dense
+    masked attention on the oracle's dequantised cache (1e-2), on the same kind of drawn inputs."""
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    rng = np.random.default_rng(9500 + seed)
+    bit = int(rng.choice([2, 4, 8]))
+    mode = int(rng.integers(0, 2))
+    groups = int(rng.choice([1, 2, 4, 7, 8]))
+    Bkv = int(rng.integers(1, 4))
+    M = 64 * int(rng.integers(1, 9))
+    kth = int(rng.choice([38, 64, 89, 115]))
+    Kp = orc.prune_rows(draw(rng, Bkv, M, seed % 5), kth)
+    Vp = orc.prune_rows(draw(rng, Bkv, M, (seed + 2) % 5), kth)
+    kq = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
+    vq = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    for got, xp, is_value in ((kq, Kp, 0), (vq, Vp, 1)):
+        for g, r in zip(got, orc.compress_quant(xp, is_value, bit)):
+            g = g.cpu().numpy()
+            if g.dtype == np.float16:
+                assert np.array_equal(g.view(np.uint16), r.view(np.uint16))
+            else:
+                assert np.array_equal(g, r)
+    kr = [t.cpu().numpy() for t in kq]
+    vr = [t.cpu().numpy() for t in vq]
+    Kd = np.stack([orc.decode_quant(kr[0], kr[2], kr[1], kr[5], kr[6], b, M, D, 0, bit, mode) for b in range(Bkv)])
+    Vd = np.stack([orc.decode_quant(vr[0], vr[2], vr[1], vr[5], vr[6], b, M, D, 1, bit, mode) for b in range(Bkv)])
+    q = rng.standard_normal((Bkv * groups, D)).astype(np.float16)
+    _, _, o_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
+    o = mpq.decode_attention_quant(kq, vq, to_gpu(q), groups, bit, dequant_mode=mode)
+    scale = max(np.abs(o_ref.astype(np.float64)).max(), 1e-30)
+    assert np.abs(o.cpu().numpy().astype(np.float64) - o_ref).max() < 1e-2 * scale
