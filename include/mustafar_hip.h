@@ -194,8 +194,10 @@ int mstf_compress_value_quant(void* stream, const mstf_half* x, int B, int M, in
  * matrix (q - zero) * scale; dequant_mode 0 = fp32 arithmetic rounded once to fp16, 1 = fp16
  * arithmetic (SpMM_Kernel_Quant.cuh:190-191,238-240).  counts/units may be NULL (derived from the
  * bitmaps, as the non-_meta key entry point does).  bit in {2, 4, 8}; capacity must equal 32 / bit.
- * tile_off must be the running sum of the tiles' word counts (what the producer writes), scales and zeros
- * 4-byte aligned, head_dim 64 or 128. */
+ * The words of the 128 tiles of one side of a 64-token block must be contiguous in `packed`, in tile order (what
+ * the producer writes); blocks may lie anywhere, so a cache grown the reference's way - a chunk's words appended
+ * behind the old ones, its offsets shifted (models/llama_mustafar_quant_kernel.py:322-345) - is read as it is.
+ * scales and zeros 4-byte aligned, head_dim 64 or 128. */
 int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
                         const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
                         const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq, int groups,

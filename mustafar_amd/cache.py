@@ -260,3 +260,105 @@ class SparseKVCache:
             self.v_win = self.v_win[:, :, CHUNK:].contiguous()
             self.compressed_length += CHUNK
         return out
+
+
+class QuantSparseKVCache:
+    """The quantised caller's state machine (models/llama_mustafar_quant_kernel.py:305-345, 425-575): prefill split,
+    a dense local window, 256-token chunks pruned + quantised + appended, decode over [compressed | window].
+
+    The compressed sides are the reference's 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales,
+    zeros]; a chunk is appended as the reference does it (:322-345): its packed words go behind the existing ones
+    and its tile offsets are shifted by the old size, the per-tile arrays are concatenated along the tile axis.  A
+    head's tiles are then no longer contiguous across chunks, which the consumers allow: they only rely on the
+    words of one 64-token block being contiguous.
+
+    fused: the compressed part of a step is one launch (decode_attention_quant) whose (max, sum) joins the dense
+    window under one softmax; otherwise the reference's key formulation -> softmax -> value formulation sequence."""
+
+    def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, bit=2,
+                 dequant_mode=0, fused=False):
+        self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
+        self.bit, self.dequant_mode, self.fused = bit, dequant_mode, fused
+        self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
+        self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
+        self.k = self.v = None          # 7-element lists
+        self.k_win = self.v_win = None  # [bs, n_kv, Lw, D] dense
+        self.compressed_length = 0
+        self.kv_len = 0
+
+    def _compress(self, K, V):
+        from . import compression_quant as cq
+        bs, n_kv, M, D = K.shape
+        Kp = ops.prune_rows(K.reshape(-1, D).contiguous(), self.kth_k).view(bs * n_kv, M, D)
+        Vp = ops.prune_rows(V.reshape(-1, D).contiguous(), self.kth_v).view(bs * n_kv, M, D)
+        return (list(cq.convert_key_batched_quant(Kp, return_metadata=True, bit=self.bit)),
+                list(cq.convert_value_batched_quant(Vp, bit=self.bit)))
+
+    @staticmethod
+    def _append(old, new):
+        """models/llama_mustafar_quant_kernel.py:322-345."""
+        shifted = new[1] + old[2].numel()
+        return [torch.cat([old[0], new[0]], 1), torch.cat([old[1], shifted], 1), torch.cat([old[2], new[2]], 0),
+                torch.cat([old[3], new[3]], 1), torch.cat([old[4], new[4]], 1), torch.cat([old[5], new[5]], 1),
+                torch.cat([old[6], new[6]], 1)]
+
+    def _grow(self, K, V):
+        ck, cv = self._compress(K, V)
+        self.k = ck if self.k is None else self._append(self.k, ck)
+        self.v = cv if self.v is None else self._append(self.v, cv)
+
+    def prefill(self, K, V):
+        """K, V: [bs, n_kv, L, D] fp16 (after RoPE)."""
+        L = K.shape[2]
+        Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
+        if Lc > 0:
+            self._grow(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
+        self.compressed_length, self.kv_len = Lc, L
+        self.k_win = K[:, :, Lc:].contiguous().clone()
+        self.v_win = V[:, :, Lc:].contiguous().clone()
+
+    def decode(self, q, k_new, v_new):
+        """q: [bs, n_q, 1, D]; k_new, v_new: [bs, n_kv, 1, D].  Returns the attention output [bs, n_q, 1, D]."""
+        from . import mustafar_package_quant as mpq
+        bs, n_q, _, D = q.shape
+        g, Lc, cap = self.groups, self.compressed_length, 32 // self.bit
+        Bq = bs * n_q
+        self.kv_len += 1
+        self.k_win = torch.cat([self.k_win, k_new], dim=2)
+        self.v_win = torch.cat([self.v_win, v_new], dim=2)
+        s_loc = torch.matmul(q, _repeat_kv(self.k_win, g).transpose(2, 3))            # [bs, n_q, 1, Lw]
+        if Lc > 0 and self.fused:
+            lse = torch.empty((Bq, 2), dtype=torch.float32, device=q.device)
+            o_c = mpq.decode_attention_quant(self.k, self.v, q.reshape(Bq, D).contiguous(), g, self.bit,
+                                             self.dequant_mode, lse=lse)
+            m_c, l_c = lse[:, 0].view(bs, n_q, 1, 1), lse[:, 1].view(bs, n_q, 1, 1)
+            w = (s_loc / ops.sqrt_head_dim(D)).float()
+            M = torch.maximum(m_c, w.amax(-1, keepdim=True))
+            p = torch.exp(w - M)
+            a = l_c * torch.exp(m_c - M)
+            num = a * o_c.view(bs, n_q, 1, D).float() + torch.matmul(p, _repeat_kv(self.v_win, g).float())
+            out = (num / (a + p.sum(-1, keepdim=True))).half()
+        else:
+            if Lc > 0:
+                k = self.k
+                padded_query = torch.nn.functional.pad(q.view(Bq, -1, D), (0, 0, 0, 7))
+                s_cmp = mpq.mustafar_key_formulation_quant_meta(k[0], k[2], k[1], k[3], k[4], k[5], k[6], padded_query, Lc,
+                                                                D, Bq, g, self.bit, cap, self.dequant_mode)
+                s = torch.cat([s_cmp[:, 0:1, :].view(bs, n_q, 1, Lc), s_loc], dim=-1)
+            else:
+                s = s_loc
+            p = ops.scale_softmax(s.contiguous(), D)
+            out = torch.matmul(p[..., Lc:], _repeat_kv(self.v_win, g))
+            if Lc > 0:
+                v = self.v
+                score = p[..., :Lc].reshape(Bq, Lc).contiguous()
+                o_cmp = mpq.mustafar_value_formulation_quant_decode_n1(v[0], v[2], v[1], v[3], v[4], v[5], v[6], score,
+                                                                       None, D, Lc, Bq, g, self.bit, cap,
+                                                                       self.dequant_mode)
+                out = out + o_cmp.view(bs, n_q, 1, D)
+        if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.k_win.shape[2] >= CHUNK:
+            self._grow(self.k_win[:, :, :CHUNK].contiguous(), self.v_win[:, :, :CHUNK].contiguous())
+            self.k_win = self.k_win[:, :, CHUNK:].contiguous()
+            self.v_win = self.v_win[:, :, CHUNK:].contiguous()
+            self.compressed_length += CHUNK
+        return out

@@ -106,3 +106,58 @@ def test_short_prompt_stays_dense_until_first_chunk(window_kernel):
         out = cache.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
     assert cache.compressed_length == 256 and cache.kv_len == 300   # 288 - 32 - 0 == 256 triggers the first chunk
     assert torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("fused,bit", [(False, 2), (True, 2), (True, 4)])
+def test_quantised_cache_prefill_decode_append(fused, bit):
+    """The quantised caller's state machine: after the prefill and two chunk appends (the reference's append: words
+    behind the old ones, offsets shifted) every checked decode step matches dense masked attention over
+    [oracle-dequantised compressed part | dense window] within 1e-2, and the per-tile arrays equal a one-shot
+    quantisation of the same tokens."""
+    from mustafar_amd.cache import QuantSparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D, res = 1, 2, 4, 128, 64
+    L0, steps = 400, 300                       # prefill: Lc = 256, window 144; appends at kv_len 576 and 832?
+    total = L0 + steps
+    K, V = orc.make_kv(123, bs * n_kv, total, D)
+    rng = np.random.default_rng(2)
+    Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
+    cache = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=fused)
+    cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
+    assert cache.compressed_length == 256
+
+    def dequantised(src, Lc, is_value):
+        xp = orc.prune_rows(np.ascontiguousarray(src[:, :Lc]), 89)
+        b, off, packed, _, _, sc, zp = orc.compress_quant(xp, is_value, bit)
+        return np.stack([orc.decode_quant(b, packed, off, sc, zp, h, Lc, D, is_value, bit, 0) for h in range(bs * n_kv)])
+
+    checked = 0
+    for t in range(steps):
+        pos = L0 + t
+        Lc_before = cache.compressed_length
+        q = torch.from_numpy(Q[t]).to(dev).view(bs, n_kv * g, 1, D)
+        out = cache.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
+        if t % 53 == 0 or cache.compressed_length != Lc_before or t == steps - 1:
+            Kf, Vf = K[:, :pos + 1].copy(), V[:, :pos + 1].copy()
+            Kf[:, :Lc_before] = dequantised(K, Lc_before, 0)
+            Vf[:, :Lc_before] = dequantised(V, Lc_before, 1)
+            _, _, ref = orc.dense_masked_attention(Q[t], Kf, Vf, g)
+            assert rel_rowmax(out.cpu().numpy().reshape(-1, D), ref) < 1e-2, (t, pos)
+            checked += 1
+    assert cache.compressed_length == 512 and cache.kv_len == total and checked >= 6
+    # per-tile arrays equal a one-shot quantisation; the packed words are the same words, chunk by chunk
+    Lc = cache.compressed_length
+    for side, src, is_value in ((cache.k, K, 0), (cache.v, V, 1)):
+        ref = orc.compress_quant(orc.prune_rows(np.ascontiguousarray(src[:, :Lc]), 89), is_value, bit)
+        for i in (0, 3, 4):
+            assert np.array_equal(side[i].cpu().numpy(), ref[i])
+        for i in (5, 6):
+            assert np.array_equal(side[i].cpu().numpy().view(np.uint16), ref[i].view(np.uint16))
+        got_off, got_words = side[1].cpu().numpy(), side[2].cpu().numpy()
+        units = ref[4]
+        for h in range(bs * n_kv):
+            for t in (0, 17, units.shape[1] // 2 + 3, units.shape[1] - 1):
+                n = int(units[h, t])
+                assert np.array_equal(got_words[got_off[h, t]:got_off[h, t] + n], ref[2][ref[1][h, t]:ref[1][h, t] + n])
