@@ -5,7 +5,8 @@ greedy decode, reporting tokens/s and the share of the step spent in attention o
 
 The model is only the carrier of the measurement: weights are N(0, 0.02) and nothing is loaded from disk.
 `cache="sparse"` uses SparseKVCache (compressed tokens and window in three launches, pooled storage);
-`cache="dense_masked"` keeps the pruned tokens
+`cache="sparse_quant2"` / `"sparse_quant4"` use QuantSparseKVCache (pruned + 2- or 4-bit codes, one fused launch over the
+compressed tokens, window through torch operators); `cache="dense_masked"` keeps the pruned tokens
 dense and attends with torch ops - the reference's own dense path (models/llama_mustafar_Kt_Mag_Vt_Mag.py:836-1026) -
 and is what the sparse run is compared against.
 
@@ -20,7 +21,7 @@ import torch
 import torch.nn.functional as F
 
 from . import ops
-from .cache import CHUNK, SparseKVCache, _repeat_kv
+from .cache import CHUNK, QuantSparseKVCache, SparseKVCache, _repeat_kv
 
 
 class Config:
@@ -115,6 +116,9 @@ class Decoder:
         if cache == "sparse":
             self.caches = [SparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length, fused=True,
                                          max_tokens=max_tokens, window_kernel=True) for _ in range(c.layers)]
+        elif cache in ("sparse_quant2", "sparse_quant4"):
+            self.caches = [QuantSparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length,
+                                              bit=int(cache[-1]), fused=True) for _ in range(c.layers)]
         else:
             self.caches = [DenseMaskedCache(groups, c.head_dim, sparsity, sparsity, residual_length)
                            for _ in range(c.layers)]
@@ -260,7 +264,7 @@ def main():
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--sparsity", type=float, default=0.7)
     ap.add_argument("--residual", type=int, default=256)
-    ap.add_argument("--cache", default="sparse", choices=["sparse", "dense_masked"])
+    ap.add_argument("--cache", default="sparse", choices=["sparse", "sparse_quant2", "sparse_quant4", "dense_masked"])
     ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph (sparse cache only)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
