@@ -216,6 +216,18 @@ int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint3
                                 const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out, int tokens,
                                 int head_dim, int Bq, int groups, int bit, int capacity, int dequant_mode,
                                 void* workspace, size_t workspace_bytes);
+/* mstf_decode_attention_window_f16 over a quantised cache: the whole attention of a decode step of the quantised
+ * caller (models/llama_mustafar_quant_kernel.py:437-575: key formulation | q.K_win^T, / sqrt(d), softmax, value
+ * formulation + P_win.V_win) as the quantised fused kernel, the dense-window kernel and one merge.  Window
+ * arguments, win_len_dev and the workspace size as for mstf_decode_attention_window_f16. */
+int mstf_decode_attention_window_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                       const uint32_t* k_tile_off, const mstf_half* k_scales, const mstf_half* k_zeros,
+                                       const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+                                       const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q,
+                                       const mstf_half* k_win, const mstf_half* v_win, int win_len,
+                                       const int32_t* win_len_dev, int win_stride, mstf_half* out, float* lse_out,
+                                       int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
+                                       int dequant_mode, void* workspace, size_t workspace_bytes);
 
 
 #ifdef __cplusplus

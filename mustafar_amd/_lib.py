@@ -51,6 +51,7 @@ SIGNATURES = {
     "mstf_value_spmv_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _sz]),
     "mstf_decode_attention_quant": (_i, [_vp] * 14 + [_i, _i, _i, _i, _i, _i, _i, _vp, _sz]),
+    "mstf_decode_attention_window_quant": (_i, [_vp] * 14 + [_i, _vp, _i, _vp, _vp] + [_i] * 7 + [_vp, _sz]),
 }
 
 

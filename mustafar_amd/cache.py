@@ -187,8 +187,12 @@ class SparseKVCache:
         self._vbuf.index_copy_(1, self._widx, v_new.reshape(bs * n_kv, 1, D))
         self._widx += 1
         self._wlen_dev += 1
-        return ops.decode_attention_window(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), self._kbuf, self._vbuf,
-                                           self._kbuf.shape[1], self.groups, win_len_dev=self._wlen_dev).view(bs, n_q, 1, D)
+        return self._attend_device(q.reshape(bs * n_q, D).contiguous()).view(bs, n_q, 1, D)
+
+    def _attend_device(self, q2):
+        """Attention of the query rows q2 [Bq, D] over [compressed | window buffer] (three launches)."""
+        return ops.decode_attention_window(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1], self.groups,
+                                           win_len_dev=self._wlen_dev)
 
     def advance(self):
         """Host-side bookkeeping after decode_device (or a replay of it): counts the token and, when the window holds
@@ -262,7 +266,7 @@ class SparseKVCache:
         return out
 
 
-class QuantSparseKVCache:
+class QuantSparseKVCache(SparseKVCache):
     """The quantised caller's state machine (models/llama_mustafar_quant_kernel.py:305-345, 425-575): prefill split,
     a dense local window, 256-token chunks pruned + quantised + appended, decode over [compressed | window].
 
@@ -273,18 +277,21 @@ class QuantSparseKVCache:
     words of one 64-token block being contiguous.
 
     fused: the compressed part of a step is one launch (decode_attention_quant) whose (max, sum) joins the dense
-    window under one softmax; otherwise the reference's key formulation -> softmax -> value formulation sequence."""
+    window under one softmax; otherwise the reference's key formulation -> softmax -> value formulation sequence.
+    window_kernel: as in SparseKVCache - the window in a pre-allocated buffer, the whole attention of a step as
+    decode_attention_window_quant (three launches, capturable with decode_device / advance)."""
 
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, bit=2,
-                 dequant_mode=0, fused=False):
-        self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
-        self.bit, self.dequant_mode, self.fused = bit, dequant_mode, fused
-        self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
-        self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
-        self.k = self.v = None          # 7-element lists
-        self.k_win = self.v_win = None  # [bs, n_kv, Lw, D] dense
-        self.compressed_length = 0
-        self.kv_len = 0
+                 dequant_mode=0, fused=False, window_kernel=False):
+        super().__init__(groups, head_dim, k_sparsity, v_sparsity, residual_length, fused=fused,
+                         window_kernel=window_kernel)
+        self.bit, self.dequant_mode = bit, dequant_mode
+        # self.k / self.v: 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales, zeros]
+
+    def _attend_device(self, q2):
+        from . import mustafar_package_quant as mpq
+        return mpq.decode_attention_window_quant(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1],
+                                                 self.groups, self.bit, self.dequant_mode, win_len_dev=self._wlen_dev)
 
     def _compress(self, K, V):
         from . import compression_quant as cq
@@ -307,19 +314,11 @@ class QuantSparseKVCache:
         self.k = ck if self.k is None else self._append(self.k, ck)
         self.v = cv if self.v is None else self._append(self.v, cv)
 
-    def prefill(self, K, V):
-        """K, V: [bs, n_kv, L, D] fp16 (after RoPE)."""
-        L = K.shape[2]
-        Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
-        if Lc > 0:
-            self._grow(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
-        self.compressed_length, self.kv_len = Lc, L
-        self.k_win = K[:, :, Lc:].contiguous().clone()
-        self.v_win = V[:, :, Lc:].contiguous().clone()
-
     def decode(self, q, k_new, v_new):
         """q: [bs, n_q, 1, D]; k_new, v_new: [bs, n_kv, 1, D].  Returns the attention output [bs, n_q, 1, D]."""
         from . import mustafar_package_quant as mpq
+        if self.window_kernel:
+            return self._decode_window_kernel(q, k_new, v_new)
         bs, n_q, _, D = q.shape
         g, Lc, cap = self.groups, self.compressed_length, 32 // self.bit
         Bq = bs * n_q

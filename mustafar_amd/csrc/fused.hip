@@ -538,6 +538,26 @@ int mstf::merge_splits(hipStream_t st, const void* workspace, mstf_half* out, fl
     return check_launch();
 }
 
+int mstf::window_launch(hipStream_t st, const mstf_half* k_win, const mstf_half* v_win, const mstf_half* q,
+                        void* workspace, int win_len, const int32_t* win_len_dev, int win_stride, int head_dim, int Bq,
+                        int groups, int nst, int split0)
+{
+    float* part_o = reinterpret_cast<float*>(workspace);
+    float* part_ml = part_o + (size_t)Bq * nst * head_dim;
+    const _Float16* kw = reinterpret_cast<const _Float16*>(k_win);
+    const _Float16* vw = reinterpret_cast<const _Float16*>(v_win);
+    const _Float16* qh = reinterpret_cast<const _Float16*>(q);
+    const float sq = sqrtf((float)head_dim);
+    const dim3 grid((unsigned)window_blocks(win_len), (unsigned)(Bq / groups));
+    if (groups <= 4)
+        hipLaunchKernelGGL(window_attention_kernel<1>, grid, dim3(64), 0, st, kw, vw, qh, part_o, part_ml, win_len,
+                           win_len_dev, win_stride, groups, nst, split0, sq);
+    else
+        hipLaunchKernelGGL(window_attention_kernel<2>, grid, dim3(64), 0, st, kw, vw, qh, part_o, part_ml, win_len,
+                           win_len_dev, win_stride, groups, nst, split0, sq);
+    return check_launch();
+}
+
 static int splits_of(int tokens, int Bq, int groups)
 {
     return fused_nsplit(tokens, fused_blocks_per_wave(tokens, Bq / groups));
@@ -595,7 +615,6 @@ extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, co
                                            groups);
 }
 
-static int window_blocks(int win_len) { return (win_len + 63) / 64; }
 
 extern "C" size_t mstf_decode_attention_window_workspace_bytes(int tokens, int max_window, int head_dim, int Bq,
                                                                int groups)
@@ -627,7 +646,6 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
     const int ns = tokens > 0 ? splits_of(tokens, Bq, groups) : 0, nwb = window_blocks(win_len), nst = ns + nwb;
-    const int Bkv = Bq / groups;
     int rc;
     if (tokens > 0) {
         // the compressed tokens fill split slots 0 .. ns-1 of every row
@@ -638,21 +656,8 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
                            tokens, head_dim, Bq, groups, workspace, 0, nst);
         if (rc != MSTF_OK) return rc;
     }
-    float* part_o = reinterpret_cast<float*>(workspace);
-    float* part_ml = part_o + (size_t)Bq * nst * head_dim;
-    const _Float16* kw = reinterpret_cast<const _Float16*>(k_win);
-    const _Float16* vw = reinterpret_cast<const _Float16*>(v_win);
-    const _Float16* qh = reinterpret_cast<const _Float16*>(q);
-    const float sq = sqrtf((float)head_dim);
-    const dim3 grid((unsigned)nwb, (unsigned)Bkv);
-    if (groups <= 4)
-        hipLaunchKernelGGL(window_attention_kernel<1>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
-                           win_len, win_len_dev, win_stride, groups, nst, ns, sq);
-    else
-        hipLaunchKernelGGL(window_attention_kernel<2>, grid, dim3(64), 0, as_stream(stream), kw, vw, qh, part_o, part_ml,
-                           win_len, win_len_dev, win_stride, groups, nst, ns, sq);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)Bq), dim3(128), 0, as_stream(stream), part_o, part_ml,
-                       reinterpret_cast<_Float16*>(out), lse_out, nst, head_dim);
-    return check_launch();
+    if ((rc = window_launch(as_stream(stream), k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq,
+                            groups, nst, ns)) != MSTF_OK)
+        return rc;
+    return merge_splits(as_stream(stream), workspace, out, lse_out, nst, head_dim, Bq);
 }

@@ -33,6 +33,13 @@ static inline int fused_nsplit(int tokens, int bpw = 1)
 // (defined beside the merge kernel).
 int merge_splits(hipStream_t st, const void* workspace, mstf_half* out, float* lse_out, int ns, int head_dim, int Bq);
 
+// Launches the dense-window kernel: the (max, sum, output) triples of the window's 64-token blocks go into split
+// slots split0 .. of a workspace with nst slots per query row (defined beside the kernel).
+int window_launch(hipStream_t st, const mstf_half* k_win, const mstf_half* v_win, const mstf_half* q, void* workspace,
+                  int win_len, const int32_t* win_len_dev, int win_stride, int head_dim, int Bq, int groups, int nst,
+                  int split0);
+static inline int window_blocks(int win_len) { return (win_len + 63) / 64; }
+
 __device__ __forceinline__ float wave_max_same_column(float v)
 {
     // lanes 4b+j for b = 0..15 hold column j: combine over b with xor shuffles of 4, 8, 16, 32

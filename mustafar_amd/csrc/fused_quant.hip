@@ -191,16 +191,14 @@ static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp
 
 using namespace mstf;
 
-extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
-                                           const uint32_t* k_tile_off, const mstf_half* k_scales,
-                                           const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
-                                           const uint32_t* v_tile_off, const mstf_half* v_scales,
-                                           const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out,
-                                           int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
-                                           int dequant_mode, void* workspace, size_t workspace_bytes)
+// Shared argument checks of the quantised fused entry points.
+static int quant_check(const void* k_bmp, const void* k_packed, const void* k_tile_off, const void* k_scales,
+                       const void* k_zeros, const void* v_bmp, const void* v_packed, const void* v_tile_off,
+                       const void* v_scales, const void* v_zeros, const void* q, int tokens, int head_dim, int Bq,
+                       int groups, int bit, int capacity, int dequant_mode)
 {
     if (!k_bmp || !k_packed || !k_tile_off || !k_scales || !k_zeros || !v_bmp || !v_packed || !v_tile_off || !v_scales ||
-        !v_zeros || !q || !out)
+        !v_zeros || !q)
         return MSTF_EINVAL;
     if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
     if (dequant_mode != 0 && dequant_mode != 1) return MSTF_EINVAL;
@@ -209,33 +207,99 @@ extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, 
     if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
     if (!aligned_to(k_bmp, 8) || !aligned_to(v_bmp, 8) || !aligned_to(k_packed, 4) || !aligned_to(v_packed, 4) ||
         !aligned_to(k_tile_off, 4) || !aligned_to(v_tile_off, 4) || !aligned_to(k_scales, 4) || !aligned_to(v_scales, 4) ||
-        !aligned_to(k_zeros, 4) || !aligned_to(v_zeros, 4) || !aligned_to(q, 16) || !aligned_to(out, 2) ||
-        (lse_out && !aligned_to(lse_out, 4)))
+        !aligned_to(k_zeros, 4) || !aligned_to(v_zeros, 4) || !aligned_to(q, 16))
         return MSTF_EALIGN;
-    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
-    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
-    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
-    hipStream_t st = as_stream(stream);
+    return MSTF_OK;
+}
+
+// The quantised kernel over the compressed tokens: fills split slots 0 .. fused_nsplit(tokens)-1 of a workspace
+// with nst slots per query row (or writes the final output when write_final).
+static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off,
+                        const mstf_half* k_scales, const mstf_half* k_zeros, const uint64_t* v_bmp,
+                        const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
+                        const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
+                        int groups, int bit, int dequant_mode, void* workspace, int nst, int write_final)
+{
     const int Bkv = Bq / groups, ns = fused_nsplit(tokens);
     float* part_o = reinterpret_cast<float*>(workspace);
-    float* part_ml = part_o + (size_t)Bq * ns * head_dim;
-    // with one split and no (max, sum) requested the kernel writes the final output itself
-    const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
+    float* part_ml = part_o + (size_t)Bq * nst * head_dim;
     const dim3 grid((unsigned)ns, (unsigned)Bkv);
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
     _Float16* oh = reinterpret_cast<_Float16*>(out);
     const float sq = sqrtf((float)head_dim);
-#define MSTF_FQ(NMV, BITV)                                                                                              \
-    launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, \
-                                   v_scales, v_zeros, qh, oh, part_o, part_ml, tokens, groups, ns, write_final, sq,     \
-                                   dequant_mode)
+    const uint16_t* ks = reinterpret_cast<const uint16_t*>(k_scales);
+    const uint16_t* kz = reinterpret_cast<const uint16_t*>(k_zeros);
+    const uint16_t* vs = reinterpret_cast<const uint16_t*>(v_scales);
+    const uint16_t* vz = reinterpret_cast<const uint16_t*>(v_zeros);
+#define MSTF_FQ(NMV, BITV)                                                                                             \
+    launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, ks, kz, v_bmp, v_packed, v_tile_off, vs, vz, \
+                                   qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode)
     if (groups <= 4) {
         if (bit == 2) MSTF_FQ(1, 2); else if (bit == 4) MSTF_FQ(1, 4); else MSTF_FQ(1, 8);
     } else {
         if (bit == 2) MSTF_FQ(2, 2); else if (bit == 4) MSTF_FQ(2, 4); else MSTF_FQ(2, 8);
     }
 #undef MSTF_FQ
-    int rc = check_launch();
+    return check_launch();
+}
+
+extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                           const uint32_t* k_tile_off, const mstf_half* k_scales,
+                                           const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
+                                           const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                           const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out,
+                                           int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
+                                           int dequant_mode, void* workspace, size_t workspace_bytes)
+{
+    if (!out) return MSTF_EINVAL;
+    int rc = quant_check(k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
+                         tokens, head_dim, Bq, groups, bit, capacity, dequant_mode);
+    if (rc != MSTF_OK) return rc;
+    if (!aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int ns = fused_nsplit(tokens);
+    // with one split and no (max, sum) requested the kernel writes the final output itself
+    const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
+    rc = quant_launch(st, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
+                      out, tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, ns, write_final);
     if (rc != MSTF_OK || write_final) return rc;
     return merge_splits(st, workspace, out, lse_out, ns, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_attention_window_quant(
+    void* stream, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off, const mstf_half* k_scales,
+    const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+    const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q, const mstf_half* k_win,
+    const mstf_half* v_win, int win_len, const int32_t* win_len_dev, int win_stride, mstf_half* out, float* lse_out,
+    int tokens, int head_dim, int Bq, int groups, int bit, int capacity, int dequant_mode, void* workspace,
+    size_t workspace_bytes)
+{
+    if (!q || !k_win || !v_win || !out) return MSTF_EINVAL;
+    if (tokens < 0 || win_len <= 0 || win_stride < win_len || Bq <= 0 || groups <= 0 || Bq % groups != 0)
+        return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (!aligned_to(q, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int ns = tokens > 0 ? fused_nsplit(tokens) : 0, nst = ns + window_blocks(win_len);
+    int rc;
+    if (tokens > 0) {
+        rc = quant_check(k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
+                         tokens, head_dim, Bq, groups, bit, capacity, dequant_mode);
+        if (rc != MSTF_OK) return rc;
+        rc = quant_launch(st, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales,
+                          v_zeros, q, nullptr, tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, nst, 0);
+        if (rc != MSTF_OK) return rc;
+    }
+    if ((rc = window_launch(st, k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq, groups, nst,
+                            ns)) != MSTF_OK)
+        return rc;
+    return merge_splits(st, workspace, out, lse_out, nst, head_dim, Bq);
 }

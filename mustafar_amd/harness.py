@@ -5,8 +5,8 @@ greedy decode, reporting tokens/s and the share of the step spent in attention o
 
 The model is only the carrier of the measurement: weights are N(0, 0.02) and nothing is loaded from disk.
 `cache="sparse"` uses SparseKVCache (compressed tokens and window in three launches, pooled storage);
-`cache="sparse_quant2"` / `"sparse_quant4"` use QuantSparseKVCache (pruned + 2- or 4-bit codes, one fused launch over the
-compressed tokens, window through torch operators); `cache="dense_masked"` keeps the pruned tokens
+`cache="sparse_quant2"` / `"sparse_quant4"` use QuantSparseKVCache (pruned + 2- or 4-bit codes, the same three launches
+over the quantised format); `cache="dense_masked"` keeps the pruned tokens
 dense and attends with torch ops - the reference's own dense path (models/llama_mustafar_Kt_Mag_Vt_Mag.py:836-1026) -
 and is what the sparse run is compared against.
 
@@ -118,7 +118,8 @@ class Decoder:
                                          max_tokens=max_tokens, window_kernel=True) for _ in range(c.layers)]
         elif cache in ("sparse_quant2", "sparse_quant4"):
             self.caches = [QuantSparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length,
-                                              bit=int(cache[-1]), fused=True) for _ in range(c.layers)]
+                                              bit=int(cache[-1]), fused=True, window_kernel=True)
+                           for _ in range(c.layers)]
         else:
             self.caches = [DenseMaskedCache(groups, c.head_dim, sparsity, sparsity, residual_length)
                            for _ in range(c.layers)]
@@ -283,7 +284,7 @@ def main():
     warm = min(8, args.new_tokens // 4)
     loop = None
     if args.graph:
-        assert args.cache == "sparse"
+        assert args.cache.startswith("sparse")
         loop = GraphedGreedyLoop(dec, nxt, args.prompt)
         for t in range(warm):
             loop.step()

@@ -135,6 +135,36 @@ def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, d
     return o
 
 
+def decode_attention_window_quant(key_side, value_side, q, k_win, v_win, win_len, num_key_value_groups, bit,
+                                  dequant_mode=0, out=None, lse=None, win_len_dev=None):
+    """The whole attention of a decode step over [quantised compressed tokens | dense window] in three launches
+    (ops.decode_attention_window for the quantised format).  key_side / value_side may be None while nothing is
+    compressed yet.  k_win, v_win: [Bkv, stride, 128] fp16, the first win_len tokens valid; win_len_dev: optional
+    int32 device scalar with the valid length (for replay from a captured graph)."""
+    def five(side):
+        return side if len(side) == 5 else (side[0], side[1], side[2], side[5], side[6])
+    D = q.shape[-1]
+    Bq = q.numel() // D
+    L = lib()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    if key_side is not None:
+        kb, ko, kp, ks, kz = five(key_side)
+        vb, vo, vp, vs, vz = five(value_side)
+        tokens = kb.shape[1] * 64 // D
+        ptrs = [kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), ks.data_ptr(), kz.data_ptr(), vb.data_ptr(), vp.data_ptr(),
+                vo.data_ptr(), vs.data_ptr(), vz.data_ptr()]
+    else:
+        tokens, ptrs = 0, [None] * 10
+    ws = ops.workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(tokens, int(win_len), D, Bq,
+                                                                                int(num_key_value_groups)))
+    check(L.mstf_decode_attention_window_quant(
+        torch.cuda.current_stream().cuda_stream, *ptrs, q.contiguous().data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
+        int(win_len), win_len_dev.data_ptr() if win_len_dev is not None else None, int(k_win.shape[1]), o.data_ptr(),
+        lse.data_ptr() if lse is not None else None, tokens, D, Bq, int(num_key_value_groups), int(bit), 32 // int(bit),
+        int(dequant_mode), ws.data_ptr(), ws.numel()), "mstf_decode_attention_window_quant")
+    return o
+
+
 # aliases the reference exports for its model code (pybind_quant.cpp:96-176)
 mustafar_quant_sparse_forward = mustafar_key_formulation_quant
 mustafar_quant_sparse_forward_meta = mustafar_key_formulation_quant_meta

@@ -108,8 +108,9 @@ def test_short_prompt_stays_dense_until_first_chunk(window_kernel):
     assert torch.isfinite(out).all()
 
 
-@pytest.mark.parametrize("fused,bit", [(False, 2), (True, 2), (True, 4)])
-def test_quantised_cache_prefill_decode_append(fused, bit):
+@pytest.mark.parametrize("fused,bit,window_kernel", [(False, 2, False), (True, 2, False), (True, 4, False),
+                                                     (True, 2, True), (True, 8, True)])
+def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
     """The quantised caller's state machine: after the prefill and two chunk appends (the reference's append: words
     behind the old ones, offsets shifted) every checked decode step matches dense masked attention over
     [oracle-dequantised compressed part | dense window] within 1e-2, and the per-tile arrays equal a one-shot
@@ -124,7 +125,7 @@ def test_quantised_cache_prefill_decode_append(fused, bit):
     Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
-    cache = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=fused)
+    cache = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=fused, window_kernel=window_kernel)
     cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
     assert cache.compressed_length == 256
 
