@@ -247,3 +247,38 @@ def test_quant_c_abi_rejects_bad_arguments():
     assert L.mstf_key_spmv_quant(None, a, a, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 2, 16, 2) == -1   # mode
     assert L.mstf_key_spmv_quant(None, a, None, a, None, None, a, a, a, a, 64, 128, 1, 1, 1, 2, 16, 0) == -1
     assert L.mstf_compress_key_quant(None, a, 1, 64, 128, 0, 2, a, a, a, a, a, a, a, None, 0, None, 0) == -4
+
+
+@pytest.mark.parametrize("bit,groups,Bkv,Lc,Lw", [(2, 4, 2, 512, 300), (4, 8, 1, 256, 64), (2, 1, 3, 0, 257),
+                                                  (8, 2, 2, 1024, 511)])
+def test_quant_decode_attention_with_dense_window(bit, groups, Bkv, Lc, Lw):
+    """Quantised compressed tokens and dense window under one softmax (mstf_decode_attention_window_quant) against the
+    oracle's dense masked attention over [dequantised compressed part | window]; Lc = 0 is the window alone."""
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    D = 128
+    Bq = Bkv * groups
+    K, V = orc.make_kv(700 + Lc + Lw + bit, Bkv, Lc + Lw, D)
+    q = np.random.default_rng(Lw + bit).standard_normal((Bq, D)).astype(np.float16)
+    Kf, Vf = K.copy(), V.copy()
+    kq = vq = None
+    if Lc > 0:
+        Kp = orc.prune_rows(np.ascontiguousarray(K[:, :Lc]), 89)
+        Vp = orc.prune_rows(np.ascontiguousarray(V[:, :Lc]), 89)
+        kq = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
+        vq = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+        kr = [t.cpu().numpy() for t in kq]
+        vr = [t.cpu().numpy() for t in vq]
+        Kf[:, :Lc] = np.stack([orc.decode_quant(kr[0], kr[2], kr[1], kr[5], kr[6], b, Lc, D, 0, bit) for b in range(Bkv)])
+        Vf[:, :Lc] = np.stack([orc.decode_quant(vr[0], vr[2], vr[1], vr[5], vr[6], b, Lc, D, 1, bit) for b in range(Bkv)])
+    _, _, out_ref = orc.dense_masked_attention(q, Kf, Vf, groups)
+    cap = Lw + 21
+    kw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev())
+    vw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev())
+    kw[:, :Lw] = to_gpu(K[:, Lc:])
+    vw[:, :Lw] = to_gpu(V[:, Lc:])
+    o = mpq.decode_attention_window_quant(kq, vq, to_gpu(q), kw, vw, Lw, groups, bit)
+    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
+    wl = torch.tensor([Lw], dtype=torch.int32, device=dev())
+    o_dev = mpq.decode_attention_window_quant(kq, vq, to_gpu(q), kw, vw, cap, groups, bit, win_len_dev=wl)
+    assert torch.equal(o_dev, o)
