@@ -79,3 +79,35 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_install_aliases_gives_the_reference_module_names():
+    """The import lines of the reference's model files resolve to the mirrors, with the names their pybind modules
+    export (kernel/kernel_wrapper/pybind.cpp:9-10, kernel_quant/kernel_wrapper/pybind_quant.cpp:10-176)."""
+    import importlib
+    import sys
+    import mustafar_amd
+    saved = {k: sys.modules.get(k) for k in ("mustafar_package", "mustafar_package_quant", "kernel", "kernel.compression",
+                                             "kernel_quant", "kernel_quant.compression_quant")}
+    try:
+        mustafar_amd.install_aliases()
+        mp = importlib.import_module("mustafar_package")
+        mpq = importlib.import_module("mustafar_package_quant")
+        compression = importlib.import_module("kernel.compression")
+        compression_quant = importlib.import_module("kernel_quant.compression_quant")
+        for name in ("mustafar_key_formulation", "mustafar_value_formulation"):
+            assert callable(getattr(mp, name))
+        for name in ("mustafar_key_formulation_quant", "mustafar_key_formulation_quant_meta",
+                     "mustafar_value_formulation_quant", "mustafar_value_formulation_quant_decode_n1",
+                     "mustafar_quant_sparse_forward", "mustafar_quant_sparse_forward_meta",
+                     "mustafar_quant_sparse_value_forward", "mustafar_quant_sparse_value_forward_decode_n1"):
+            assert callable(getattr(mpq, name))
+        assert callable(compression.convert_key_batched) and callable(compression.convert_value_batched)
+        assert callable(compression_quant.convert_key_batched_quant)
+        assert callable(compression_quant.convert_value_batched_quant)
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
