@@ -127,10 +127,11 @@ def test_decode_attention_full_size(data):
     assert torch.equal(o_half.float() * 2, o.float()) or rel_rowmax(o_half[:, 0] * 2, o[:, 0]) < 1e-3
 
 
-@pytest.mark.parametrize("bkv,blocks,groups", [(140, 31, 4), (150, 56, 2), (40, 112, 8), (600, 64, 1)])
+@pytest.mark.parametrize("bkv,blocks,groups", [(140, 31, 4), (150, 56, 2), (40, 112, 8), (600, 64, 1), (8, 2048, 4)])
 def test_decode_attention_many_blocks(bkv, blocks, groups):
     """More 64-token blocks than resident wavefronts: every wavefront of the fused kernel walks several blocks
-    (2, 3, 2 and 8 here, with a ragged last wavefront in the first two) and folds them before the workgroup combine."""
+    (2, 3, 2, 8 and 4 here, with a ragged last wavefront in the first two; the last case is one long context of
+    131072 tokens per head, which also takes the softmax kernel beyond the rows it keeps in registers) and folds them before the workgroup combine."""
     from mustafar_amd import ops
     from mustafar_amd._lib import lib
     dev = torch.device("cuda:0")
@@ -149,18 +150,27 @@ def test_decode_attention_many_blocks(bkv, blocks, groups):
     cv = ops.compress(V, True, kth=KTH)
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
     o = ops.decode_attention(ck, cv, q, groups, lse=lse)
-    assert rel_rowmax(o, o_ref) < 2e-3
+    # Beyond ~32K tokens the reference formula rounds its probabilities into the fp16 subnormals and loses accuracy
+    # of its own; the fused kernel keeps un-normalised weights (<= 1) in fp16 and normalises in fp32.  So the fused
+    # output is held to 2e-3 against the same attention with fp32 probabilities, and to a looser bound against the
+    # reference formula for the long case; the three-launch path, which rounds as the reference does, is held to it.
     w = (s_ref / math.sqrt(D)).float()
+    Vp = torch_prune(V, KTH)
+    o_exact = torch.einsum("bgl,bld->bgd", torch.softmax(w, -1).view(bkv, groups, length), Vp.float()).half().view(-1, D)
+    assert rel_rowmax(o, o_exact) < 2e-3
+    tol_ref = 2e-3 if length <= 32768 else 4e-3
+    assert rel_rowmax(o, o_ref) < tol_ref
     m_ref = w.amax(-1)
     assert float((lse[:, 0] - m_ref).abs().max()) <= 2e-2 * max(float(m_ref.abs().max()), 1.0)
     l_ref = torch.exp(w - m_ref[:, None]).sum(-1)
     assert float((lse[:, 1] * torch.exp(lse[:, 0] - m_ref) - l_ref).abs().max()) <= 5e-3 * float(l_ref.max())
     o2 = ops.decode_attention(ck, cv, q, groups)            # route without (max, sum) output
-    assert rel_rowmax(o2, o_ref) < 2e-3
+    assert rel_rowmax(o2, o_exact) < 2e-3
     # the three-launch path on the same cache
     p = ops.scale_softmax(ops.key_spmv(ck, q.view(Bq, 1, D), groups), D)
     o3 = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o, o3[:, 0]) < 2e-3
+    assert rel_rowmax(o3[:, 0], o_ref) < 2e-3
+    assert rel_rowmax(o, o3[:, 0]) < tol_ref
 
 
 def test_compress_twice_is_idempotent(data):
