@@ -70,6 +70,21 @@ __device__ __forceinline__ uint32_t tile_addr(uint64_t b, uint32_t base, uint32_
     const uint64_t m = lanes_of(b);
     return select_lane(m, rank_below(m) * 2u + base, zaddr);
 }
+// The same with the tile's base given as idx[t] (4-byte units) and the LDS address `rel` of unit 0:
+// base = (ov << 2) + rel is one scalar instruction (s_lshl2_add_u32; the compiler emits a shift and an add), and
+// it sits in one statement with its consumers so that no hazard no-op is placed behind it.  Every instruction of
+// the per-tile sequence costs the wavefront an issue slot, scalar ones included.
+__device__ __forceinline__ uint32_t tile_addr_idx(uint64_t b, uint32_t ov, uint32_t rel, uint32_t zaddr)
+{
+    const uint64_t m = lanes_of(b);
+    const uint32_t r = rank_below(m);
+    uint32_t a, t;
+    asm("s_lshl2_add_u32 %1, %3, %4\n\tv_lshl_add_u32 %0, %2, 1, %1\n\tv_cndmask_b32 %0, %5, %0, %6"
+        : "=&v"(a), "=&s"(t)
+        : "v"(r), "s"(ov), "s"(rel), "v"(zaddr), "s"(m)
+        : "scc");
+    return a;
+}
 // (16-bit LDS loads cannot merge into one register here: with SRAM ECC they clear the other half,
 // hence the explicit pack of two tiles into one fp16x2 register.)
 __device__ __forceinline__ uint32_t pack_h2(_Float16 lo, _Float16 hi)
@@ -109,7 +124,7 @@ __device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, u
 {
     uint32_t a[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(b.mv[2 * i], b.mv[2 * i + 1]), b.ov[i] * 4u + rel, zaddr);
+    for (int i = 0; i < 8; i++) a[i] = tile_addr_idx(u64_of(b.mv[2 * i], b.mv[2 * i + 1]), b.ov[i], rel, zaddr);
     _Float16 h[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
