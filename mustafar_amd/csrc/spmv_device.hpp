@@ -122,6 +122,11 @@ template <int NM>
 __device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, uint32_t zaddr, uint32_t waddr,
                                                  uint32_t wgroup, f4_t (&acc)[NM])
 {
+    // the weights of the batch first: their LDS load then returns together with the gathers instead of costing a
+    // second round trip after them
+    u32x4_t qm[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
     uint32_t a[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) a[i] = tile_addr_idx(u64_of(b.mv[2 * i], b.mv[2 * i + 1]), b.ov[i], rel, zaddr);
@@ -132,10 +137,8 @@ __device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, u
     const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
 #pragma unroll
     for (int m = 0; m < NM; m++) {
-        const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
-        const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(qm[m][0], qm[m][1]), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(qm[m][2], qm[m][3]), acc[m], 0, 0, 0);
     }
 }
 
