@@ -91,6 +91,41 @@ int mstf_append_value_f16(void* stream, const mstf_half* x, int B, int M, int N,
                           const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow,
                           void* workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------------------------ compression from the projection output
+ * The prefill of the reference turns the projection outputs [batch, tokens, heads * 128] into [batch, heads,
+ * tokens, 128] views, rotates the keys (apply_rotary_pos_emb of transformers 4.43.1, called at
+ * models/llama_mustafar_kernel.py:373-374), prunes the first M tokens in place and copies them into a contiguous
+ * [batch * heads, M, 128] matrix for the compressor (:540-560).  These entry points read the rows where the
+ * projection left them and fuse the rotation:
+ *   source element (batch entry bt, token t, KV head h, channel c) = x[bt*stride_batch + t*stride_token +
+ *   h*stride_head + c], strides in elements and multiples of 8, `rows` tokens per head; heads are numbered
+ *   b = bt*heads + h in every output, as the reference's reshape numbers them;
+ *   cos, sin (both or neither; keys only): fp16 [batch entry][token][128] with strides rope_stride_batch (0 when all
+ *   batch entries share the positions) and rope_stride_token.  Every one of the `rows` tokens becomes
+ *   (x * cos) + (rotate_half(x) * sin), each product and the sum rounded to fp16 as the half-precision tensor
+ *   expression rounds them, and is written to rot (strides like x; rot may be x itself with the same strides -
+ *   the one case in which an input is modified - but must not overlap it otherwise);
+ *   the first M tokens (M % 64 == 0, M <= rows; M may be 0 with cos / sin: rotation only) are then pruned and
+ *   compressed exactly as mstf_compress_*_f16 / mstf_append_*_f16 would compress the contiguous copy, with
+ *   B = batch * heads.  nz must be given (there is no sizing-only mode).  Workspace:
+ *   mstf_compress_workspace_bytes(batch * heads, M, 128). */
+typedef struct mstf_proj_source {
+    const mstf_half* x;
+    int64_t stride_batch, stride_token, stride_head;
+    int batch, heads, rows;
+    const mstf_half* cos;
+    const mstf_half* sin;
+    int64_t rope_stride_batch, rope_stride_token;
+    mstf_half* rot;
+    int64_t rot_stride_batch, rot_stride_token, rot_stride_head;
+} mstf_proj_source;
+int mstf_compress_proj_f16(void* stream, const mstf_proj_source* src, int is_value, int M, int N, int kth,
+                           uint64_t* bmp, uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz,
+                           uint64_t nz_capacity_halfs, void* workspace, size_t workspace_bytes);
+int mstf_append_proj_f16(void* stream, const mstf_proj_source* src, int is_value, int M, int N, int kth,
+                         uint64_t* bmp, uint32_t* idx, const uint32_t* dst_off, const uint32_t* dst_limit,
+                         mstf_half* nz, uint32_t* overflow, void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ key SpMV (K1)
  * Replaces mustafar_key_formulation (kernel/kernel_wrapper/mustafar_wrapper.cu:19-133 ->
  * Key_SplitK_API, kernel/csrc/SpMM_API.cu:179 -> Key_Kernel, kernel/csrc/SpMM_Kernel.cuh:240-520):

@@ -17,6 +17,18 @@ _i64 = ctypes.c_int64
 _u64 = ctypes.c_uint64
 _sz = ctypes.c_size_t
 
+
+
+class ProjSource(ctypes.Structure):
+    """struct mstf_proj_source of include/mustafar_hip.h."""
+    _fields_ = [("x", _vp), ("stride_batch", _i64), ("stride_token", _i64), ("stride_head", _i64),
+                ("batch", _i), ("heads", _i), ("rows", _i),
+                ("cos", _vp), ("sin", _vp), ("rope_stride_batch", _i64), ("rope_stride_token", _i64),
+                ("rot", _vp), ("rot_stride_batch", _i64), ("rot_stride_token", _i64), ("rot_stride_head", _i64)]
+
+
+_ps = ctypes.POINTER(ProjSource)
+
 # name -> (restype, argtypes); must list every symbol of include/mustafar_hip.h
 SIGNATURES = {
     "mstf_strerror": (ctypes.c_char_p, [_i]),
@@ -30,6 +42,8 @@ SIGNATURES = {
     "mstf_scatter_value_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _u64]),
     "mstf_append_key_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "mstf_append_value_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "mstf_compress_proj_f16": (_i, [_vp, _ps, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _sz]),
+    "mstf_append_proj_f16": (_i, [_vp, _ps, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "mstf_key_spmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     "mstf_value_spmv_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "mstf_value_spmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz]),

@@ -94,6 +94,30 @@ class CompressedPool:
         self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
         self.tokens += M
 
+    def append_proj(self, x, kth, M, cos=None, sin=None, rot=None):
+        """The first M tokens of x [batch, rows, heads per batch entry, head_dim] (a view of the projection output,
+        ops.proj_source) without a contiguous copy; with cos / sin all rows are rotated into rot (default: in place)
+        before the first M are compressed."""
+        import ctypes
+        src, rot = ops.proj_source(x, cos, sin, rot)
+        B, N = x.shape[0] * x.shape[2], x.shape[3]
+        assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
+        L = lib()
+        Tc = M * N // 64
+        bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
+        idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
+        dst = self.nz_off + self.idx[:, -1] // 4
+        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, max(M, 64), N))
+        check(L.mstf_append_proj_f16(torch.cuda.current_stream().cuda_stream, ctypes.byref(src), int(self.is_value), M, N,
+                                     int(kth), bmp_c.data_ptr(), idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(),
+                                     self.nz.data_ptr(), self.overflow.data_ptr(), ws.data_ptr(), ws.numel()),
+              "mstf_append_proj_f16")
+        if M > 0:
+            self.bmp = torch.cat([self.bmp, bmp_c], dim=1)
+            self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
+            self.tokens += M
+        return rot
+
     def view(self):
         """The cache as the operators take it (ops.key_spmv / value_spmv / decode_attention)."""
         return ops.CompressedKV(self.bmp, self.idx, self.nz, self.nz_off, self.tokens, self.head_dim, self.is_value,
@@ -149,12 +173,41 @@ class SparseKVCache:
         cv = ops.compress(V.reshape(bs * n_kv, L, D), True, kth=self.kth_v)
         return ck, cv
 
+    def prefill_proj(self, kx, vx, cos, sin):
+        """Prefill straight from the projection outputs kx, vx [bs, L, n_kv, D] (views of [bs, L, n_kv * D]; the keys
+        not yet rotated) and the rotary factors cos, sin [L, D] or [bs, L, D]: the keys are rotated in place, the
+        first Lc tokens of both sides are compressed from where they lie (no transposed or contiguous copy), the rest
+        becomes the dense window.  Returns the rotated keys and the values as [bs, n_kv, L, D] views for the prefill
+        attention (models/llama_mustafar_kernel.py:373-374, 531-560 in one pass over K and one over V)."""
+        bs, L, n_kv, D = kx.shape
+        Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
+        if self.max_tokens > 0:
+            if self.k_pool is None:
+                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, kx.device)
+                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, kx.device)
+            self.k_pool.append_proj(kx, self.kth_k, Lc, cos, sin)
+            if Lc > 0:
+                self.v_pool.append_proj(vx, self.kth_v, Lc)
+                self.k, self.v = self.k_pool.view(), self.v_pool.view()
+        else:
+            ck, _ = ops.compress_proj(kx, False, self.kth_k, Lc, cos, sin)
+            if Lc > 0:
+                cv, _ = ops.compress_proj(vx, True, self.kth_v, Lc)
+                self.k, self.v = ck, cv
+        K, V = kx.transpose(1, 2), vx.transpose(1, 2)
+        self._prefill_window(K, V, Lc)
+        return K, V
+
     def prefill(self, K, V):
         """K, V: [bs, n_kv, L, D] fp16 (after RoPE)."""
         L = K.shape[2]
         Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
         if Lc > 0:
             self._grow(K[:, :, :Lc].contiguous(), V[:, :, :Lc].contiguous())
+        self._prefill_window(K, V, Lc)
+
+    def _prefill_window(self, K, V, Lc):
+        L = K.shape[2]
         self.compressed_length, self.kv_len = Lc, L
         if self.window_kernel:
             bs, n_kv, _, D = K.shape

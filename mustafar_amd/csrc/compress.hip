@@ -61,6 +61,53 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
     }
 }
 
+// The same for rows in the layout of a projection output (RowsView), one unit per wavefront, optionally with the
+// rotary embedding applied first.  With ROPE the grid covers all `rows` tokens of a head (ceil(rows / 64) units):
+// every unit rotates its rows and writes them to rot (same kind of layout, rot.x may be the input itself), and only
+// the units below M / 64 go on to prune and count.  cos / sin: [batch entry][token][128] fp16 with strides rb, rt.
+struct RopeTables {
+    const _Float16* cos;
+    const _Float16* sin;
+    int64_t rb, rt;
+};
+template <bool IS_VALUE, bool ROPE>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void proj_count_kernel(
+    RowsView src, RopeTables rope, RowsView rot, int rows, int M, int kth, uint64_t* __restrict__ bmp,
+    uint32_t* __restrict__ idx, uint32_t* __restrict__ unit_tot)
+{
+    __shared__ uint32_t slab[kHalfSlabDw];
+    const int lane = lane_id();
+    const int nblk = M / 64;
+    const int nblk_all = ROPE ? (rows + 63) / 64 : nblk;
+    const size_t T = (size_t)M * kD / 64;
+    const int unit = (int)blockIdx.x;
+    const int b = unit / nblk_all, tb = unit - b * nblk_all;
+    uint32_t mag[64];
+    unit_rows(src.head(b), (int64_t)tb * 64, (int64_t)rows, slab, lane, mag, src.st);
+    if (ROPE) {
+        const int bt = b / src.heads;
+        const int64_t t = (int64_t)tb * 64 + lane;
+        rope_row(mag, rope.cos + bt * rope.rb + t * rope.rt, rope.sin + bt * rope.rb + t * rope.rt, t < rows);
+        unit_rows_store(const_cast<_Float16*>(rot.head(b)), (int64_t)tb * 64, (int64_t)rows, slab, lane, mag, rot.st);
+        if (tb >= nblk) return;  // uniform: a unit of the dense tail
+    }
+#pragma unroll
+    for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
+    uint64_t bmA, bmB;
+    unit_keep<IS_VALUE>(mag, kth, lane, bmA, bmB);
+    uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
+    bo[lane] = bmA;
+    bo[64 + lane] = bmB;
+    const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
+    uint32_t totA, totB;
+    const uint32_t eA = wave_excl_scan(cA, lane, totA);
+    const uint32_t eB = wave_excl_scan(cB, lane, totB);
+    uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
+    io[lane] = eA;
+    io[64 + lane] = totA + eB;
+    if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
+}
+
 // ------------------------------------------------------------------------------- scans
 // grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base, idx[b][T] = head total.
 // With nz_off given (the compress entry points) the workgroup also adds up the unit totals of all earlier heads:
@@ -162,8 +209,9 @@ __device__ __forceinline__ void scatter_half(const uint32_t (&v)[32], uint64_t b
 // the unit-local offsets of the count kernel, which are completed here with unit_base (ADD_BASE true).
 // head_limit (nullable): end of head b's slab in 16-byte units from nz; a unit whose values would pass it is
 // skipped and *overflow is set.
-template <bool IS_VALUE, bool ADD_BASE>
-__global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, int M,
+// PROJ: the rows come through `view` (x is ignored) instead of the contiguous [B, M, 128] matrix x.
+template <bool IS_VALUE, bool ADD_BASE, bool PROJ = false>
+__global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, RowsView view, int M,
                                                               const uint64_t* __restrict__ bmp, uint32_t* idx,
                                                               const uint32_t* __restrict__ unit_base,
                                                               const uint32_t* __restrict__ nz_off,
@@ -216,7 +264,10 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
         uint32_t bytes = ((h == 0 ? mid : end) - s_h) * 4u;
         if (bytes > 64u * 128u) bytes = 64u * 128u;  // never true for offsets that follow from the bitmaps
         uint32_t v[32];
-        half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, buf, lane);
+        if (PROJ)
+            half_slab_load(view.head(b), (int64_t)tb * 64, (int64_t)M, h, buf, lane, view.st);
+        else
+            half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, buf, lane);
         __builtin_amdgcn_wave_barrier();
         row_of_lane(buf, lane, v, 0);
         __builtin_amdgcn_wave_barrier();
@@ -289,7 +340,7 @@ static int scatter_impl(void* stream, const mstf_half* x, int B, int M, int N, c
     if (!bmp || !idx || !nz_off || !nz) return MSTF_EINVAL;
     if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz_off, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
     hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, false>), dim3((unsigned)(B * (M / 64))), dim3(64), 0,
-                       as_stream(stream), reinterpret_cast<const _Float16*>(x), M, bmp, const_cast<uint32_t*>(idx),
+                       as_stream(stream), reinterpret_cast<const _Float16*>(x), RowsView{}, M, bmp, const_cast<uint32_t*>(idx),
                        (const uint32_t*)nullptr, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
                        (uint32_t*)nullptr);
     return check_launch();
@@ -332,8 +383,8 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     if ((rc = check_launch()) != MSTF_OK) return rc;
     if (nz) {
         if (!aligned_to(nz, 16)) return MSTF_EALIGN;
-        hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M,
-                           bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
+        hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh,
+                           RowsView{}, M, bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
                            (uint32_t*)nullptr);
     } else {
         hipLaunchKernelGGL(finalize_idx_kernel, dim3((unsigned)(((size_t)nblk * kD + 255) / 256), (unsigned)B), dim3(256),
@@ -367,8 +418,83 @@ static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, in
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
                        (uint32_t*)nullptr, (uint64_t*)nullptr, nblk, kD);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bmp,
-                       idx, unit_base, dst_off, reinterpret_cast<char*>(nz), ~0ull, dst_limit, overflow);
+    hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, RowsView{},
+                       M, bmp, idx, unit_base, dst_off, reinterpret_cast<char*>(nz), ~0ull, dst_limit, overflow);
+    return check_launch();
+}
+
+// Rows in the layout of a projection output, optionally rotated first.  dst_off == nullptr: the compress contract
+// (nz_off and *total_halfs are outputs), else the append contract (dst_off / dst_limit / overflow are inputs).
+static int proj_impl(void* stream, const mstf_proj_source* s, int is_value, int M, int N, int kth, uint64_t* bmp,
+                     uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, const uint32_t* dst_off,
+                     const uint32_t* dst_limit, mstf_half* nz, uint64_t cap, uint32_t* overflow, void* ws, size_t ws_bytes)
+{
+    if (!s || !s->x || s->batch <= 0 || s->heads <= 0 || s->rows <= 0 || M < 0 || M > s->rows || kth < 0 || kth > N)
+        return MSTF_EINVAL;
+    if (N != kD || M % 64 != 0) return MSTF_EUNSUPPORTED;
+    const bool rope = s->cos || s->sin;
+    if (rope && (!s->cos || !s->sin || !s->rot || is_value)) return MSTF_EINVAL;
+    if (M == 0 && !rope) return MSTF_EINVAL;
+    const int64_t strides[] = {s->stride_batch, s->stride_token, s->stride_head, rope ? s->rope_stride_batch : 0,
+                               rope ? s->rope_stride_token : 0, rope ? s->rot_stride_batch : 0,
+                               rope ? s->rot_stride_token : 0, rope ? s->rot_stride_head : 0};
+    for (int64_t v : strides)
+        if (v < 0 || v % 8 != 0) return MSTF_EINVAL;
+    if (!aligned_to(s->x, 16) || (rope && (!aligned_to(s->cos, 16) || !aligned_to(s->sin, 16) || !aligned_to(s->rot, 16))))
+        return MSTF_EALIGN;
+    const int64_t B64 = (int64_t)s->batch * s->heads;
+    const int64_t units_all = B64 * ((s->rows + 63) / 64);
+    if (units_all > 0x7FFFFFFF || M / 64 > 8192) return MSTF_EUNSUPPORTED;
+    const int B = (int)B64;
+    const int nblk = M / 64;
+    hipStream_t st = as_stream(stream);
+    const RowsView src{reinterpret_cast<const _Float16*>(s->x), s->stride_batch, s->stride_token, s->stride_head, s->heads};
+    const RowsView rot{reinterpret_cast<const _Float16*>(s->rot), s->rot_stride_batch, s->rot_stride_token,
+                       s->rot_stride_head, s->heads};
+    const RopeTables tab{reinterpret_cast<const _Float16*>(s->cos), reinterpret_cast<const _Float16*>(s->sin),
+                         s->rope_stride_batch, s->rope_stride_token};
+    uint32_t* unit_tot = nullptr;
+    uint32_t* unit_base = nullptr;
+    if (M > 0) {
+        if (!bmp || !idx || !nz) return MSTF_EINVAL;
+        if (dst_off ? (!dst_limit || !overflow) : (!nz_off || !total_halfs)) return MSTF_EINVAL;
+        if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
+        if (dst_off ? (!aligned_to(dst_off, 4) || !aligned_to(dst_limit, 4) || !aligned_to(overflow, 4))
+                    : (!aligned_to(nz_off, 4) || !aligned_to(total_halfs, 8)))
+            return MSTF_EALIGN;
+        if (!ws || ws_bytes < compress_ws_bytes(B, M)) return MSTF_EWORKSPACE;
+        if (!aligned_to(ws, 256)) return MSTF_EALIGN;
+        unit_tot = reinterpret_cast<uint32_t*>(ws);
+        unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + round_up((size_t)B * nblk * 4, 256));
+    }
+    const unsigned grid = rope ? (unsigned)units_all : (unsigned)(B * nblk);
+#define MSTF_PC(V, R)                                                                                              \
+    hipLaunchKernelGGL((proj_count_kernel<V, R>), dim3(grid), dim3(64), 0, st, src, tab, rot, s->rows, M, kth, bmp, idx, \
+                       unit_tot)
+    if (rope)
+        MSTF_PC(false, true);
+    else if (is_value)
+        MSTF_PC(true, false);
+    else
+        MSTF_PC(false, false);
+#undef MSTF_PC
+    int rc = check_launch();
+    if (rc != MSTF_OK || M == 0) return rc;
+    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
+                       dst_off ? (uint32_t*)nullptr : nz_off, dst_off ? (uint64_t*)nullptr : total_halfs, nblk, kD);
+    if ((rc = check_launch()) != MSTF_OK) return rc;
+    const RowsView rd = rope ? rot : src;  // the scatter pass reads the rotated rows
+    const uint32_t* base_of_head = dst_off ? dst_off : nz_off;
+    const uint64_t capacity = dst_off ? ~0ull : cap;
+#define MSTF_PS(V)                                                                                                  \
+    hipLaunchKernelGGL((compress_scatter_kernel<V, true, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st,       \
+                       (const _Float16*)nullptr, rd, M, bmp, idx, unit_base, base_of_head, reinterpret_cast<char*>(nz), \
+                       capacity, dst_limit, overflow)
+    if (is_value)
+        MSTF_PS(true);
+    else
+        MSTF_PS(false);
+#undef MSTF_PS
     return check_launch();
 }
 
@@ -438,4 +564,21 @@ extern "C" int mstf_prune_rows_f16(void* stream, const mstf_half* x, mstf_half* 
     hipLaunchKernelGGL(prune_rows_kernel, dim3((unsigned)units), dim3(64), 0, as_stream(stream),
                        reinterpret_cast<const _Float16*>(x), reinterpret_cast<_Float16*>(y), rows, kth);
     return check_launch();
+}
+
+extern "C" int mstf_compress_proj_f16(void* stream, const mstf_proj_source* src, int is_value, int M, int N, int kth,
+                                      uint64_t* bmp, uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs,
+                                      mstf_half* nz, uint64_t nz_capacity_halfs, void* workspace, size_t workspace_bytes)
+{
+    return proj_impl(stream, src, is_value, M, N, kth, bmp, idx, nz_off, total_halfs, nullptr, nullptr, nz,
+                     nz_capacity_halfs, nullptr, workspace, workspace_bytes);
+}
+
+extern "C" int mstf_append_proj_f16(void* stream, const mstf_proj_source* src, int is_value, int M, int N, int kth,
+                                    uint64_t* bmp, uint32_t* idx, const uint32_t* dst_off, const uint32_t* dst_limit,
+                                    mstf_half* nz, uint32_t* overflow, void* workspace, size_t workspace_bytes)
+{
+    if (!dst_off) return MSTF_EINVAL;
+    return proj_impl(stream, src, is_value, M, N, kth, bmp, idx, nullptr, nullptr, dst_off, dst_limit, nz, 0, overflow,
+                     workspace, workspace_bytes);
 }

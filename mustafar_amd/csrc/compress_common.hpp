@@ -16,18 +16,19 @@ typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ us2_t as_us2(uint32_t x) { return __builtin_bit_cast(us2_t, x); }
 __device__ __forceinline__ uint32_t us2_u32(us2_t x) { return __builtin_bit_cast(uint32_t, x); }
 
-// Streams channels [64h, 64h+64) of rows [row0, row0+64) of a [rows, 128] fp16 matrix into the padded
-// half-slab (rows >= rows_valid as zeros); afterwards lane = token reads its own 32 dwords with row_of_lane.
+// Streams channels [64h, 64h+64) of rows [row0, row0+64) of an fp16 matrix with 128 channels per row and `stride`
+// elements between rows (128: a plain [rows, 128] matrix) into the padded half-slab (rows >= rows_valid as
+// zeros); afterwards lane = token reads its own 32 dwords with row_of_lane.
 __device__ __forceinline__ void half_slab_load(const _Float16* x, int64_t row0, int64_t rows_valid, int h, uint32_t* slab,
-                                               int lane)
+                                               int lane, int64_t stride = kD)
 {
-    const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD) + h * 8;
+    const _Float16* src = x + row0 * stride + h * 64;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const int e = j * 64 + lane;  // 16-byte piece index inside the half-slab: 8 pieces per row
         const int row = e >> 3, c16 = e & 7;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + row < rows_valid) v = src[row * 16 + c16];
+        if (row0 + row < rows_valid) v = *reinterpret_cast<const uint4*>(src + row * stride + c16 * 8);
         uint32_t* d = slab + row * kHalfRowDw + c16 * 4;
         d[0] = v.x;
         d[1] = v.y;
@@ -44,14 +45,84 @@ __device__ __forceinline__ void row_of_lane(const uint32_t* slab, int lane, uint
 }
 // Both halves of the lane's row (raw fp16 pairs, signs included) through one half-slab buffer.
 __device__ __forceinline__ void unit_rows(const _Float16* x, int64_t row0, int64_t rows_valid, uint32_t* slab, int lane,
-                                          uint32_t (&r)[64])
+                                          uint32_t (&r)[64], int64_t stride = kD)
 {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        half_slab_load(x, row0, rows_valid, h, slab, lane);
+        half_slab_load(x, row0, rows_valid, h, slab, lane, stride);
         __builtin_amdgcn_wave_barrier();
         row_of_lane(slab, lane, r, 32 * h);
         __builtin_amdgcn_wave_barrier();
+    }
+}
+// The reverse: the lane's row r[0 .. 64) to rows [row0, row0+64) of a matrix with `stride` elements between rows
+// (rows >= rows_valid are not written), as 16-byte stores.
+__device__ __forceinline__ void unit_rows_store(_Float16* y, int64_t row0, int64_t rows_valid, uint32_t* slab, int lane,
+                                                const uint32_t (&r)[64], int64_t stride)
+{
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
+        __builtin_amdgcn_wave_barrier();
+        _Float16* dst = y + row0 * stride + h * 64;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = j * 64 + lane;
+            const int row = e >> 3, c16 = e & 7;
+            const uint32_t* sp = slab + row * kHalfRowDw + c16 * 4;
+            if (row0 + row < rows_valid)
+                *reinterpret_cast<uint4*>(dst + row * stride + c16 * 8) = make_uint4(sp[0], sp[1], sp[2], sp[3]);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// Rows that are not a contiguous [heads, rows, 128] matrix: element (batch entry bt, token t, KV head h, channel c)
+// at x[bt * sb + t * st + h * sh + c].  A projection output [batch, tokens, heads * 128] has sb = tokens * heads * 128,
+// st = heads * 128, sh = 128.  Heads are numbered b = bt * heads + h.
+struct RowsView {
+    const _Float16* x;
+    int64_t sb, st, sh;
+    int heads;
+    __device__ __forceinline__ const _Float16* head(int b) const
+    {
+        const int bt = b / heads;
+        return x + bt * sb + (b - bt * heads) * sh;
+    }
+};
+
+// Rotary position embedding of the lane's row in place, with the roundings of the half-precision expression
+// (x * cos) + (rotate_half(x) * sin), rotate_half(x) = [-x[64:], x[:64]]: both products and the sum are rounded to
+// fp16 one by one (no fused multiply-add).  cos_row / sin_row: the 128 fp16 factors of the lane's token.
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void rope_row(uint32_t (&r)[64], const _Float16* cos_row, const _Float16* sin_row, bool valid)
+{
+#pragma clang fp contract(off)
+    const uint4* cp = reinterpret_cast<const uint4*>(cos_row);
+    const uint4* sp = reinterpret_cast<const uint4*>(sin_row);
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        uint4 c1 = make_uint4(0u, 0u, 0u, 0u), c2 = c1, s1 = c1, s2 = c1;
+        if (valid) {
+            c1 = cp[q];
+            c2 = cp[8 + q];
+            s1 = sp[q];
+            s2 = sp[8 + q];
+        }
+        const uint32_t C1[4] = {c1.x, c1.y, c1.z, c1.w}, C2[4] = {c2.x, c2.y, c2.z, c2.w};
+        const uint32_t S1[4] = {s1.x, s1.y, s1.z, s1.w}, S2[4] = {s2.x, s2.y, s2.z, s2.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int j = 4 * q + k;
+            const h2_t a = __builtin_bit_cast(h2_t, r[j]), b = __builtin_bit_cast(h2_t, r[j + 32]);
+            const h2_t p1 = a * __builtin_bit_cast(h2_t, C1[k]);
+            const h2_t p2 = (-b) * __builtin_bit_cast(h2_t, S1[k]);
+            const h2_t p3 = b * __builtin_bit_cast(h2_t, C2[k]);
+            const h2_t p4 = a * __builtin_bit_cast(h2_t, S2[k]);
+            r[j] = __builtin_bit_cast(uint32_t, (h2_t)(p1 + p2));
+            r[j + 32] = __builtin_bit_cast(uint32_t, (h2_t)(p3 + p4));
+        }
     }
 }
 

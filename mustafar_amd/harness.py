@@ -93,8 +93,12 @@ def _rope(x, tables):
 
 
 class Decoder:
-    def __init__(self, cfg, device, seed=0, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=0):
+    def __init__(self, cfg, device, seed=0, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=0,
+                 proj_prefill=True):
+        """proj_prefill: the fp16 sparse cache takes the keys and values of the prompt straight from the projection
+        output (keys rotated by the compressor's own kernel, no transposed or contiguous copies)."""
         self.cfg, self.dev = cfg, device
+        self.proj_prefill = proj_prefill
         g = torch.Generator(device=device)
         g.manual_seed(seed)
 
@@ -156,17 +160,25 @@ class Decoder:
         c = self.cfg
         bs, L = ids.shape
         tables = _rope_tables(torch.arange(L, device=self.dev), c.head_dim, c.rope_theta, torch.float16)
+        half = c.head_dim // 2
+        usin = torch.cat([-tables[1][:, :half], tables[1][:, half:]], -1)   # sin itself: the kernel rotates with rotate_half
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            q, k, v = self._qkv(lw, h, tables)
-            k = k.contiguous()
+            if self.proj_prefill and type(cache) is SparseKVCache:
+                qkv = F.linear(h, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim)
+                q = _rope(qkv[:, :, : c.n_q].transpose(1, 2), tables)
+                k, v = cache.prefill_proj(qkv[:, :, c.n_q: c.n_q + c.n_kv], qkv[:, :, c.n_q + c.n_kv:], tables[0], usin)
+            else:
+                q, k, v = self._qkv(lw, h, tables)
+                k = k.contiguous()
             outs = []
             for b0 in range(0, bs, seq_chunk):   # bounded working set of the prefill attention
                 outs.append(F.scaled_dot_product_attention(q[b0:b0 + seq_chunk], k[b0:b0 + seq_chunk], v[b0:b0 + seq_chunk],
                                                            is_causal=True, enable_gqa=True))
             a = torch.cat(outs, 0).transpose(1, 2).reshape(bs, L, c.n_q * c.head_dim)
-            cache.prefill(k, v)
+            if not (self.proj_prefill and type(cache) is SparseKVCache):
+                cache.prefill(k, v)
             x = x + F.linear(a, lw["o"])
             h = _rms_norm(x, lw["ln2"], c.rms_eps)
             for b0 in range(0, bs, seq_chunk):
@@ -267,11 +279,15 @@ def main():
     ap.add_argument("--residual", type=int, default=256)
     ap.add_argument("--cache", default="sparse", choices=["sparse", "sparse_quant2", "sparse_quant4", "dense_masked"])
     ap.add_argument("--graph", action="store_true", help="replay the decode step from a HIP graph (sparse cache only)")
+    ap.add_argument("--copy-prefill", action="store_true",
+                    help="prefill through rotated, transposed, contiguous copies of K and V instead of compressing "
+                         "them where the projection left them")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = Config(layers=args.layers)
     max_tokens = ((args.prompt + args.new_tokens + CHUNK - 1) // CHUNK) * CHUNK
-    dec = Decoder(cfg, dev, cache=args.cache, sparsity=args.sparsity, residual_length=args.residual, max_tokens=max_tokens)
+    dec = Decoder(cfg, dev, cache=args.cache, sparsity=args.sparsity, residual_length=args.residual, max_tokens=max_tokens,
+                  proj_prefill=not args.copy_prefill)
     g = torch.Generator(device=dev)
     g.manual_seed(1)
     ids = torch.randint(0, cfg.vocab, (args.batch, args.prompt), generator=g, device=dev)

@@ -101,6 +101,56 @@ def compress(x, is_value, kth=0, capacity_halfs=None):
     return CompressedKV(bmp, idx, nz, nz_off, M, N, is_value, total)
 
 
+def proj_source(x, cos=None, sin=None, rot=None):
+    """The mstf_proj_source of x [batch, rows, heads, 128] fp16 (any strides with contiguous channels, e.g. a view of
+    a projection output [batch, rows, heads * 128]).  cos, sin: [rows, 128] or [batch, rows, 128] fp16 (keys only);
+    rot: where the rotated rows go, shaped like x (default: x itself, in place).  Returns (struct, rot)."""
+    from ._lib import ProjSource
+    assert x.is_cuda and x.dtype == torch.float16 and x.dim() == 4 and x.stride(3) == 1
+    src = ProjSource()
+    src.x = x.data_ptr()
+    src.stride_batch, src.stride_token, src.stride_head = x.stride(0), x.stride(1), x.stride(2)
+    src.batch, src.rows, src.heads = x.shape[0], x.shape[1], x.shape[2]
+    if cos is not None:
+        assert sin is not None and cos.dtype == sin.dtype == torch.float16 and cos.shape == sin.shape
+        assert cos.stride(-1) == 1 and sin.stride() == cos.stride() and cos.shape[-2] >= x.shape[1]
+        rot = x if rot is None else rot
+        assert rot.shape == x.shape and rot.dtype == torch.float16 and rot.stride(3) == 1
+        src.cos, src.sin = cos.data_ptr(), sin.data_ptr()
+        src.rope_stride_batch = cos.stride(0) if cos.dim() == 3 and cos.shape[0] > 1 else 0
+        src.rope_stride_token = cos.stride(-2)
+        src.rot = rot.data_ptr()
+        src.rot_stride_batch, src.rot_stride_token, src.rot_stride_head = rot.stride(0), rot.stride(1), rot.stride(2)
+    return src, rot
+
+
+def compress_proj(x, is_value, kth, M, cos=None, sin=None, rot=None, capacity_halfs=None):
+    """Prune and compress the first M tokens of x [batch, rows, heads, 128] where the projection left them, the keys
+    rotated first when cos / sin are given (all rows are rotated and written to rot).  Heads are numbered
+    batch * heads + head.  Returns (CompressedKV, rot)."""
+    import ctypes
+    src, rot = proj_source(x, cos, sin, rot)
+    B, N, dev = x.shape[0] * x.shape[2], x.shape[3], x.device
+    T = M * N // 64
+    L = lib()
+    cap = B * M * N if capacity_halfs is None else int(capacity_halfs)
+    bmp = torch.empty((B, T), dtype=torch.int64, device=dev)
+    idx = torch.empty((B, T + 1), dtype=torch.int32, device=dev)
+    nz_off = torch.empty((B,), dtype=torch.int32, device=dev)
+    total = torch.empty((1,), dtype=torch.int64, device=dev)
+    nz = torch.empty((max(cap, 8),), dtype=torch.float16, device=dev)
+    ws = workspace(dev, L.mstf_compress_workspace_bytes(B, max(M, 64), N))
+    check(L.mstf_compress_proj_f16(_stream(), ctypes.byref(src), int(is_value), M, N, int(kth), bmp.data_ptr(),
+                                   idx.data_ptr(), nz_off.data_ptr(), total.data_ptr(), nz.data_ptr(), cap,
+                                   ws.data_ptr(), ws.numel()), "mstf_compress_proj_f16")
+    if M == 0:
+        return None, rot
+    if capacity_halfs is None:
+        n = int(total.item())
+        return CompressedKV(bmp, idx, nz[:n], nz_off, M, N, is_value, n), rot
+    return CompressedKV(bmp, idx, nz, nz_off, M, N, is_value, total), rot
+
+
 def key_spmv(ck, q, groups, n_rows=1, out=None):
     """scores[bq, n, t] = sum_d K[bq // groups][t, d] * q[bq, n, d]   (unscaled).  q: [Bq, n_rows, D]."""
     assert q.dtype == torch.float16 and q.is_contiguous()

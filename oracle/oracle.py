@@ -201,6 +201,27 @@ def spmv_quant(bmp, packed, tile_off, scales, zeros, Bm, is_value, Lc, D, groups
     return C, Cf
 
 
+# ------------------------------------------------------- rotary embedding in front of the compressor
+def rope_tables(positions, D=128, theta=500000.0):
+    """cos, sin [len(positions), D] fp16 as LlamaRotaryEmbedding of transformers 4.43.1 builds them (the reference
+    calls it at models/llama_mustafar_kernel.py:373): inv_freq = theta^(-2i/D), emb = [freqs, freqs], cos and sin in
+    fp32, cast to the activations' dtype."""
+    inv = (1.0 / (np.float32(theta) ** (np.arange(0, D, 2, dtype=np.float32) / np.float32(D)))).astype(np.float32)
+    f = np.asarray(positions, np.float32)[:, None] * inv[None, :]
+    emb = np.concatenate([f, f], axis=-1)
+    return np.cos(emb).astype(np.float16), np.sin(emb).astype(np.float16)
+
+
+def rope_rows(x, cos, sin):
+    """apply_rotary_pos_emb of transformers 4.43.1 (called at models/llama_mustafar_kernel.py:374) on fp16 rows
+    x [..., tokens, D] with cos, sin [tokens, D]: (x * cos) + (rotate_half(x) * sin), every product and the sum
+    rounded to fp16 (numpy's float16 arithmetic rounds each operation once, like the half-precision tensor ops)."""
+    x = np.asarray(x, np.float16)
+    h = x.shape[-1] // 2
+    rot = np.concatenate([-x[..., h:], x[..., :h]], axis=-1)
+    return ((x * cos).astype(np.float16) + (rot * sin).astype(np.float16)).astype(np.float16)
+
+
 # ------------------------------------------------------- synthetic inputs
 def make_kv(seed, Bkv, L, D=128, outlier_channels=4, outlier_scale=10.0):
     """Seeded K and V: fp16 N(0,1); K gets `outlier_channels` channels per head scaled by `outlier_scale`."""

@@ -56,3 +56,26 @@ def test_graphed_loop_generates_the_same_tokens_as_the_eager_loop():
     got = torch.cat(got, 1)
     assert loop.captures == 2 and graphed.caches[0].compressed_length == eager.caches[0].compressed_length == 512
     assert torch.equal(got, toks)
+
+
+def test_prefill_from_the_projection_output_fills_the_same_cache():
+    """Prompt keys / values compressed where the projection left them (keys rotated in the compressor's kernel)
+    against the route through rotated, transposed, contiguous copies: the first layer's cache is identical bit for
+    bit (its inputs are), the logits agree."""
+    from mustafar_amd.harness import Config, Decoder
+    dev = torch.device("cuda:0")
+    cfg = Config(hidden=512, layers=2, n_q=4, n_kv=2, head_dim=128, ffn=1024, vocab=1000)
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    ids = torch.randint(0, cfg.vocab, (3, 600), generator=g, device=dev)
+    a = Decoder(cfg, dev, seed=4, cache="sparse", max_tokens=1024, proj_prefill=False)
+    b = Decoder(cfg, dev, seed=4, cache="sparse", max_tokens=1024, proj_prefill=True)
+    la, lb = a.prefill(ids), b.prefill(ids)
+    ca, cb = a.caches[0], b.caches[0]
+    assert ca.compressed_length == cb.compressed_length == 256
+    for sa, sb in ((ca.k, cb.k), (ca.v, cb.v)):
+        assert torch.equal(sa.bmp, sb.bmp) and torch.equal(sa.idx, sb.idx)
+        assert torch.equal(sa.nz.view(torch.int16), sb.nz.view(torch.int16))
+    assert torch.equal(ca.k_win.view(torch.int16), cb.k_win.view(torch.int16))
+    assert torch.equal(ca.v_win.view(torch.int16), cb.v_win.view(torch.int16))
+    assert float((la - lb).abs().max() / la.abs().max()) < 1e-2
