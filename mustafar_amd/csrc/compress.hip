@@ -61,51 +61,100 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
     }
 }
 
-// The same for rows in the layout of a projection output (RowsView), one unit per wavefront, optionally with the
-// rotary embedding applied first.  With ROPE the grid covers all `rows` tokens of a head (ceil(rows / 64) units):
-// every unit rotates its rows and writes them to rot (same kind of layout, rot.x may be the input itself), and only
-// the units below M / 64 go on to prune and count.  cos / sin: [batch entry][token][128] fp16 with strides rb, rt.
+// The same for rows in the layout of a projection output (RowsView), optionally with the rotary embedding applied
+// first.  With ROPE the units cover all `rows` tokens of a head (ceil(rows / 64) per head): every unit rotates its
+// rows on the way in - in the layout of the loads, where a lane holds 8 channels of a row and their partners 64
+// channels on, so that x, cos, sin and the rotated rows all move as 128-byte runs - writes them to rot (same kind of
+// layout; rot.x may be the input itself) and only the units below M / 64 go on to prune and count.
+// cos / sin: [batch entry][token][128] fp16 with strides rb, rt.
 struct RopeTables {
     const _Float16* cos;
     const _Float16* sin;
     int64_t rb, rt;
 };
+__device__ __forceinline__ void unit_fetch_rotated(const RowsView& src, const RopeTables& rope, const RowsView& rot, int b,
+                                                   int tb, int rows, int lane, UnitRaw& raw)
+{
+    const int bt = b / src.heads;
+    const _Float16* xb = src.head(b);
+    _Float16* rb = const_cast<_Float16*>(rot.head(b));
+    const _Float16* cb = rope.cos + bt * rope.rb;
+    const _Float16* sb = rope.sin + bt * rope.rb;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int e = j * 64 + lane;
+        const int64_t t = (int64_t)tb * 64 + (e >> 3);
+        const int c = (e & 7) * 8;
+        const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+        uint4 x0 = z, x1 = z, c0 = z, c1 = z, s0 = z, s1 = z;
+        if (t < rows) {
+            const _Float16* xp = xb + t * src.st + c;
+            const _Float16* cp = cb + t * rope.rt + c;
+            const _Float16* sp = sb + t * rope.rt + c;
+            x0 = *reinterpret_cast<const uint4*>(xp);
+            x1 = *reinterpret_cast<const uint4*>(xp + 64);
+            c0 = *reinterpret_cast<const uint4*>(cp);
+            c1 = *reinterpret_cast<const uint4*>(cp + 64);
+            s0 = *reinterpret_cast<const uint4*>(sp);
+            s1 = *reinterpret_cast<const uint4*>(sp + 64);
+        }
+        rope_piece(x0, x1, c0, c1, s0, s1, raw.v[0][j], raw.v[1][j]);
+        if (t < rows) {
+            _Float16* rp = rb + t * rot.st + c;
+            *reinterpret_cast<uint4*>(rp) = raw.v[0][j];
+            *reinterpret_cast<uint4*>(rp + 64) = raw.v[1][j];
+        }
+    }
+}
+// grid = ceil(units / upw), 64 threads; units = B * (ROPE ? ceil(rows / 64) : M / 64); upw = 1 with ROPE.
 template <bool IS_VALUE, bool ROPE>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void proj_count_kernel(
     RowsView src, RopeTables rope, RowsView rot, int rows, int M, int kth, uint64_t* __restrict__ bmp,
-    uint32_t* __restrict__ idx, uint32_t* __restrict__ unit_tot)
+    uint32_t* __restrict__ idx, uint32_t* __restrict__ unit_tot, int units, int upw)
 {
     __shared__ uint32_t slab[kHalfSlabDw];
     const int lane = lane_id();
     const int nblk = M / 64;
     const int nblk_all = ROPE ? (rows + 63) / 64 : nblk;
     const size_t T = (size_t)M * kD / 64;
-    const int unit = (int)blockIdx.x;
-    const int b = unit / nblk_all, tb = unit - b * nblk_all;
-    uint32_t mag[64];
-    unit_rows(src.head(b), (int64_t)tb * 64, (int64_t)rows, slab, lane, mag, src.st);
-    if (ROPE) {
-        const int bt = b / src.heads;
-        const int64_t t = (int64_t)tb * 64 + lane;
-        rope_row(mag, rope.cos + bt * rope.rb + t * rope.rt, rope.sin + bt * rope.rb + t * rope.rt, t < rows);
-        unit_rows_store(const_cast<_Float16*>(rot.head(b)), (int64_t)tb * 64, (int64_t)rows, slab, lane, mag, rot.st);
-        if (tb >= nblk) return;  // uniform: a unit of the dense tail
+    const int unit0 = (int)blockIdx.x * upw;
+    int n = units - unit0;
+    n = n > upw ? upw : n;
+    UnitRaw raw;
+    if (!ROPE) {
+        const int b0 = unit0 / nblk_all;
+        unit_fetch(src.head(b0), (int64_t)(unit0 - b0 * nblk_all) * 64, lane, raw, src.st);
     }
+#pragma unroll 1
+    for (int u = 0; u < n; u++) {
+        const int unit = unit0 + u;
+        const int b = unit / nblk_all, tb = unit - b * nblk_all;
+        if (ROPE) {
+            unit_fetch_rotated(src, rope, rot, b, tb, rows, lane, raw);
+            if (tb >= nblk) continue;  // uniform: a unit of the dense tail
+        }
+        uint32_t mag[64];
+        unit_rows_from(raw, slab, lane, mag);
+        if (!ROPE && u + 1 < n) {
+            const int bn = (unit + 1) / nblk_all;
+            unit_fetch(src.head(bn), (int64_t)(unit + 1 - bn * nblk_all) * 64, lane, raw, src.st);
+        }
 #pragma unroll
-    for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
-    uint64_t bmA, bmB;
-    unit_keep<IS_VALUE>(mag, kth, lane, bmA, bmB);
-    uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
-    bo[lane] = bmA;
-    bo[64 + lane] = bmB;
-    const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
-    uint32_t totA, totB;
-    const uint32_t eA = wave_excl_scan(cA, lane, totA);
-    const uint32_t eB = wave_excl_scan(cB, lane, totB);
-    uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
-    io[lane] = eA;
-    io[64 + lane] = totA + eB;
-    if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
+        for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
+        uint64_t bmA, bmB;
+        unit_keep<IS_VALUE>(mag, kth, lane, bmA, bmB);
+        uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
+        bo[lane] = bmA;
+        bo[64 + lane] = bmB;
+        const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
+        uint32_t totA, totB;
+        const uint32_t eA = wave_excl_scan(cA, lane, totA);
+        const uint32_t eB = wave_excl_scan(cB, lane, totB);
+        uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
+        io[lane] = eA;
+        io[64 + lane] = totA + eB;
+        if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
+    }
 }
 
 // ------------------------------------------------------------------------------- scans
@@ -467,10 +516,12 @@ static int proj_impl(void* stream, const mstf_proj_source* s, int is_value, int 
         unit_tot = reinterpret_cast<uint32_t*>(ws);
         unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + round_up((size_t)B * nblk * 4, 256));
     }
-    const unsigned grid = rope ? (unsigned)units_all : (unsigned)(B * nblk);
+    const int units = rope ? (int)units_all : B * nblk;
+    const int upw = !rope && units >= 4096 ? 2 : 1;
+    const unsigned grid = (unsigned)((units + upw - 1) / upw);
 #define MSTF_PC(V, R)                                                                                              \
     hipLaunchKernelGGL((proj_count_kernel<V, R>), dim3(grid), dim3(64), 0, st, src, tab, rot, s->rows, M, kth, bmp, idx, \
-                       unit_tot)
+                       unit_tot, units, upw)
     if (rope)
         MSTF_PC(false, true);
     else if (is_value)

@@ -55,29 +55,6 @@ __device__ __forceinline__ void unit_rows(const _Float16* x, int64_t row0, int64
         __builtin_amdgcn_wave_barrier();
     }
 }
-// The reverse: the lane's row r[0 .. 64) to rows [row0, row0+64) of a matrix with `stride` elements between rows
-// (rows >= rows_valid are not written), as 16-byte stores.
-__device__ __forceinline__ void unit_rows_store(_Float16* y, int64_t row0, int64_t rows_valid, uint32_t* slab, int lane,
-                                                const uint32_t (&r)[64], int64_t stride)
-{
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-#pragma unroll
-        for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
-        __builtin_amdgcn_wave_barrier();
-        _Float16* dst = y + row0 * stride + h * 64;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int e = j * 64 + lane;
-            const int row = e >> 3, c16 = e & 7;
-            const uint32_t* sp = slab + row * kHalfRowDw + c16 * 4;
-            if (row0 + row < rows_valid)
-                *reinterpret_cast<uint4*>(dst + row * stride + c16 * 8) = make_uint4(sp[0], sp[1], sp[2], sp[3]);
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
-}
-
 // Rows that are not a contiguous [heads, rows, 128] matrix: element (batch entry bt, token t, KV head h, channel c)
 // at x[bt * sb + t * st + h * sh + c].  A projection output [batch, tokens, heads * 128] has sb = tokens * heads * 128,
 // st = heads * 128, sh = 128.  Heads are numbered b = bt * heads + h.
@@ -92,38 +69,30 @@ struct RowsView {
     }
 };
 
-// Rotary position embedding of the lane's row in place, with the roundings of the half-precision expression
-// (x * cos) + (rotate_half(x) * sin), rotate_half(x) = [-x[64:], x[:64]]: both products and the sum are rounded to
-// fp16 one by one (no fused multiply-add).  cos_row / sin_row: the 128 fp16 factors of the lane's token.
+// Rotary position embedding of 8 channels c .. c+7 < 64 of a row (x0) and their partners c+64 .. (x1), with the
+// roundings of the half-precision expression (x * cos) + (rotate_half(x) * sin), rotate_half(x) = [-x[64:], x[:64]]:
+// both products and the sum are rounded to fp16 one by one (no fused multiply-add).
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void rope_row(uint32_t (&r)[64], const _Float16* cos_row, const _Float16* sin_row, bool valid)
+__device__ __forceinline__ void rope_piece(const uint4& x0, const uint4& x1, const uint4& c0, const uint4& c1,
+                                           const uint4& s0, const uint4& s1, uint4& o0, uint4& o1)
 {
 #pragma clang fp contract(off)
-    const uint4* cp = reinterpret_cast<const uint4*>(cos_row);
-    const uint4* sp = reinterpret_cast<const uint4*>(sin_row);
+    const uint32_t X0[4] = {x0.x, x0.y, x0.z, x0.w}, X1[4] = {x1.x, x1.y, x1.z, x1.w};
+    const uint32_t C0[4] = {c0.x, c0.y, c0.z, c0.w}, C1[4] = {c1.x, c1.y, c1.z, c1.w};
+    const uint32_t S0[4] = {s0.x, s0.y, s0.z, s0.w}, S1[4] = {s1.x, s1.y, s1.z, s1.w};
+    uint32_t O0[4], O1[4];
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        uint4 c1 = make_uint4(0u, 0u, 0u, 0u), c2 = c1, s1 = c1, s2 = c1;
-        if (valid) {
-            c1 = cp[q];
-            c2 = cp[8 + q];
-            s1 = sp[q];
-            s2 = sp[8 + q];
-        }
-        const uint32_t C1[4] = {c1.x, c1.y, c1.z, c1.w}, C2[4] = {c2.x, c2.y, c2.z, c2.w};
-        const uint32_t S1[4] = {s1.x, s1.y, s1.z, s1.w}, S2[4] = {s2.x, s2.y, s2.z, s2.w};
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int j = 4 * q + k;
-            const h2_t a = __builtin_bit_cast(h2_t, r[j]), b = __builtin_bit_cast(h2_t, r[j + 32]);
-            const h2_t p1 = a * __builtin_bit_cast(h2_t, C1[k]);
-            const h2_t p2 = (-b) * __builtin_bit_cast(h2_t, S1[k]);
-            const h2_t p3 = b * __builtin_bit_cast(h2_t, C2[k]);
-            const h2_t p4 = a * __builtin_bit_cast(h2_t, S2[k]);
-            r[j] = __builtin_bit_cast(uint32_t, (h2_t)(p1 + p2));
-            r[j + 32] = __builtin_bit_cast(uint32_t, (h2_t)(p3 + p4));
-        }
+    for (int k = 0; k < 4; k++) {
+        const h2_t a = __builtin_bit_cast(h2_t, X0[k]), b = __builtin_bit_cast(h2_t, X1[k]);
+        const h2_t p1 = a * __builtin_bit_cast(h2_t, C0[k]);
+        const h2_t p2 = (-b) * __builtin_bit_cast(h2_t, S0[k]);
+        const h2_t p3 = b * __builtin_bit_cast(h2_t, C1[k]);
+        const h2_t p4 = a * __builtin_bit_cast(h2_t, S1[k]);
+        O0[k] = __builtin_bit_cast(uint32_t, (h2_t)(p1 + p2));
+        O1[k] = __builtin_bit_cast(uint32_t, (h2_t)(p3 + p4));
     }
+    o0 = make_uint4(O0[0], O0[1], O0[2], O0[3]);
+    o1 = make_uint4(O1[0], O1[1], O1[2], O1[3]);
 }
 
 // The same in two steps, for a wavefront that requests its next unit while it works on the current one:
@@ -132,15 +101,15 @@ __device__ __forceinline__ void rope_row(uint32_t (&r)[64], const _Float16* cos_
 struct UnitRaw {
     uint4 v[2][8];
 };
-__device__ __forceinline__ void unit_fetch(const _Float16* x, int64_t row0, int lane, UnitRaw& raw)
+__device__ __forceinline__ void unit_fetch(const _Float16* x, int64_t row0, int lane, UnitRaw& raw, int64_t stride = kD)
 {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        const uint4* src = reinterpret_cast<const uint4*>(x + row0 * kD) + h * 8;
+        const _Float16* src = x + row0 * stride + h * 64;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const int e = j * 64 + lane;
-            raw.v[h][j] = src[(e >> 3) * 16 + (e & 7)];
+            raw.v[h][j] = *reinterpret_cast<const uint4*>(src + (e >> 3) * stride + (e & 7) * 8);
         }
     }
 }
