@@ -25,7 +25,7 @@ namespace mstf {
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
 template <int NM, bool MULTI>
-__global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
+__global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(4))) void decode_attention_kernel(
     const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
@@ -85,27 +85,29 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         // boundaries, lanes 16.. the value boundaries): no stage then waits for a scalar load from HBM
         // before it can issue its value stream
         static_assert(kKeySubs < 16 && kValSubs < 48, "boundary lanes");
-        auto boundaries = [&](const uint32_t* ik, const uint32_t* iv) {
-            uint32_t b = 0u;
-            if (lane <= kKeySubs) b = ik[lane * kSubTiles];
-            else if (lane >= 16 && lane <= 16 + kValSubs) b = iv[(lane - 16) * kSubTiles];
-            return b;
-        };
+        // (one unconditional load from a selected address: a branch here would split the block while the coming
+        // scalar batch is live)
+        const bool bnd_v = lane >= 16 && lane <= 16 + kValSubs;
+        const int bnd_i = bnd_v ? (lane - 16) * kSubTiles : (lane <= kKeySubs ? lane * kSubTiles : 0);
+        auto boundaries = [&](const uint32_t* ik, const uint32_t* iv) { return (bnd_v ? iv : ik)[bnd_i]; };
         uint32_t bnd = boundaries(ixK, ixV);
         uint32_t bnd_next = bnd;  // MULTI: boundaries of the coming block
+        const uint32_t lane16 = (uint32_t)lane * 16u;
+        const uint32_t off8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
+        const uint32_t off4 = (uint32_t)(lane <= kSubTiles ? lane : kSubTiles) * 4u;
         auto issue = [&](int n) {
             const int bl = n < kKeySubs ? n : 16 + n - kKeySubs;
             const uint32_t s0 = __builtin_amdgcn_readlane(bnd, bl);
             const uint32_t s1 = __builtin_amdgcn_readlane(bnd, bl + 1);
-            sub_issue(nz_of(n) + (size_t)s0 * 4u, sub_bytes(s0, s1), my + (n & 1) * kSubBytes, lane);
-            return touch_sub(bm_of(n), ix_of(n), lane);
+            sub_issue_flat(nz_of(n) + (size_t)s0 * 4u, sub_bytes(s0, s1), lbase + (uint32_t)(n & 1) * kSubBytes, lane16);
+            return touch_sub_flat(bm_of(n), ix_of(n), off8, off4);
         };
         // first key sub-chunk of the coming block (adv = D tiles ahead; adv = 0 and no bytes after the last block)
         auto issue_coming = [&](int adv) {
             const uint32_t s0 = __builtin_amdgcn_readlane(bnd_next, 0);
             const uint32_t s1 = __builtin_amdgcn_readlane(bnd_next, 1);
-            sub_issue(nzK + (size_t)s0 * 4u, adv ? sub_bytes(s0, s1) : 0u, my, lane);
-            return touch_sub(bmK + adv, ixK + adv, lane);
+            sub_issue_flat(nzK + (size_t)s0 * 4u, adv ? sub_bytes(s0, s1) : 0u, lbase, lane16);
+            return touch_sub_flat(bmK + adv, ixK + adv, off8, off4);
         };
 
         // the query rows of this KV head: groups x D fp16, contiguous
@@ -127,21 +129,30 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
         // ahead; the chain runs across the stages, from the key tiles into the value tiles and (MULTI) into the
         // coming block.
         constexpr int kBatches = kSubTiles / 8, kSideBatches = D / 8;
-        Batch cur = load_batch(bmK, ixK);
-        auto stage_batches = [&](int n, uint32_t buf, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM], int adv) {
+        Batch cur = load_batch_scalar(bmK, ixK);
+        // nc, woffc: stage index and byte offset of the stage's first weight from wbase, as constants (they end up in
+        // immediate operands)
+        auto stage_batches = [&](auto nc, uint32_t buf, uint32_t wbase, auto woffc, uint32_t wgroup, f4_t (&acc)[NM],
+                                 int adv) {
+            constexpr int n = decltype(nc)::value;
+            constexpr int woff = decltype(woffc)::value;
             const uint32_t rel = buf - cur.ov[0] * 4u;  // idx counts 4-byte units from the start of the head's values
-#pragma unroll
-            for (int g = 0; g < kBatches; g++) {
-                const int g1 = n * kBatches + g + 1;
-                Batch nxt = cur;
-                if (g1 < 2 * kSideBatches)
-                    nxt = g1 < kSideBatches ? prefetch_batch(bmK + 8 * g1, ixK + 8 * g1)
-                                            : prefetch_batch(bmV + 8 * (g1 - kSideBatches), ixV + 8 * (g1 - kSideBatches));
-                else if (MULTI)
-                    nxt = prefetch_batch(bmK + adv, ixK + adv);
-                batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
+            static_for<kBatches>([&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                constexpr int g1 = n * kBatches + g + 1;  // the coming batch, counted over key then value tiles
+                constexpr int wo = woff + g * 16;
+                Batch nxt;
+                if constexpr (g1 < kSideBatches)
+                    batch_step_exec<NM, true, g1 * 64, g1 * 32, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc);
+                else if constexpr (g1 < 2 * kSideBatches)
+                    batch_step_exec<NM, true, (g1 - kSideBatches) * 64, (g1 - kSideBatches) * 32, wo>(cur, nxt, bmV, ixV, rel,
+                                                                                                    zaddr, wbase, wgroup, acc);
+                else if constexpr (MULTI)
+                    batch_step_exec<NM, true, 0, 0, wo>(cur, nxt, bmK + adv, ixK + adv, rel, zaddr, wbase, wgroup, acc);
+                else
+                    batch_step_exec<NM, false, 0, 0, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc);
                 cur = nxt;
-            }
+            });
         };
 
 #pragma unroll 1
@@ -155,37 +166,37 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_kernel(
                 blk_v[m][0] = f4_t{0.f, 0.f, 0.f, 0.f};
                 blk_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
             }
-#pragma unroll
-            for (int n = 0; n < kStages; n++) {
+            static_for<kStages>([&](auto nc) {
+                constexpr int n = decltype(nc)::value;
                 wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for the first one)
                 // The buffer of sub-chunk n-1 is refilled now: every LDS read of that sub-chunk fed an MFMA that was
-                // issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would also
-                // drain the scalar prefetch of the coming batch and expose its round trip at every stage.)
+                // issued before this point, so the reads have returned.
                 __builtin_amdgcn_sched_barrier(0);
-                if (n + 1 < kStages) touch = issue(n + 1);
-                else if (MULTI) touch = issue_coming(adv);
+                if constexpr (n + 1 < kStages) touch = issue(n + 1);
+                else if constexpr (MULTI) touch = issue_coming(adv);
                 const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
-                if (n < kKeySubs) {
-                    stage_batches(n, buf, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k, adv);
+                if constexpr (n < kKeySubs) {
+                    stage_batches(nc, buf, qrow, std::integral_constant<int, n * kSubTiles * 2>{}, (uint32_t)D * 8u, acc_k,
+                                  adv);
                 } else {
-                    if (n == kKeySubs) {
+                    if constexpr (n == kKeySubs) {
                         block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_blk, l_blk);
                         // its latency is covered by the value phase; the wait of the next stage completes it
                         if (MULTI) bnd_next = boundaries(ixK + adv, ixV + adv);
                     }
-                    const int vs = n - kKeySubs;                  // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
+                    constexpr int vs = n - kKeySubs;              // value sub-chunk: half = vs / 2, tokens (vs % 2)*32..
                     constexpr int kSubsPerHalf = 64 / kSubTiles;
-                    const int half = vs / kSubsPerHalf;
-                    const uint32_t wa = prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u;
+                    constexpr int half = vs / kSubsPerHalf;
                     f4_t tmp[NM];
 #pragma unroll
                     for (int m = 0; m < NM; m++) tmp[m] = blk_v[m][half];
-                    stage_batches(n, buf, wa, 4u * kPRow, tmp, adv);
+                    stage_batches(nc, buf, prow, std::integral_constant<int, (vs % kSubsPerHalf) * kSubTiles * 2>{},
+                                  4u * kPRow, tmp, adv);
 #pragma unroll
                     for (int m = 0; m < NM; m++) blk_v[m][half] = tmp[m];
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
+            });
             if (!MULTI) {
 #pragma unroll
                 for (int m = 0; m < NM; m++) {

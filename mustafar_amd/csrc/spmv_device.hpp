@@ -1,6 +1,7 @@
 // Device-side building blocks shared by the SpMV kernels (spmv.hip) and the fused decode kernel
 // (fused.hip): LDS-direct staging, tile decompression and the MFMA accumulation of a sub-chunk.
 #pragma once
+#include <utility>
 #include "common.hpp"
 
 namespace mstf {
@@ -142,6 +143,108 @@ __device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, u
     }
 }
 
+// The same batch with the wavefront's exec mask set to each tile's bitmap in turn: only the lanes whose element is
+// present compute a rank and read LDS, the others keep the zero their destination was cleared to (four destinations
+// per 16-byte LDS read of the zero slot at zaddr; LDS reads of a wavefront return in order, so the gathers land on
+// top), so the select instruction disappears - per tile one s_brev_b64 into exec, two v_mbcnt on exec, the
+// scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (v112-v127, the top of the budget of a kernel that runs four wavefronts per SIMD, listed as
+// clobbered) because nothing of the compiler's may be scheduled while exec is partial; the wavefront must be in
+// uniform control flow with all 64 lanes active.  The scalar loads of the coming batch (PREFETCH) are part of the
+// statement: requested first, completed by its one wait - the compiler, which cannot see that wait, would otherwise
+// put one of its own in front of the statement and expose the round trip of a request it has just made.
+//   nbm + BOFF bytes, nix + IOFF bytes : bitmaps and offsets of the coming batch
+//   wbase + WOFF                      : LDS byte address of w[lane & 3][first tile of the batch]
+template <int NM, bool PREFETCH, int BOFF, int IOFF, int WOFF>
+__device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, const uint64_t* nbm, const uint32_t* nix,
+                                                uint32_t rel, uint32_t zaddr, uint32_t wbase, uint32_t wgroup,
+                                                f4_t (&acc)[NM])
+{
+    u32x4_t qm[NM];
+#pragma unroll
+    for (int m = 1; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(wbase + (uint32_t)WOFF + (uint32_t)m * wgroup);
+    uint32_t v0, v1, v2, v3, t;
+#define MSTF_TILE(I, H, A)                                       \
+    "s_brev_b64 exec, %[m" #I "]\n\t"                            \
+    "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
+    "v_mbcnt_hi_u32_b32 v" #A ", exec_hi, v" #A "\n\t"           \
+    "s_lshl2_add_u32 %[t], %[o" #I "], %[rel]\n\t"               \
+    "v_lshl_add_u32 v" #A ", v" #A ", 1, %[t]\n\t"               \
+    "ds_read_u16 v" #H ", v" #A "\n\t"
+#define MSTF_GATHER                                                                                                  \
+    "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                                   \
+    "ds_read_b128 v[112:115], %[z]\n\t"                                                                              \
+    "ds_read_b128 v[116:119], %[z]\n\t"                                                                              \
+    MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)                              \
+    MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)                              \
+    "s_mov_b64 exec, -1\n\t"                                                                                         \
+    "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
+    "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                                          \
+    "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                                          \
+    "v_lshl_or_b32 %[v2], v117, 16, v116\n\t"                                                                          \
+    "v_lshl_or_b32 %[v3], v119, 16, v118"
+#define MSTF_GATHER_IN                                                                                               \
+    [m0] "s"(u64_of(b.mv[0], b.mv[1])), [m1] "s"(u64_of(b.mv[2], b.mv[3])), [m2] "s"(u64_of(b.mv[4], b.mv[5])),      \
+        [m3] "s"(u64_of(b.mv[6], b.mv[7])), [m4] "s"(u64_of(b.mv[8], b.mv[9])), [m5] "s"(u64_of(b.mv[10], b.mv[11])), \
+        [m6] "s"(u64_of(b.mv[12], b.mv[13])), [m7] "s"(u64_of(b.mv[14], b.mv[15])), [o0] "s"(b.ov[0]),               \
+        [o1] "s"(b.ov[1]), [o2] "s"(b.ov[2]), [o3] "s"(b.ov[3]), [o4] "s"(b.ov[4]), [o5] "s"(b.ov[5]),               \
+        [o6] "s"(b.ov[6]), [o7] "s"(b.ov[7]), [rel] "s"(rel), [wa] "v"(wbase), [woff] "i"(WOFF), [z] "v"(zaddr)
+#define MSTF_GATHER_CLOBBER                                                                                          \
+    "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127",  \
+        "scc", "memory"
+    if constexpr (PREFETCH) {
+        asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t"
+                     "s_load_dwordx8 %[no], %[ni], %[ioff]\n\t" MSTF_GATHER
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [t] "=&s"(t),
+                       [nm] "=&s"(nxt.mv), [no] "=&s"(nxt.ov)
+                     : MSTF_GATHER_IN, [nb] "s"(nbm), [ni] "s"(nix), [boff] "i"(BOFF), [ioff] "i"(IOFF)
+                     : MSTF_GATHER_CLOBBER);
+    } else {
+        asm volatile(MSTF_GATHER
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [t] "=&s"(t)
+                     : MSTF_GATHER_IN
+                     : MSTF_GATHER_CLOBBER);
+        nxt = b;
+    }
+#undef MSTF_TILE
+#undef MSTF_GATHER
+#undef MSTF_GATHER_IN
+#undef MSTF_GATHER_CLOBBER
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(qm[m][0], qm[m][1]), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(qm[m][2], qm[m][3]), acc[m], 0, 0, 0);
+        // pins the products here: left free, they may all be sunk to the first use of the sums, with every
+        // batch's operands kept in registers until then
+        asm volatile("" : "+v"(acc[m]));
+    }
+}
+
+// The first batch of a chain for batch_step_exec: requested and waited for in one statement, so that the values are
+// in scalar registers whatever the compiler makes of other loads through the same pointers.
+__device__ __forceinline__ Batch load_batch_scalar(const uint64_t* bm, const uint32_t* ix)
+{
+    Batch b;
+    asm volatile("s_load_dwordx16 %0, %2, 0\n\ts_load_dwordx8 %1, %3, 0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(b.mv), "=&s"(b.ov)
+                 : "s"(bm), "s"(ix)
+                 : "memory");
+    return b;
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
+// constant expression in the body (immediate operands of the statement above).
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+
 // The next batch's scalar loads, requested a whole batch ahead and pinned where they are written: left to
 // itself the scheduler sinks them to their first use and every batch waits out an L2 round trip.
 __device__ __forceinline__ Batch prefetch_batch(const uint64_t* bm, const uint32_t* ix)
@@ -201,6 +304,49 @@ __device__ __forceinline__ Touch touch_sub(const uint64_t* bm, const uint32_t* i
 __device__ __forceinline__ void wait_vm0_keep(Touch& t)
 {
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(t.bm.x), "+v"(t.bm.y), "+v"(t.ix)::"memory");
+}
+
+// sub_issue and touch_sub without control flow, for a caller that keeps scalar state (the coming batch) in
+// registers across them: a lane predicate written as a branch splits the block there, and values that live
+// across such a split may end up in vector registers.  The four pieces are issued with exec set by hand
+// (piece i: the lanes with lane*16 + i*1024 < bytes; an empty exec issues nothing) - one compare, one exec write
+// and the load per piece, where the branches cost ten instructions; the wavefront must have all 64 lanes active.
+//   dst_lds : LDS byte address of the buffer (wave-uniform);  lane16 = lane * 16
+__device__ __forceinline__ void sub_issue_flat(const char* src, uint32_t bytes, uint32_t dst_lds, uint32_t lane16)
+{
+    static_assert(kSubBytes == 4096, "four 1 KB pieces");
+    uint32_t t, m0_kept;  // m0 is the compiler's to manage: handed back as it was found
+    asm volatile("s_mov_b32 %[keep], m0\n\t"
+                 "s_mov_b32 m0, %[dst]\n\t"
+                 "v_cmp_gt_i32 vcc, %[b], %[l]\n\t"
+                 "s_mov_b64 exec, vcc\n\t"
+                 "global_load_lds_dwordx4 %[l], %[src]\n\t"
+                 "s_sub_i32 %[t], %[b], 0x400\n\t"
+                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
+                 "s_mov_b64 exec, vcc\n\t"
+                 "global_load_lds_dwordx4 %[l], %[src] offset:1024\n\t"
+                 "s_sub_i32 %[t], %[b], 0x800\n\t"
+                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
+                 "s_mov_b64 exec, vcc\n\t"
+                 "global_load_lds_dwordx4 %[l], %[src] offset:2048\n\t"
+                 "s_sub_i32 %[t], %[b], 0xc00\n\t"
+                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
+                 "s_mov_b64 exec, vcc\n\t"
+                 "global_load_lds_dwordx4 %[l], %[src] offset:3072\n\t"
+                 "s_mov_b64 exec, -1\n\t"
+                 "s_mov_b32 m0, %[keep]"
+                 : [t] "=&s"(t), [keep] "=&s"(m0_kept)
+                 : [dst] "s"(dst_lds), [b] "s"(bytes), [l] "v"(lane16), [src] "s"(src)
+                 : "vcc", "scc", "memory");
+}
+// Every lane touches one bitmap and one offset of the sub-chunk; the lanes beyond it repeat the last one.
+//   off8 = min(lane, kSubTiles - 1) * 8, off4 = min(lane, kSubTiles) * 4
+__device__ __forceinline__ Touch touch_sub_flat(const uint64_t* bm, const uint32_t* ix, uint32_t off8, uint32_t off4)
+{
+    Touch t;
+    t.bm = *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(bm) + off8);
+    t.ix = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(ix) + off4);
+    return t;
 }
 
 // Walks `nsubs` sub-chunks of one KV head with a two-deep pipeline: while sub-chunk n is being
