@@ -23,7 +23,7 @@ namespace mstf {
 // C[(kv*rows + row0 + n)*Lc + token] = sum_d K[token][d] * Bm[(kv*rows + row0 + n)*D + d],  n < NW.
 // LDS per wavefront: value double buffer + zero slot + the NW query rows (4*NM rows reserved).
 template <int NW>
-__global__ __launch_bounds__(256) void key_spmv_kernel(const uint64_t* __restrict__ bmp, const char* __restrict__ nz,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void key_spmv_kernel(const uint64_t* __restrict__ bmp, const char* __restrict__ nz,
                                                        const uint32_t* __restrict__ idx,
                                                        const uint32_t* __restrict__ nz_off,
                                                        const _Float16* __restrict__ Bm, _Float16* __restrict__ C,
@@ -134,8 +134,11 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_kernel(
             const size_t tok0 = (size_t)(first + n / subs_per_blk) * 64 + (size_t)(n % subs_per_blk) * kSubTiles;
 #pragma unroll
             for (int i = 0; i < (NM * 4 + kRowsPer - 1) / kRowsPer; i++) {
-                const int row = kRowsPer * i + lane / kDwPerRow;
-                if (row < NW) dma4(wk + (size_t)row * Lc + tok0 + 2 * (lane % kDwPerRow), wl + (n & 1) * kWBuf + i * 256);
+                // no lane predicate (a branch here would split the block while the coming scalar batch is live): the
+                // lanes of rows >= NW fetch row NW - 1 again, into buffer rows whose products are never stored
+                int row = kRowsPer * i + lane / kDwPerRow;
+                row = row < NW ? row : NW - 1;
+                dma4(wk + (size_t)row * Lc + tok0 + 2 * (lane % kDwPerRow), wl + (n & 1) * kWBuf + i * 256);
             }
         },
         [=](int n) { return wrow + (uint32_t)(n & 1) * kWBuf; }, 4u * kWRow, bmk, ixk, nzk, my, lane, acc);

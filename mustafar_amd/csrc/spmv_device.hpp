@@ -359,38 +359,57 @@ __device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stag
                                           const uint64_t* bmk, const uint32_t* ixk, const char* nzk, char* my, int lane,
                                           f4_t (&acc)[NM])
 {
+    // stage_w must be free of lane-dependent branches: the coming scalar batch is live across it (see sub_issue_flat)
     const uint32_t lbase = lds_addr(my);
     const uint32_t zaddr = lbase + 2 * kSubBytes;
     if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
     if (nsubs <= 0) return;
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+    const uint32_t off8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
+    const uint32_t off4 = (uint32_t)(lane <= kSubTiles ? lane : kSubTiles) * 4u;
     size_t t_cur = tile_of(0);
-    const uint32_t s0 = ixk[t_cur];
-    sub_issue(nzk + (size_t)s0 * 4u, sub_bytes(s0, ixk[t_cur + kSubTiles]), my, lane);
+    // (the offsets may come back through a vector load; the statements below want them in scalar registers)
+    auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+    const uint32_t s0 = uni(ixk[t_cur]);
+    sub_issue_flat(nzk + (size_t)s0 * 4u, sub_bytes(s0, uni(ixk[t_cur + kSubTiles])), lbase, lane16);
     stage_w(0);
-    Touch touch = touch_sub(bmk + t_cur, ixk + t_cur, lane);
+    Touch touch = touch_sub_flat(bmk + t_cur, ixk + t_cur, off8, off4);
     size_t t_nxt = nsubs > 1 ? tile_of(1) : t_cur;
-    uint32_t s_nxt = ixk[t_nxt], e_nxt = ixk[t_nxt + kSubTiles];
-    Batch cur = load_batch(bmk + t_cur, ixk + t_cur);
+    uint32_t s_nxt = uni(ixk[t_nxt]), e_nxt = uni(ixk[t_nxt + kSubTiles]);
+    Batch cur = load_batch_scalar(bmk + t_cur, ixk + t_cur);
+    constexpr int G = kSubTiles / 8;
     for (int n = 0; n < nsubs; n++) {
         wait_vm0_keep(touch);  // sub-chunk n (values, weights) has landed
         // Buffer (n+1)&1 is refilled now.  Its last reader was sub-chunk n-1, and every LDS read of that sub-chunk
-        // fed an MFMA issued before this point, so the reads have returned.  (An s_waitcnt lgkmcnt instead would
-        // also drain the scalar request for the coming batch and expose its round trip at every sub-chunk.)
+        // fed an MFMA issued before this point, so the reads have returned.
         __builtin_amdgcn_sched_barrier(0);
         if (n + 1 < nsubs) {
-            sub_issue(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), my + ((n + 1) & 1) * kSubBytes, lane);
+            sub_issue_flat(nzk + (size_t)s_nxt * 4u, sub_bytes(s_nxt, e_nxt), lbase + (uint32_t)((n + 1) & 1) * kSubBytes,
+                           lane16);
             stage_w(n + 1);
-            touch = touch_sub(bmk + t_nxt, ixk + t_nxt, lane);
+            touch = touch_sub_flat(bmk + t_nxt, ixk + t_nxt, off8, off4);
         }
         const size_t t_now = t_cur;
         t_cur = t_nxt;
         if (n + 2 < nsubs) {
             t_nxt = tile_of(n + 2);
-            s_nxt = ixk[t_nxt];
-            e_nxt = ixk[t_nxt + kSubTiles];
+            s_nxt = uni(ixk[t_nxt]);
+            e_nxt = uni(ixk[t_nxt + kSubTiles]);
         }
-        sub_accumulate<NM>(cur, bmk + t_now, ixk + t_now, bmk + t_cur, ixk + t_cur, lbase + (uint32_t)(n & 1) * kSubBytes,
-                           zaddr, waddr_of(n), wgroup, acc);
+        const uint32_t rel = lbase + (uint32_t)(n & 1) * kSubBytes - cur.ov[0] * 4u;
+        const uint32_t wbase = waddr_of(n);
+        const uint64_t* bm_now = bmk + t_now;
+        const uint32_t* ix_now = ixk + t_now;
+        static_for<G>([&](auto gc) {
+            constexpr int g = decltype(gc)::value;
+            Batch nxt;
+            if constexpr (g + 1 < G)
+                batch_step_exec<NM, true, (g + 1) * 64, (g + 1) * 32, g * 16>(cur, nxt, bm_now, ix_now, rel, zaddr, wbase,
+                                                                             wgroup, acc);
+            else  // the first batch of the coming sub-chunk (of this one again after the last: loaded, never used)
+                batch_step_exec<NM, true, 0, 0, g * 16>(cur, nxt, bmk + t_cur, ixk + t_cur, rel, zaddr, wbase, wgroup, acc);
+            cur = nxt;
+        });
         __builtin_amdgcn_sched_barrier(0);
     }
     wait_lgkm0();
