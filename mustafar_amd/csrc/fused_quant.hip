@@ -138,15 +138,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             dequant_stage<BIT>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
                                lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), lane, mode);
-            const uint64_t* bm = S.bmp + t;
-            u32x16_t cur = load_bitmaps(bm);
-#pragma unroll
-            for (int g = 0; g < kSubTiles / 8; g++) {
-                u32x16_t nxt = cur;
-                if (g + 1 < kSubTiles / 8) nxt = prefetch_bitmaps(bm + 8 * (g + 1));
-                batch_accumulate_img<NM>(cur, lbase + (uint32_t)g * 1024u, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
-                cur = nxt;
-            }
+            stage_img_exec<NM>(S.bmp + t, lbase, zaddr, waddr, wgroup, acc);
         };
 
 #pragma unroll

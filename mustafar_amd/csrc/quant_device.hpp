@@ -130,6 +130,87 @@ __device__ __forceinline__ void batch_accumulate_img(const u32x16_t& mv, uint32_
     }
 }
 
+// The same with the gather under the tile's exec mask (see batch_step_exec in spmv_device.hpp): one statement per
+// batch of 8 tiles on fixed registers v112-v127; the image slots of tile i sit at img + IMG + 128 * i, so the tile's
+// base is an immediate offset of the LDS read.  PREFETCH: the bitmaps of the coming batch (bm + BOFF bytes) are
+// requested first and completed by the statement's wait.
+template <int NM, bool PREFETCH, int BOFF, int IMG, int WOFF>
+__device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t& nxt, const uint64_t* bm, uint32_t img,
+                                                    uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM])
+{
+    u32x4_t qm[NM];
+#pragma unroll
+    for (int m = 1; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(wbase + (uint32_t)WOFF + (uint32_t)m * wgroup);
+    uint32_t v0, v1, v2, v3;
+#define MSTF_TILE(I, H, A)                                       \
+    "s_brev_b64 exec, %[m" #I "]\n\t"                            \
+    "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
+    "v_mbcnt_hi_u32_b32 v" #A ", exec_hi, v" #A "\n\t"           \
+    "v_lshl_add_u32 v" #A ", v" #A ", 1, %[img]\n\t"             \
+    "ds_read_u16 v" #H ", v" #A " offset:%[i" #I "]\n\t"
+#define MSTF_GATHER                                                                                  \
+    "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                   \
+    "ds_read_b128 v[112:115], %[z]\n\t"                                                              \
+    "ds_read_b128 v[116:119], %[z]\n\t"                                                              \
+    MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)      \
+    MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)      \
+    "s_mov_b64 exec, -1\n\t"                                                                         \
+    "s_waitcnt lgkmcnt(0)\n\t"                                                                       \
+    "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                        \
+    "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                        \
+    "v_lshl_or_b32 %[v2], v117, 16, v116\n\t"                                                        \
+    "v_lshl_or_b32 %[v3], v119, 16, v118"
+#define MSTF_IN                                                                                                      \
+    [m0] "s"(u64_of(mv[0], mv[1])), [m1] "s"(u64_of(mv[2], mv[3])), [m2] "s"(u64_of(mv[4], mv[5])),                  \
+        [m3] "s"(u64_of(mv[6], mv[7])), [m4] "s"(u64_of(mv[8], mv[9])), [m5] "s"(u64_of(mv[10], mv[11])),            \
+        [m6] "s"(u64_of(mv[12], mv[13])), [m7] "s"(u64_of(mv[14], mv[15])), [img] "s"(img), [wa] "v"(wbase),         \
+        [woff] "i"(WOFF), [z] "v"(zaddr), [i0] "i"(IMG), [i1] "i"(IMG + 128), [i2] "i"(IMG + 256), [i3] "i"(IMG + 384), \
+        [i4] "i"(IMG + 512), [i5] "i"(IMG + 640), [i6] "i"(IMG + 768), [i7] "i"(IMG + 896)
+#define MSTF_CLOBBER                                                                                                 \
+    "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",  \
+        "v126", "v127", "memory"
+    if constexpr (PREFETCH) {
+        asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t" MSTF_GATHER
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [nm] "=&s"(nxt)
+                     : MSTF_IN, [nb] "s"(bm), [boff] "i"(BOFF)
+                     : MSTF_CLOBBER);
+    } else {
+        asm volatile(MSTF_GATHER
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0])
+                     : MSTF_IN
+                     : MSTF_CLOBBER);
+        nxt = mv;
+    }
+#undef MSTF_TILE
+#undef MSTF_GATHER
+#undef MSTF_IN
+#undef MSTF_CLOBBER
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(qm[m][0], qm[m][1]), acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(qm[m][2], qm[m][3]), acc[m], 0, 0, 0);
+        asm volatile("" : "+v"(acc[m]));  // pins the products here (see batch_step_exec)
+    }
+}
+
+// The kSubTiles tiles of one dequantised stage: bitmaps of the first batch requested and waited for here (the
+// dequantisation in front has lane-dependent branches, so nothing scalar is carried across it), the others one
+// batch ahead.  img: LDS address of the stage's image; wbase: LDS address of w[lane & 3][first tile of the stage].
+template <int NM>
+__device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t img, uint32_t zaddr, uint32_t wbase,
+                                               uint32_t wgroup, f4_t (&acc)[NM])
+{
+    constexpr int G = kSubTiles / 8;
+    u32x16_t cur;
+    asm volatile("s_load_dwordx16 %0, %1, 0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(cur) : "s"(bm) : "memory");
+    static_for<G>([&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        u32x16_t nxt;
+        batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 1024, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup, acc);
+        cur = nxt;
+    });
+}
+
 __device__ __forceinline__ u32x16_t load_bitmaps(const uint64_t* bm) { return *reinterpret_cast<const u32x16_a4*>(bm); }
 __device__ __forceinline__ u32x16_t prefetch_bitmaps(const uint64_t* bm)
 {

@@ -96,14 +96,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
                            lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, lane, mode);
         const uint64_t* bm = c.bmp + t_now;
         const uint32_t waddr = waddr_of(n);
-        u32x16_t cur = load_bitmaps(bm);
-#pragma unroll
-        for (int g = 0; g < kSubTiles / 8; g++) {
-            u32x16_t nxt = cur;
-            if (g + 1 < kSubTiles / 8) nxt = prefetch_bitmaps(bm + 8 * (g + 1));
-            batch_accumulate_img<NM>(cur, lbase + (uint32_t)g * 1024u, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
-            cur = nxt;
-        }
+        stage_img_exec<NM>(bm, lbase, zaddr, waddr, wgroup, acc);
         wait_lgkm0();  // every read of the image and of the staged buffers is done before they are rewritten
     }
 }
@@ -111,7 +104,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
 // ------------------------------------------------------------------------------- key
 // One wavefront per (KV head, token block); see key_spmv_kernel.
 template <int NW, int BIT>
-__global__ __launch_bounds__(256) void key_spmv_quant_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void key_spmv_quant_kernel(
     const uint64_t* __restrict__ bmp, const uint32_t* packed, const uint32_t* __restrict__ tile_off,
     const uint32_t* tile_off_dma, const uint16_t* scales, const uint16_t* zeros, const _Float16* Bm,
     _Float16* __restrict__ C, int Lc, int D, int nblk, int ntasks, int rows_per_kv, int row0, int mode)
