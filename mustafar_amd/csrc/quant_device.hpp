@@ -107,31 +107,9 @@ __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uin
     }
 }
 
-// Expands 8 tiles of the image and accumulates them (see batch_accumulate for the MFMA layout).
-//   mv   : the 8 bitmaps;  base0: LDS address of the first tile's image slots
-template <int NM>
-__device__ __forceinline__ void batch_accumulate_img(const u32x16_t& mv, uint32_t base0, uint32_t zaddr, uint32_t waddr,
-                                                     uint32_t wgroup, f4_t (&acc)[NM])
-{
-    uint32_t a[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) a[i] = tile_addr(u64_of(mv[2 * i], mv[2 * i + 1]), base0 + (uint32_t)i * 128u, zaddr);
-    _Float16 h[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
-    const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
-    const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
-#pragma unroll
-    for (int m = 0; m < NM; m++) {
-        const u32x4_t qm = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
-        const uint32_t q0 = qm[0], q1 = qm[1], q2 = qm[2], q3 = qm[3];
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(q0, q1), acc[m], 0, 0, 0);
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(q2, q3), acc[m], 0, 0, 0);
-    }
-}
-
-// The same with the gather under the tile's exec mask (see batch_step_exec in spmv_device.hpp): one statement per
-// batch of 8 tiles on fixed registers v112-v127; the image slots of tile i sit at img + IMG + 128 * i, so the tile's
+// Expands 8 tiles of the image and accumulates them, the gather under the tile's exec mask (see batch_step_exec in
+// spmv_device.hpp for the statement and the MFMA layout): one statement per batch of 8 tiles on fixed registers
+// v112-v127; the image slots of tile i sit at img + IMG + 128 * i, so the tile's
 // base is an immediate offset of the LDS read.  PREFETCH: the bitmaps of the coming batch (bm + BOFF bytes) are
 // requested first and completed by the statement's wait.
 template <int NM, bool PREFETCH, int BOFF, int IMG, int WOFF>
@@ -209,15 +187,6 @@ __device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t img,
         batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 1024, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup, acc);
         cur = nxt;
     });
-}
-
-__device__ __forceinline__ u32x16_t load_bitmaps(const uint64_t* bm) { return *reinterpret_cast<const u32x16_a4*>(bm); }
-__device__ __forceinline__ u32x16_t prefetch_bitmaps(const uint64_t* bm)
-{
-    __builtin_amdgcn_sched_barrier(0);
-    const u32x16_t v = load_bitmaps(bm);
-    __builtin_amdgcn_sched_barrier(0);
-    return v;
 }
 
 }  // namespace mstf

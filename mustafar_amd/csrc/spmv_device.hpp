@@ -38,54 +38,6 @@ __device__ __forceinline__ void dma4(const void* src, void* dst_wave_uniform)
     __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)src, (MSTF_LDS void*)dst_wave_uniform, 4, 0, 0);
 }
 
-// Streams `bytes` (a multiple of 16, <= kSubBytes) into LDS: piece i of lane l lands at dst + (i*64 + l)*16.
-// The lane's source address is formed once; the 1 KB pieces differ only in the instruction's immediate offset
-// (which moves the global and the LDS address alike).  Whole pieces need no lane predicate, only the last,
-// partial one does - so a sub-chunk costs two or three vector instructions besides the loads themselves.
-__device__ __forceinline__ void sub_issue(const char* src, uint32_t bytes, char* dst, int lane)
-{
-    const char* mine = src + (uint32_t)lane * 16u;
-    const uint32_t whole = bytes >> 10, rest = bytes & 1023u;  // wave-uniform
-#define MSTF_PIECE(I)                                                                                              \
-    if ((uint32_t)(I) < whole) {                                                                                   \
-        __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)mine, (MSTF_LDS void*)dst, 16, (I) * 1024, 0);  \
-    } else if ((uint32_t)(I) == whole && (uint32_t)lane * 16u < rest) {                                            \
-        __builtin_amdgcn_global_load_lds((MSTF_GLOBAL const void*)mine, (MSTF_LDS void*)dst, 16, (I) * 1024, 0);  \
-    }
-    static_assert(kSubBytes / 1024 == 4 || kSubBytes / 1024 == 2, "pieces per sub-chunk");
-    MSTF_PIECE(0)
-    MSTF_PIECE(1)
-    if (kSubBytes / 1024 == 4) {
-        MSTF_PIECE(2)
-        MSTF_PIECE(3)
-    }
-#undef MSTF_PIECE
-}
-
-// LDS byte address of D[t][lane] for one tile (the zero slot when the lane's element is absent).
-//   b     : tile bitmap, MSB-first (wave-uniform, scalar registers)
-//   base  : LDS byte address of the tile's values (wave-uniform, scalar: one s_lshl2_add on idx[t])
-// rank = popcount(mask below lane) comes from v_mbcnt.
-__device__ __forceinline__ uint32_t tile_addr(uint64_t b, uint32_t base, uint32_t zaddr)
-{
-    const uint64_t m = lanes_of(b);
-    return select_lane(m, rank_below(m) * 2u + base, zaddr);
-}
-// The same with the tile's base given as idx[t] (4-byte units) and the LDS address `rel` of unit 0:
-// base = (ov << 2) + rel is one scalar instruction (s_lshl2_add_u32; the compiler emits a shift and an add), and
-// it sits in one statement with its consumers so that no hazard no-op is placed behind it.  Every instruction of
-// the per-tile sequence costs the wavefront an issue slot, scalar ones included.
-__device__ __forceinline__ uint32_t tile_addr_idx(uint64_t b, uint32_t ov, uint32_t rel, uint32_t zaddr)
-{
-    const uint64_t m = lanes_of(b);
-    const uint32_t r = rank_below(m);
-    uint32_t a, t;
-    asm("s_lshl2_add_u32 %1, %3, %4\n\tv_lshl_add_u32 %0, %2, 1, %1\n\tv_cndmask_b32 %0, %5, %0, %6"
-        : "=&v"(a), "=&s"(t)
-        : "v"(r), "s"(ov), "s"(rel), "v"(zaddr), "s"(m)
-        : "scc");
-    return a;
-}
 // (16-bit LDS loads cannot merge into one register here: with SRAM ECC they clear the other half,
 // hence the explicit pack of two tiles into one fp16x2 register.)
 __device__ __forceinline__ uint32_t pack_h2(_Float16 lo, _Float16 hi)
@@ -101,55 +53,22 @@ struct Batch {
     u32x16_t mv;  // 8 bitmaps as (lo, hi) pairs
     u32x8_t ov;   // idx of the 8 tiles (4-byte units from the start of the KV head's values)
 };
-__device__ __forceinline__ Batch load_batch(const uint64_t* bm, const uint32_t* ix)
-{
-    Batch b;
-    b.mv = *reinterpret_cast<const u32x16_a4*>(bm);
-    b.ov = *reinterpret_cast<const u32x8_a4*>(ix);
-    return b;
-}
 
 // Decompresses 8 staged tiles and accumulates them.  For every group of 4 tiles the lane builds its own
 // four values D[t..t+3][lane] (A operand) and reads the four weights of "its" accumulator (lane & 3) of each
 // accumulator group from LDS (B operand); v_mfma_f32_4x4x4f16 then yields, in lane 4b+j, the sums of
 // positions 4b..4b+3 for accumulator 4m+j:
 //     acc[m][r] += sum_t D[t][4b + r] * w[4m + j][t]
-// Per tile the scalar unit spends one s_brev_b64, a shift and an add, the vector unit two v_mbcnt, one
-// v_lshl_add, one v_cndmask and half a v_perm.
 //   rel    : LDS byte address of the staged values minus 4 * idx of the first staged tile
-//   zaddr  : LDS address of two zero bytes
-//   waddr  : LDS byte address of w[lane & 3][first tile of the batch]; wgroup: bytes between groups of 4 rows
-template <int NM>
-__device__ __forceinline__ void batch_accumulate(const Batch& b, uint32_t rel, uint32_t zaddr, uint32_t waddr,
-                                                 uint32_t wgroup, f4_t (&acc)[NM])
-{
-    // the weights of the batch first: their LDS load then returns together with the gathers instead of costing a
-    // second round trip after them
-    u32x4_t qm[NM];
-#pragma unroll
-    for (int m = 0; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(waddr + (uint32_t)m * wgroup);
-    uint32_t a[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) a[i] = tile_addr_idx(u64_of(b.mv[2 * i], b.mv[2 * i + 1]), b.ov[i], rel, zaddr);
-    _Float16 h[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) h[i] = lds_load_h(a[i]);
-    const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
-    const uint32_t v2 = pack_h2(h[4], h[5]), v3 = pack_h2(h[6], h[7]);
-#pragma unroll
-    for (int m = 0; m < NM; m++) {
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(qm[m][0], qm[m][1]), acc[m], 0, 0, 0);
-        acc[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v2, v3), as_h4(qm[m][2], qm[m][3]), acc[m], 0, 0, 0);
-    }
-}
-
-// The same batch with the wavefront's exec mask set to each tile's bitmap in turn: only the lanes whose element is
+//   zaddr  : LDS address of 16 zero bytes
+//   wgroup : bytes between groups of 4 weight rows
+// The gather runs with the wavefront's exec mask set to each tile's bitmap in turn: only the lanes whose element is
 // present compute a rank and read LDS, the others keep the zero their destination was cleared to (four destinations
 // per 16-byte LDS read of the zero slot at zaddr; LDS reads of a wavefront return in order, so the gathers land on
 // top), so the select instruction disappears - per tile one s_brev_b64 into exec, two v_mbcnt on exec, the
-// scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (v112-v127, the top of the budget of a kernel that runs four wavefronts per SIMD, listed as
-// clobbered) because nothing of the compiler's may be scheduled while exec is partial; the wavefront must be in
-// uniform control flow with all 64 lanes active.  The scalar loads of the coming batch (PREFETCH) are part of the
+// scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (v112-v127, the top of the
+// budget of a kernel that runs four wavefronts per SIMD, listed as clobbered) because nothing of the compiler's may
+// be scheduled while exec is partial; the wavefront must be in uniform control flow with all 64 lanes active.  The scalar loads of the coming batch (PREFETCH) are part of the
 // statement: requested first, completed by its one wait - the compiler, which cannot see that wait, would otherwise
 // put one of its own in front of the statement and expose the round trip of a request it has just made.
 //   nbm + BOFF bytes, nix + IOFF bytes : bitmaps and offsets of the coming batch
@@ -245,38 +164,6 @@ __device__ __forceinline__ void static_for(F&& f)
 }
 
 
-// The next batch's scalar loads, requested a whole batch ahead and pinned where they are written: left to
-// itself the scheduler sinks them to their first use and every batch waits out an L2 round trip.
-__device__ __forceinline__ Batch prefetch_batch(const uint64_t* bm, const uint32_t* ix)
-{
-    __builtin_amdgcn_sched_barrier(0);
-    const Batch b = load_batch(bm, ix);
-    __builtin_amdgcn_sched_barrier(0);
-    return b;
-}
-
-// One staged sub-chunk (kSubTiles tiles).
-//   cur    : bitmaps and offsets of its first 8 tiles, already requested; on return those of the first 8 tiles at
-//            (bm_next, ix_next) - the coming sub-chunk - so that the chain of scalar requests, each one batch ahead,
-//            runs across sub-chunks
-//   bm, ix : the sub-chunk's bitmaps and tile offsets (wave-uniform pointers)
-//   buf    : LDS byte address of the staged values;  zaddr: LDS address of two zero bytes
-//   waddr  : LDS byte address of w[lane & 3][tile 0 of this sub-chunk]; wgroup: bytes between groups of 4 rows
-template <int NM>
-__device__ __forceinline__ void sub_accumulate(Batch& cur, const uint64_t* bm, const uint32_t* ix,
-                                               const uint64_t* bm_next, const uint32_t* ix_next, uint32_t buf,
-                                               uint32_t zaddr, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM])
-{
-    constexpr int G = kSubTiles / 8;
-    const uint32_t rel = buf - cur.ov[0] * 4u;
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        const Batch nxt = g + 1 < G ? prefetch_batch(bm + 8 * (g + 1), ix + 8 * (g + 1)) : prefetch_batch(bm_next, ix_next);
-        batch_accumulate<NM>(cur, rel, zaddr, waddr + (uint32_t)g * 16u, wgroup, acc);
-        cur = nxt;
-    }
-}
-
 __device__ __forceinline__ uint32_t sub_bytes(uint32_t start, uint32_t end)
 {
     const uint32_t b = (end - start) * 4u;
@@ -291,15 +178,6 @@ struct Touch {
     uint2 bm;
     uint32_t ix;
 };
-__device__ __forceinline__ Touch touch_sub(const uint64_t* bm, const uint32_t* ix, int lane)
-{
-    Touch t;
-    t.bm = make_uint2(0u, 0u);
-    t.ix = 0u;
-    if (lane < kSubTiles) t.bm = *reinterpret_cast<const uint2*>(bm + lane);
-    if (lane <= kSubTiles) t.ix = ix[lane];
-    return t;
-}
 // Waits for every outstanding vector-memory operation (LDS-direct loads included).
 __device__ __forceinline__ void wait_vm0_keep(Touch& t)
 {
