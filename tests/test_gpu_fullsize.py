@@ -183,3 +183,37 @@ def test_compress_twice_is_idempotent(data):
     assert torch.equal(a.packed().view(torch.int16), b.packed().view(torch.int16))
     pr = ops.prune_rows(K.view(-1, D), KTH).view(BKV, L, D)
     assert torch.equal(pr.view(torch.int16) & 0x7FFF, Kp.view(torch.int16) & 0x7FFF)   # magnitudes; pruned keep +-0
+
+
+def test_compress_from_projection_layout_full_size():
+    """Batch 8 x 4096 tokens x 8 KV heads straight from a projection-shaped buffer [8, 4096, 48 heads, 128] (keys
+    rotated in the kernel): the rotated rows equal the half-precision tensor expression evaluated by torch on the
+    device, and both sides' compressed arrays equal those of the contiguous route, bit for bit."""
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    bs, n_q, n_kv = 8, 32, 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(31)
+    qkv = torch.randn((bs, L, n_q + 2 * n_kv, D), generator=g, device=dev, dtype=torch.float32).half()
+    qkv[:, :, n_q + 3, 17] *= 12                        # an outlier channel in one key head
+    kx, vx = qkv[:, :, n_q:n_q + n_kv], qkv[:, :, n_q + n_kv:]
+    pos = torch.arange(L, device=dev, dtype=torch.float32)
+    inv = 1.0 / (500000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
+    ang = pos[:, None] * inv[None, :]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1).half(), torch.cat([ang.sin(), ang.sin()], -1).half()
+    kt = kx.transpose(1, 2)                             # [bs, n_kv, L, D]
+    k_ref = (kt * cos) + (torch.cat((-kt[..., D // 2:], kt[..., :D // 2]), dim=-1) * sin)
+    v_ref = vx.transpose(1, 2).contiguous()
+    Lc = L - 256
+    ck_ref = ops.compress(k_ref[:, :, :Lc].reshape(bs * n_kv, Lc, D), False, kth=KTH)
+    cv_ref = ops.compress(v_ref[:, :, :Lc].reshape(bs * n_kv, Lc, D), True, kth=KTH)
+    q_before = qkv[:, :, :n_q].clone()
+    ck, rot = ops.compress_proj(kx, False, KTH, Lc, cos, sin)          # rotates qkv's key heads in place
+    cv, _ = ops.compress_proj(vx, True, KTH, Lc)
+    assert rot.data_ptr() == kx.data_ptr()
+    assert torch.equal(kx.transpose(1, 2).contiguous().view(torch.int16), k_ref.contiguous().view(torch.int16))
+    assert torch.equal(qkv[:, :, :n_q], q_before) and torch.equal(vx.transpose(1, 2), v_ref)   # neighbours untouched
+    for a, b in ((ck, ck_ref), (cv, cv_ref)):
+        assert torch.equal(a.bmp, b.bmp) and torch.equal(a.idx, b.idx) and torch.equal(a.nz_off, b.nz_off)
+        assert int(a.total_halfs) == int(b.total_halfs)
+        assert torch.equal(a.nz.view(torch.int16), b.nz.view(torch.int16))
