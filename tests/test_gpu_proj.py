@@ -170,3 +170,80 @@ def test_proj_rejects_bad_arguments():
     app = L.mstf_append_proj_f16
     assert app(None, src(), 0, 64, 128, 89, a, a, None, a, a, a, a, 1 << 16) == -1
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_layouts_against_oracle(seed):
+    """Seeded random batch / heads / rows / M / strides (gaps between tokens, heads and batch entries, a non-zero
+    storage offset), keys with rotation and values without, all arrays bit-exact against the oracle."""
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(9000 + seed)
+    batch, heads = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+    nblk = int(rng.integers(1, 5))
+    M = 64 * nblk
+    rows = M + int(rng.integers(0, 130))
+    is_value = bool(seed & 1)
+    kth = int(rng.choice([0, 1, 64, 89, 115, 128])) if is_value else int(rng.choice([1, 64, 89, 115]))
+    K, V = orc.make_kv(400 + seed, batch * heads, rows, D)
+    src = V if is_value else K
+    if kth == 0:
+        src = orc.prune_rows(src, 96)
+    x = np.ascontiguousarray(src.reshape(batch, heads, rows, D).transpose(0, 2, 1, 3))
+    pad_h, pad_t, pad_b, lead = (8 * int(rng.integers(0, 5)) for _ in range(4))
+    row_len = heads * (D + pad_h) + pad_t
+    buf = torch.full((lead + batch * ((rows + 2) * row_len + pad_b),), float("nan"), dtype=torch.float16, device=dev)
+    xg = buf[lead:].as_strided((batch, rows, heads, D), ((rows + 2) * row_len + pad_b, row_len, D + pad_h, 1))
+    xg.copy_(torch.from_numpy(x))
+    before = buf.clone()
+    if is_value:
+        _, comp = oracle_side(x, M, kth, True)
+        c, _ = ops.compress_proj(xg, True, kth, M)
+        assert torch.equal(buf.view(torch.int16), before.view(torch.int16))          # the source is only read
+    else:
+        cos, sin = orc.rope_tables(np.arange(rows) + int(rng.integers(0, 8000)))
+        rot_ref, comp = oracle_side(x, M, kth, False, cos, sin)
+        c, r = ops.compress_proj(xg, False, kth, M, torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev))
+        assert np.array_equal(bits(r.cpu().numpy()), bits(rot_ref))
+        xg.copy_(torch.from_numpy(x))                                                 # undo the in-place rotation:
+        assert torch.equal(buf.view(torch.int16), before.view(torch.int16))          # nothing else was written
+    check_compressed(c, comp)
+
+
+def test_append_proj_overflow_is_flagged():
+    from mustafar_amd.cache import CompressedPool
+    dev = torch.device("cuda:0")
+    batch, heads, rows = 1, 3, 256
+    K, _ = orc.make_kv(9, batch * heads, rows, D)
+    x = torch.from_numpy(np.ascontiguousarray(K.reshape(batch, heads, rows, D).transpose(0, 2, 1, 3))).to(dev)
+    pool = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)    # 64 tokens fit, 256 do not
+    pool.append_proj(x[:, :64], 89, 64)
+    assert int(pool.overflow) == 0 and pool.tokens == 64
+    ref = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)
+    ref.append(x[:, :64].transpose(1, 2).reshape(heads, 64, D), 89)
+    assert torch.equal(pool.nz.view(torch.int16), ref.nz.view(torch.int16)) and torch.equal(pool.idx, ref.idx)
+    before = pool.nz.clone()
+    pool.append_proj(x[:, 64:], 89, 192)
+    assert int(pool.overflow) == 1
+    for b in range(heads):
+        n = 2 * int(pool.idx[b, 128])
+        s0 = 8 * int(pool.nz_off[b])
+        assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
+
+
+def test_short_prompt_through_prefill_proj_is_only_rotated():
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, L = 2, 2, 200                                # shorter than the residual length: nothing is compressed
+    K, V = orc.make_kv(77, bs * n_kv, L, D)
+    kx = np.ascontiguousarray(K.reshape(bs, n_kv, L, D).transpose(0, 2, 1, 3))
+    vx = np.ascontiguousarray(V.reshape(bs, n_kv, L, D).transpose(0, 2, 1, 3))
+    cos, sin = orc.rope_tables(np.arange(L))
+    k_rot, _ = oracle_side(kx, 0, 0, False, cos, sin)
+    for pooled in (False, True):
+        c = SparseKVCache(4, D, 0.7, 0.7, 256, fused=True, max_tokens=512 if pooled else 0, window_kernel=pooled)
+        Kr, Vr = c.prefill_proj(torch.from_numpy(kx).to(dev), torch.from_numpy(vx).to(dev), torch.from_numpy(cos).to(dev),
+                                torch.from_numpy(sin).to(dev))
+        assert c.compressed_length == 0 and c.kv_len == L and c.k is None
+        assert np.array_equal(bits(c.k_win.cpu().numpy()), bits(k_rot.transpose(0, 2, 1, 3)))
+        assert np.array_equal(bits(c.v_win.cpu().numpy()), bits(vx.transpose(0, 2, 1, 3)))
