@@ -32,16 +32,17 @@ def _convert(inputs, is_value, bit, kth=0):
     fn = L.mstf_compress_value_quant if is_value else L.mstf_compress_key_quant
     name = "mstf_compress_value_quant" if is_value else "mstf_compress_key_quant"
     st = torch.cuda.current_stream().cuda_stream
-    # worst case: every element kept -> T * (64 // capacity) words; sized exactly after the count phase
-    # (one host read of the total, as the reference's .item() does)
-    args = (x.data_ptr(), B, M, N, int(kth), int(bit), bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(),
-            units.data_ptr(), scales.data_ptr(), zeros.data_ptr(), total.data_ptr())
-    check(fn(st, *args, None, 0, ws.data_ptr(), ws.numel()), name)
+    # one pass with room for the worst case (every element kept: 64 // capacity words per tile), then the used
+    # part is copied out so that the large buffer goes back to the allocator; the total is read once on the host, as
+    # the reference's .item() does
+    cap_words = B * T * (64 * int(bit) // 32)
+    room = torch.empty((max(cap_words, 1),), dtype=torch.int32, device=dev)
+    check(fn(st, x.data_ptr(), B, M, N, int(kth), int(bit), bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(),
+             units.data_ptr(), scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,
+             ws.data_ptr(), ws.numel()), name)
     n = int(total.item())
-    packed = torch.zeros((max(n, 1),), dtype=torch.int32, device=dev)
-    if n > 0:
-        check(fn(st, *args, packed.data_ptr(), n, ws.data_ptr(), ws.numel()), name)
-    return bmp, tile_off, packed[:n] if n > 0 else packed[:0], counts, units, scales, zeros
+    packed = room[:n].clone()
+    return bmp, tile_off, packed, counts, units, scales, zeros
 
 
 def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2):

@@ -159,9 +159,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void pr
 
 // ------------------------------------------------------------------------------- scans
 // grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base, idx[b][T] = head total.
-// With nz_off given (the compress entry points) the workgroup also adds up the unit totals of all earlier heads:
-// nz_off[b] = that sum / 4 (16-byte units), and the last head's workgroup writes the grand total in fp16 values.
-// Every workgroup re-reads at most B * nblk small numbers, which spares a launch for the scan over heads.
+// With nz_off given (the compress entry points) the workgroup also adds up the unit totals of all earlier heads
+// (sum_before): nz_off[b] = that sum / 4 (16-byte units), and the last head's workgroup writes the grand total in
+// fp16 values.
 __global__ __launch_bounds__(256) void scan_units_kernel(const uint32_t* __restrict__ unit_tot,
                                                          uint32_t* __restrict__ unit_base, uint32_t* __restrict__ idx,
                                                          uint32_t* __restrict__ nz_off,
@@ -169,32 +169,14 @@ __global__ __launch_bounds__(256) void scan_units_kernel(const uint32_t* __restr
                                                          int tiles_per_unit)
 {
     extern __shared__ uint32_t base[];  // nblk entries
-    __shared__ uint64_t wsum[4];
     const int b = (int)blockIdx.x;
     const int tid = (int)threadIdx.x;
     const uint32_t total = units_scan(unit_tot + (size_t)b * nblk, base, nblk);
     for (int i = tid; i < nblk; i += 256) unit_base[(size_t)b * nblk + i] = base[i];
     if (tid == 0) idx[(size_t)b * ((size_t)nblk * tiles_per_unit + 1) + (size_t)nblk * tiles_per_unit] = total;
     if (nz_off) {
-        uint64_t mine = 0;
-        const size_t before = (size_t)b * nblk;
-        // 16-byte loads, four of them in flight per thread (unit_tot is 256-byte aligned)
-        const uint4* ut4 = reinterpret_cast<const uint4*>(unit_tot);
-        const size_t n4 = before / 4;
-        for (size_t i = tid; i < n4; i += 1024) {
-            uint4 v[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) v[u] = i + 256 * u < n4 ? ut4[i + 256 * u] : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-            for (int u = 0; u < 4; u++) mine += (uint64_t)v[u].x + v[u].y + v[u].z + v[u].w;
-        }
-        if (tid < (int)(before - 4 * n4)) mine += unit_tot[4 * n4 + tid];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
-        if ((tid & 63) == 0) wsum[tid >> 6] = mine;
-        __syncthreads();
+        const uint64_t pre = sum_before(unit_tot, (size_t)b * nblk);
         if (tid == 0) {
-            const uint64_t pre = wsum[0] + wsum[1] + wsum[2] + wsum[3];
             nz_off[b] = (uint32_t)(pre >> 2);
             if (b == (int)gridDim.x - 1) *total_halfs = 2ull * (pre + total);
         }

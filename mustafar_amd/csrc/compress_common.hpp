@@ -361,34 +361,6 @@ __device__ __forceinline__ void unit_keep(const uint32_t (&mag)[64], int kth, in
     }
 }
 
-// Exclusive scan of per-head totals over one workgroup of 1024 threads; out[b] = sum of earlier
-// totals >> shift, *total = (sum of all) * total_mul.
-__device__ __forceinline__ void heads_scan(const uint32_t* head_tot, uint32_t* out, uint64_t* total, int B, int shift,
-                                           uint64_t total_mul)
-{
-    __shared__ uint64_t wsum[16];
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int per = (B + 1023) / 1024;
-    const int i0 = tid * per;
-    uint64_t mine = 0;
-    for (int i = i0; i < i0 + per && i < B; i++) mine += head_tot[i];
-    uint64_t inc = mine;
-    for (int o = 1; o < 64; o <<= 1) {
-        uint64_t t = __shfl_up(inc, o, 64);
-        if (lane >= o) inc += t;
-    }
-    if (lane == 63) wsum[wave] = inc;
-    __syncthreads();
-    uint64_t pre = 0;
-    for (int w = 0; w < wave; w++) pre += wsum[w];
-    uint64_t run = pre + inc - mine;
-    for (int i = i0; i < i0 + per && i < B; i++) {
-        out[i] = (uint32_t)(run >> shift);
-        run += head_tot[i];
-    }
-    if (tid == 1023) *total = total_mul * run;
-}
-
 // Exclusive scan of one head's unit totals (grid.x = head, 256 threads) into LDS `base`
 // (nblk entries); returns the head total to every thread.
 __device__ __forceinline__ uint32_t units_scan(const uint32_t* ut, uint32_t* base, int nblk)
@@ -411,6 +383,31 @@ __device__ __forceinline__ uint32_t units_scan(const uint32_t* ut, uint32_t* bas
     }
     __syncthreads();
     return carry;
+}
+
+// Sum of the `before` words in front of a head's unit totals, over one workgroup of 256 threads (16-byte loads,
+// four in flight per thread; ut is 256-byte aligned); the result is valid in thread 0.  Every workgroup re-reads
+// at most B * nblk small numbers, which spares a launch for the scan over heads.
+__device__ __forceinline__ uint64_t sum_before(const uint32_t* ut, size_t before)
+{
+    __shared__ uint64_t wsum[4];
+    const int tid = (int)threadIdx.x;
+    uint64_t mine = 0;
+    const uint4* ut4 = reinterpret_cast<const uint4*>(ut);
+    const size_t n4 = before / 4;
+    for (size_t i = tid; i < n4; i += 1024) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = i + 256 * u < n4 ? ut4[i + 256 * u] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int u = 0; u < 4; u++) mine += (uint64_t)v[u].x + v[u].y + v[u].z + v[u].w;
+    }
+    if (tid < (int)(before - 4 * n4)) mine += ut[4 * n4 + tid];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+    if ((tid & 63) == 0) wsum[tid >> 6] = mine;
+    __syncthreads();
+    return wsum[0] + wsum[1] + wsum[2] + wsum[3];
 }
 
 }  // namespace mstf

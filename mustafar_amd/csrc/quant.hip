@@ -87,26 +87,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void qu
     if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
 }
 
-// grid = B, 256 threads: unit totals -> unit bases (in place), head_tot[b].
-__global__ __launch_bounds__(256) void quant_scan_units_kernel(uint32_t* __restrict__ unit_tot,
-                                                               uint32_t* __restrict__ head_tot, int nblk)
+// grid = B, 256 threads: exclusive scan of the head's unit totals into unit_base; head_base[b] = words of all earlier
+// heads (summed from their unit totals, which spares a launch for a scan over heads); the last head's workgroup
+// writes the grand total.
+__global__ __launch_bounds__(256) void quant_scan_kernel(const uint32_t* __restrict__ unit_tot,
+                                                         uint32_t* __restrict__ unit_base,
+                                                         uint32_t* __restrict__ head_base,
+                                                         uint64_t* __restrict__ total_words, int nblk)
 {
     extern __shared__ uint32_t base[];
     const int b = (int)blockIdx.x;
-    uint32_t* ut = unit_tot + (size_t)b * nblk;
-    const uint32_t total = units_scan(ut, base, nblk);
-    for (int i = (int)threadIdx.x; i < nblk; i += 256) ut[i] = base[i];
-    if (threadIdx.x == 0) head_tot[b] = total;
+    const uint32_t total = units_scan(unit_tot + (size_t)b * nblk, base, nblk);
+    for (int i = (int)threadIdx.x; i < nblk; i += 256) unit_base[(size_t)b * nblk + i] = base[i];
+    const uint64_t pre = sum_before(unit_tot, (size_t)b * nblk);
+    if (threadIdx.x == 0) {
+        head_base[b] = (uint32_t)pre;
+        if (b == (int)gridDim.x - 1) *total_words = pre + total;
+    }
 }
 
-__global__ __launch_bounds__(1024) void quant_scan_heads_kernel(const uint32_t* __restrict__ head_tot,
-                                                                uint32_t* __restrict__ head_base,
-                                                                uint64_t* __restrict__ total_words, int B)
-{
-    heads_scan(head_tot, head_base, total_words, B, 0, 1ull);
-}
-
-// tile_off[b][t] += head base + unit base  (global word offsets, as the reference returns them)
+// tile_off[b][t] += head base + unit base  (global word offsets, as the reference returns them); only when no pack
+// follows, which does it itself.
 __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restrict__ tile_off,
                                                              const uint32_t* __restrict__ unit_base,
                                                              const uint32_t* __restrict__ head_base, int nblk, size_t T)
@@ -118,12 +119,14 @@ __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restric
 }
 
 // ------------------------------------------------------------------------------- producer: pack
-// grid = B * M/64 units, 64 threads; every lane quantises and packs its two tiles.
+// grid = B * M/64 units, 64 threads; every lane quantises and packs its two tiles.  tile_off still holds the
+// unit-local offsets of the count kernel and is completed here with the unit's and the head's base.
 template <bool IS_VALUE>
 __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restrict__ x, int M, int bit,
                                                         const uint64_t* __restrict__ bmp,
-                                                        const uint32_t* __restrict__ units,
-                                                        const uint32_t* __restrict__ tile_off,
+                                                        const uint32_t* __restrict__ units, uint32_t* tile_off,
+                                                        const uint32_t* __restrict__ unit_base,
+                                                        const uint32_t* __restrict__ head_base,
                                                         const _Float16* __restrict__ scales,
                                                         const _Float16* __restrict__ zeros,
                                                         uint32_t* __restrict__ packed, uint64_t capacity_words)
@@ -137,6 +140,7 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
     const float maxq = (float)((1 << bit) - 1);
     const size_t tile0 = (size_t)b * T + (size_t)tb * kD;
+    const uint32_t ubase = head_base[b] + unit_base[(size_t)b * nblk + tb];
 #pragma unroll 1
     for (int h = 0; h < 2; h++) {
         __builtin_amdgcn_wave_barrier();
@@ -144,7 +148,8 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
         __builtin_amdgcn_wave_barrier();
         const size_t ti = tile0 + (size_t)h * 64 + lane;
         const uint64_t m = bmp[ti];
-        const uint64_t off = tile_off[ti];
+        const uint64_t off = (uint64_t)tile_off[ti] + ubase;
+        tile_off[ti] = (uint32_t)off;
         if (off + units[ti] > capacity_words) continue;  // would not fit: leave untouched
         float sc = (float)scales[ti];
         const float zp = (float)zeros[ti];
@@ -181,9 +186,10 @@ static int cap_shift_of(int bit)
     }
 }
 
+// workspace: unit totals, unit bases (both [B][M/64]) and the head bases [B]
 static size_t quant_ws_bytes(int B, int M)
 {
-    return round_up((size_t)B * (M / 64) * 4, 256) + 2 * round_up((size_t)B * 4, 256);
+    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
 }
 
 template <bool IS_VALUE>
@@ -206,29 +212,28 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     const int nblk = M / 64;
     const size_t T = (size_t)M * kD / 64;
     char* w = reinterpret_cast<char*>(ws);
+    const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(w);
-    uint32_t* head_tot = reinterpret_cast<uint32_t*>(w + round_up((size_t)B * nblk * 4, 256));
-    uint32_t* head_base = reinterpret_cast<uint32_t*>(w + round_up((size_t)B * nblk * 4, 256) + round_up((size_t)B * 4, 256));
+    uint32_t* unit_base = reinterpret_cast<uint32_t*>(w + ub);
+    uint32_t* head_base = reinterpret_cast<uint32_t*>(w + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     int rc;
     hipLaunchKernelGGL(quant_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bit, bmp,
                        counts, units, tile_off, reinterpret_cast<_Float16*>(scales), reinterpret_cast<_Float16*>(zeros),
                        unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(quant_scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, head_tot,
-                       nblk);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(quant_scan_heads_kernel, dim3(1), dim3(1024), 0, st, head_tot, head_base, total_words, B);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(quant_finalize_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)B), dim3(256), 0, st, tile_off,
-                       unit_tot, head_base, nblk, T);
+    hipLaunchKernelGGL(quant_scan_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base,
+                       head_base, total_words, nblk);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     if (packed) {
         hipLaunchKernelGGL(quant_pack_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bit, bmp,
-                           units, tile_off, reinterpret_cast<const _Float16*>(scales),
+                           units, tile_off, unit_base, head_base, reinterpret_cast<const _Float16*>(scales),
                            reinterpret_cast<const _Float16*>(zeros), packed, cap_words);
-        if ((rc = check_launch()) != MSTF_OK) return rc;
+    } else {
+        hipLaunchKernelGGL(quant_finalize_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)B), dim3(256), 0, st,
+                           tile_off, unit_base, head_base, nblk, T);
     }
+    if ((rc = check_launch()) != MSTF_OK) return rc;
     return MSTF_OK;
 }
 
