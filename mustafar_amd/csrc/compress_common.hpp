@@ -330,12 +330,13 @@ __device__ __forceinline__ uint32_t threshold_of(const uint32_t (&mag)[64], int 
 // Threshold and tile bitmaps of one unit in one go (see unit_bitmaps for the meaning of bmA / bmB).  With pruning
 // (kth > 0) the bitmaps come from the select's own keep masks, so the magnitudes are dead once the bit planes exist:
 // value tiles spread the masks into channel order, key tiles take one ballot per channel over the lanes' mask bits.
+// Returns the row's threshold: an element is kept <=> its magnitude is >= the returned value (>= 1: zeros never are).
 template <bool IS_VALUE>
-__device__ __forceinline__ void unit_keep(const uint32_t (&mag)[64], int kth, int lane, uint64_t& bmA, uint64_t& bmB)
+__device__ __forceinline__ uint32_t unit_keep(const uint32_t (&mag)[64], int kth, int lane, uint64_t& bmA, uint64_t& bmB)
 {
     if (kth > 0) {
         uint32_t kept[4];
-        select_kth_planes<true>(mag, kth, kept);
+        const uint32_t thr = select_kth_planes<true>(mag, kth, kept);
         if (IS_VALUE) {
             bmA = spread_bitmap(kept[0], kept[1]);
             bmB = spread_bitmap(kept[2], kept[3]);
@@ -356,9 +357,10 @@ __device__ __forceinline__ void unit_keep(const uint32_t (&mag)[64], int kth, in
             bmA = u64_of(aLo, aHi);
             bmB = u64_of(bLo, bHi);
         }
-    } else {
-        unit_bitmaps<IS_VALUE>(mag, 1u, lane, bmA, bmB);
+        return thr == 0u ? 1u : thr;
     }
+    unit_bitmaps<IS_VALUE>(mag, 1u, lane, bmA, bmB);
+    return 1u;
 }
 
 // Exclusive scan of one head's unit totals (grid.x = head, 256 threads) into LDS `base`

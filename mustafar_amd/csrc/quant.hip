@@ -35,11 +35,21 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void qu
     unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, slab, lane, r);
 
     uint64_t bm[2];
+    uint32_t thr;
     {
         uint32_t mag[64];
 #pragma unroll
         for (int j = 0; j < 64; j++) mag[j] = r[j] & 0x7FFF7FFFu;
-        unit_keep<IS_VALUE>(mag, kth, lane, bm[0], bm[1]);
+        thr = unit_keep<IS_VALUE>(mag, kth, lane, bm[0], bm[1]);
+    }
+    // The pruned elements become NaN (exponent and mantissa all ones under the element's own sign), which the
+    // minimum / maximum instructions pass over: no per-element test of the bitmap is needed afterwards.
+    typedef short s2_t __attribute__((ext_vector_type(2)));
+    const us2_t t2 = as_us2(thr | (thr << 16));
+#pragma unroll
+    for (int j = 0; j < 64; j++) {
+        const s2_t d = __builtin_bit_cast(s2_t, (us2_t)(as_us2(r[j] & 0x7FFF7FFFu) - t2));   // < 0 <=> pruned
+        r[j] |= __builtin_bit_cast(uint32_t, (s2_t)(d >> 15)) & 0x7FFF7FFFu;
     }
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
     const int cap = 32 / bit;
@@ -48,22 +58,33 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void qu
     uint32_t u[2];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        // the half-slab of channels 64h.. back into LDS, so that lane = tile can walk its 64 elements:
-        // key -> (token i, channel 64h + lane); value -> (token lane, channel 64h + i)
-#pragma unroll
-        for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
-        __builtin_amdgcn_wave_barrier();
         float mn = INFINITY, mx = -INFINITY;
         const uint64_t m = bm[h];
-        for (int i = 0; i < 64; i++) {
-            const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
-            const float v = (float)sh[e];
-            if ((m >> (63 - i)) & 1ull) {
+        if (IS_VALUE) {
+            // tile (h, token = lane): the lane's own 64 channels, two per register
+            typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
+            h2v_t mn2 = {(_Float16)INFINITY, (_Float16)INFINITY}, mx2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+#pragma unroll
+            for (int j = 0; j < 32; j++) {
+                const h2v_t v = __builtin_bit_cast(h2v_t, r[32 * h + j]);
+                mn2 = __builtin_elementwise_min(mn2, v);
+                mx2 = __builtin_elementwise_max(mx2, v);
+            }
+            mn = fminf((float)mn2[0], (float)mn2[1]);
+            mx = fmaxf((float)mx2[0], (float)mx2[1]);
+        } else {
+            // tile = channel 64h + lane over the 64 tokens: the half-slab back into LDS, the lane walks its column
+#pragma unroll
+            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll 8
+            for (int i = 0; i < 64; i++) {
+                const float v = (float)sh[i * (2 * kHalfRowDw) + lane];
                 mn = fminf(mn, v);
                 mx = fmaxf(mx, v);
             }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
         const uint32_t cnt = (uint32_t)__popcll(m);
         float scale = 1.f, zero = 0.f;
         if (cnt > 0) {
