@@ -178,8 +178,11 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
         uint32_t cur = 0;
         int pos = 0;
         uint32_t w = 0;
-        for (int i = 0; i < 64; i++) {
-            if (!((m >> (63 - i)) & 1ull)) continue;
+        // only the kept elements, first to last: the wavefront loops as often as its fullest tile has non-zeros
+        // (about half of 64 at 70 % sparsity), and every round carries a division
+        for (uint64_t rem = m; rem != 0ull;) {
+            const int i = __builtin_clzll(rem);
+            rem &= ~(0x8000000000000000ull >> i);
             const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
             const float v = (float)sh[e];
             float q = floorf(v / sc + 0.5f) + zp;
