@@ -346,6 +346,15 @@ class QuantSparseKVCache(SparseKVCache):
         return mpq.decode_attention_window_quant(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1],
                                                  self.groups, self.bit, self.dequant_mode, win_len_dev=self._wlen_dev)
 
+    def prefill_proj(self, kx, vx, cos, sin):
+        """As SparseKVCache.prefill_proj for the rotation - the keys are rotated in place by the compressor's kernel,
+        in the projection's own layout - while the quantised producer, which takes contiguous rows like the
+        reference's, goes through prefill on the transposed views."""
+        ops.compress_proj(kx, False, self.kth_k, 0, cos, sin)      # M = 0: rotation only
+        K, V = kx.transpose(1, 2), vx.transpose(1, 2)
+        self.prefill(K, V)
+        return K, V
+
     def _compress(self, K, V):
         from . import compression_quant as cq
         bs, n_kv, M, D = K.shape

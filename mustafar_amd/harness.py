@@ -95,8 +95,9 @@ def _rope(x, tables):
 class Decoder:
     def __init__(self, cfg, device, seed=0, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=0,
                  proj_prefill=True):
-        """proj_prefill: the fp16 sparse cache takes the keys and values of the prompt straight from the projection
-        output (keys rotated by the compressor's own kernel, no transposed or contiguous copies)."""
+        """proj_prefill: the sparse caches take the keys and values of the prompt straight from the projection output
+        (keys rotated by the compressor's own kernel; the fp16 cache also compresses them where they lie, without
+        transposed or contiguous copies)."""
         self.cfg, self.dev = cfg, device
         self.proj_prefill = proj_prefill
         g = torch.Generator(device=device)
@@ -172,7 +173,7 @@ class Decoder:
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            if self.proj_prefill and type(cache) is SparseKVCache:
+            if self.proj_prefill and isinstance(cache, SparseKVCache):
                 qkv = F.linear(h, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim)
                 q = _rope(qkv[:, :, : c.n_q].transpose(1, 2), tables)
                 k, v = cache.prefill_proj(qkv[:, :, c.n_q: c.n_q + c.n_kv], qkv[:, :, c.n_q + c.n_kv:], tables[0], usin)
@@ -184,7 +185,7 @@ class Decoder:
                 outs.append(F.scaled_dot_product_attention(q[b0:b0 + seq_chunk], k[b0:b0 + seq_chunk], v[b0:b0 + seq_chunk],
                                                            is_causal=True, enable_gqa=True))
             a = torch.cat(outs, 0).transpose(1, 2).reshape(bs, L, c.n_q * c.head_dim)
-            if not (self.proj_prefill and type(cache) is SparseKVCache):
+            if not (self.proj_prefill and isinstance(cache, SparseKVCache)):
                 cache.prefill(k, v)
             x = x + F.linear(a, lw["o"])
             h = _rms_norm(x, lw["ln2"], c.rms_eps)

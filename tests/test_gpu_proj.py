@@ -247,3 +247,28 @@ def test_short_prompt_through_prefill_proj_is_only_rotated():
         assert c.compressed_length == 0 and c.kv_len == L and c.k is None
         assert np.array_equal(bits(c.k_win.cpu().numpy()), bits(k_rot.transpose(0, 2, 1, 3)))
         assert np.array_equal(bits(c.v_win.cpu().numpy()), bits(vx.transpose(0, 2, 1, 3)))
+
+
+def test_quantised_cache_prefill_from_projection():
+    """QuantSparseKVCache.prefill_proj (rotation by the kernel, quantised producer on the transposed views) against
+    prefill on the rotated tensors: identical lists, identical window."""
+    from mustafar_amd.cache import QuantSparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, L = 2, 2, 600
+    K, V = orc.make_kv(321, bs * n_kv, L, D)
+    kx = np.ascontiguousarray(K.reshape(bs, n_kv, L, D).transpose(0, 2, 1, 3))
+    vx = np.ascontiguousarray(V.reshape(bs, n_kv, L, D).transpose(0, 2, 1, 3))
+    cos, sin = orc.rope_tables(np.arange(L))
+    k_rot, _ = oracle_side(kx, 0, 0, False, cos, sin)
+    a = QuantSparseKVCache(4, D, 0.7, 0.7, 256, bit=2, fused=True, window_kernel=True)
+    a.prefill(torch.from_numpy(k_rot).to(dev).transpose(1, 2), torch.from_numpy(vx).to(dev).transpose(1, 2))
+    b = QuantSparseKVCache(4, D, 0.7, 0.7, 256, bit=2, fused=True, window_kernel=True)
+    b.prefill_proj(torch.from_numpy(kx).to(dev), torch.from_numpy(vx).to(dev), torch.from_numpy(cos).to(dev),
+                   torch.from_numpy(sin).to(dev))
+    assert a.compressed_length == b.compressed_length == 256
+    for sa, sb in ((a.k, b.k), (a.v, b.v)):
+        assert len(sa) == len(sb)
+        for ta, tb in zip(sa, sb):
+            assert torch.equal(ta.view(torch.uint8), tb.view(torch.uint8))
+    assert torch.equal(a.k_win.view(torch.int16), b.k_win.view(torch.int16))
+    assert torch.equal(a.v_win.view(torch.int16), b.v_win.view(torch.int16))
