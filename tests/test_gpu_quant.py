@@ -282,3 +282,37 @@ def test_quant_decode_attention_with_dense_window(bit, groups, Bkv, Lc, Lw):
     wl = torch.tensor([Lw], dtype=torch.int32, device=dev())
     o_dev = mpq.decode_attention_window_quant(kq, vq, to_gpu(q), kw, vw, cap, groups, bit, win_len_dev=wl)
     assert torch.equal(o_dev, o)
+
+
+@pytest.mark.parametrize("B,M,is_value", [(301, 128, 0), (77, 192, 1)])
+def test_quant_compress_many_heads_and_sizing_only(B, M, is_value):
+    """Hundreds of heads (the scan sums the unit totals of all earlier heads with vector loads and a tail) against
+    the oracle, and the sizing-only call (packed == NULL), which must leave the same final tile offsets and total."""
+    from mustafar_amd import compression_quant as cq, ops
+    from mustafar_amd._lib import lib
+    K, V = orc.make_kv(B + M, B, M)
+    x = orc.prune_rows(V if is_value else K, 89)
+    ref = orc.compress_quant(x, is_value, 2)
+    fn = cq.convert_value_batched_quant if is_value else cq.convert_key_batched_quant
+    got = fn(to_gpu(x), bit=2) if is_value else fn(to_gpu(x), return_metadata=True, bit=2)
+    assert np.array_equal(got[0].cpu().numpy(), ref[0])
+    assert np.array_equal(got[1].cpu().numpy(), ref[1].astype(np.int32))
+    assert np.array_equal(got[2].cpu().numpy(), ref[2])
+    # sizing only
+    L = lib()
+    xg = to_gpu(x)
+    T = M * 128 // 64
+    d = dev()
+    bmp = torch.empty((B, T), dtype=torch.int64, device=d)
+    toff = torch.empty((B, T), dtype=torch.int32, device=d)
+    cnt, uni = torch.empty_like(toff), torch.empty_like(toff)
+    sc = torch.empty((B, T), dtype=torch.float16, device=d)
+    zp = torch.empty_like(sc)
+    total = torch.zeros(1, dtype=torch.int64, device=d)
+    ws = ops.workspace(d, L.mstf_compress_quant_workspace_bytes(B, M, 128))
+    f = L.mstf_compress_value_quant if is_value else L.mstf_compress_key_quant
+    rc = f(torch.cuda.current_stream().cuda_stream, xg.data_ptr(), B, M, 128, 0, 2, bmp.data_ptr(), toff.data_ptr(),
+           cnt.data_ptr(), uni.data_ptr(), sc.data_ptr(), zp.data_ptr(), total.data_ptr(), None, 0, ws.data_ptr(), ws.numel())
+    assert rc == 0
+    assert int(total.item()) == ref[2].size
+    assert np.array_equal(toff.cpu().numpy(), ref[1].astype(np.int32))
