@@ -92,27 +92,25 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             if (n == kKeySubs + kValSubs - 1) return endV;
             return start_of(n + 1);
         };
+        const MetaLane metaK = meta_lane(K.off_dma, K.scales, K.zeros, lane);
+        const MetaLane metaV = meta_lane(V.off_dma, V.scales, V.zeros, lane);
+        const uint32_t lane4 = (uint32_t)lane * 4u;
+        const uint32_t touch8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
+        const uint32_t wordbuf_lds = lds_addr(wordbuf);
+        // (no lane-dependent branches: every piece is issued with exec set by hand or from a clamped address)
         auto issue = [&](int n) {
             const QSide& S = n < kKeySubs ? K : V;
+            const MetaLane& ML = n < kKeySubs ? metaK : metaV;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             const uint32_t s = start_of(n);
             uint32_t nw = end_of(n) - s;
             nw = nw > (uint32_t)F::kWordsMax ? (uint32_t)F::kWordsMax : nw;  // never true for a well-formed cache
-            char* wb = wordbuf + (n & 1) * F::kWordBuf;
-#pragma unroll
-            for (int i = 0; i < F::kWordsMax / 64; i++) {
-                const uint32_t o = (uint32_t)(i * 64 + lane);
-                if (o < nw) dma4(S.packed + s + o, wb + i * 256);
-            }
+            words_issue_flat<F::kWordsMax / 64>(S.packed + s, nw, wordbuf_lds + (uint32_t)(n & 1) * F::kWordBuf,
+                                                (uint32_t)lane, lane4);
             // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane)
-            const void* src = lane < 32 ? (const void*)(S.off_dma + t + lane)
-                                        : lane < 48 ? (const void*)(reinterpret_cast<const uint32_t*>(S.scales + t) + (lane - 32))
-                                                    : (const void*)(reinterpret_cast<const uint32_t*>(S.zeros + t) + (lane - 48));
-            dma4(src, metabuf + (n & 1) * kMetaBytes);
+            dma4(ML.at((uint32_t)t), metabuf + (n & 1) * kMetaBytes);
             // pulls the stage's bitmaps into L2 ahead of the scalar loads of the expansion
-            uint2 b = make_uint2(0u, 0u);
-            if (lane < kSubTiles) b = *reinterpret_cast<const uint2*>(S.bmp + t + lane);
-            return b;
+            return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(S.bmp + t) + touch8);
         };
 
         // the query rows of this KV head: groups x D fp16, contiguous

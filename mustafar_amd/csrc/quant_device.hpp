@@ -107,6 +107,57 @@ __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uin
     }
 }
 
+// LDS-direct loads of a stage's packed words without control flow (see sub_issue_flat in spmv_device.hpp): piece i
+// of lane l is word 64 * i + l of src, issued for the lanes with 64 * i + l < nw by setting exec by hand; the
+// wavefront must have all 64 lanes active.  dst_lds: LDS byte address of the word buffer; lane4 = lane * 4.
+template <int PIECES>
+__device__ __forceinline__ void words_issue_flat(const uint32_t* src, uint32_t nw, uint32_t dst_lds, uint32_t lane,
+                                                 uint32_t lane4)
+{
+    static_assert(PIECES == 2 || PIECES == 4 || PIECES == 8, "pieces of 64 words");
+    uint32_t t, m0_kept;
+#define MSTF_WPIECE(I)                                                     \
+    "s_sub_i32 %[t], %[n], " #I " * 64\n\t"                                \
+    "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"                                     \
+    "s_mov_b64 exec, vcc\n\t"                                              \
+    "global_load_lds_dword %[l4], %[src] offset:" #I " * 256\n\t"
+#define MSTF_WHEAD "s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[dst]\n\t"
+#define MSTF_WTAIL "s_mov_b64 exec, -1\n\ts_mov_b32 m0, %[keep]"
+#define MSTF_WOPS                                                                                      \
+    : [t] "=&s"(t), [keep] "=&s"(m0_kept)                                                              \
+    : [dst] "s"(dst_lds), [n] "s"(nw), [l] "v"(lane), [l4] "v"(lane4), [src] "s"(src)                  \
+    : "vcc", "scc", "memory"
+    if constexpr (PIECES == 2)
+        asm volatile(MSTF_WHEAD MSTF_WPIECE(0) MSTF_WPIECE(1) MSTF_WTAIL MSTF_WOPS);
+    else if constexpr (PIECES == 4)
+        asm volatile(MSTF_WHEAD MSTF_WPIECE(0) MSTF_WPIECE(1) MSTF_WPIECE(2) MSTF_WPIECE(3) MSTF_WTAIL MSTF_WOPS);
+    else
+        asm volatile(MSTF_WHEAD MSTF_WPIECE(0) MSTF_WPIECE(1) MSTF_WPIECE(2) MSTF_WPIECE(3) MSTF_WPIECE(4)
+                         MSTF_WPIECE(5) MSTF_WPIECE(6) MSTF_WPIECE(7) MSTF_WTAIL MSTF_WOPS);
+#undef MSTF_WPIECE
+#undef MSTF_WHEAD
+#undef MSTF_WTAIL
+#undef MSTF_WOPS
+}
+
+// Where a lane fetches its 4 bytes of a stage's metadata from (lanes 0..31 the word offsets of the 32 tiles, 32..47
+// the scales, 48..63 the zero-points, two per lane): the address for tile 0 and the shift that turns a tile index
+// into the lane's byte offset, formed once, so that a stage needs one shift and one 64-bit add.
+struct MetaLane {
+    const char* p0;
+    uint32_t shift;
+    __device__ __forceinline__ const void* at(uint32_t t) const { return p0 + ((size_t)t << shift); }
+};
+__device__ __forceinline__ MetaLane meta_lane(const uint32_t* off_dma, const uint16_t* scales, const uint16_t* zeros, int lane)
+{
+    MetaLane m;
+    m.p0 = lane < 32 ? reinterpret_cast<const char*>(off_dma + lane)
+                     : lane < 48 ? reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(scales) + (lane - 32))
+                                 : reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(zeros) + (lane - 48));
+    m.shift = lane < 32 ? 2u : 1u;
+    return m;
+}
+
 // Expands 8 tiles of the image and accumulates them, the gather under the tile's exec mask (see batch_step_exec in
 // spmv_device.hpp for the statement and the MFMA layout): one statement per batch of 8 tiles on fixed registers
 // v112-v127; the image slots of tile i sit at img + IMG + 128 * i, so the tile's

@@ -53,25 +53,22 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
         const uint32_t cnt = (uint32_t)__builtin_popcountll(c.bmp[t + kSubTiles - 1]);
         e = c.off[t + kSubTiles - 1] + ((cnt + (uint32_t)F::kCap - 1u) >> F::kCapShift);
     };
+    const MetaLane meta = meta_lane(c.off_dma, c.scales, c.zeros, lane);
+    const uint32_t lane4 = (uint32_t)lane * 4u;
+    const uint32_t touch8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
+    const uint32_t wordbuf_lds = lds_addr(wordbuf);
+    auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+    // (no lane-dependent branches in the word and metadata loads: exec set by hand, clamped touch address)
     auto issue = [&](int n, size_t t, uint32_t s, uint32_t e) {
-        uint32_t nw = e - s;
+        uint32_t nw = uni(e) - uni(s);
         nw = nw > (uint32_t)F::kWordsMax ? (uint32_t)F::kWordsMax : nw;  // never true for a well-formed cache
-        char* wb = wordbuf + (n & 1) * F::kWordBuf;
-#pragma unroll
-        for (int i = 0; i < F::kWordsMax / 64; i++) {
-            const uint32_t o = (uint32_t)(i * 64 + lane);
-            if (o < nw) dma4(c.packed + s + o, wb + i * 256);
-        }
+        words_issue_flat<F::kWordsMax / 64>(c.packed + uni(s), nw, wordbuf_lds + (uint32_t)(n & 1) * F::kWordBuf,
+                                            (uint32_t)lane, lane4);
         // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane)
-        const void* src = lane < 32 ? (const void*)(c.off_dma + t + lane)
-                                    : lane < 48 ? (const void*)(reinterpret_cast<const uint32_t*>(c.scales + t) + (lane - 32))
-                                                : (const void*)(reinterpret_cast<const uint32_t*>(c.zeros + t) + (lane - 48));
-        dma4(src, metabuf + (n & 1) * kMetaBytes);
+        dma4(meta.at((uint32_t)t), metabuf + (n & 1) * kMetaBytes);
         stage_w(n);
         // pulls the stage's bitmaps into L2 ahead of the scalar loads of the expansion
-        uint2 b = make_uint2(0u, 0u);
-        if (lane < kSubTiles) b = *reinterpret_cast<const uint2*>(c.bmp + t + lane);
-        return b;
+        return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(c.bmp + t) + touch8);
     };
 
     size_t t_cur = tile_of(0);
