@@ -61,6 +61,13 @@ def test_argument_validation_returns_before_any_launch(lib):
     assert L.mstf_compress_key_f16(None, None, 1, 64, 128, 0, None, None, None, None, None, 0, None, 0) == -1
     assert L.mstf_compress_value_quant(None, None, 1, 64, 128, 0, 2, None, None, None, None, None, None, None, None, 0,
                                        None, 0) == -1
+    src = _lib.ProjSource()                                   # all zero: no source pointer
+    assert L.mstf_compress_proj_f16(None, None, 0, 64, 128, 89, None, None, None, None, None, 0, None, 0) == -1
+    assert L.mstf_compress_proj_f16(None, ctypes.byref(src), 0, 64, 128, 89, None, None, None, None, None, 0, None, 0) == -1
+    assert L.mstf_append_proj_f16(None, ctypes.byref(src), 1, 64, 128, 89, None, None, None, None, None, None, None, 0) == -1
+    assert L.mstf_decode_attention_f16(None, *([None] * 11), 64, 128, 4, 4, None, 0) == -1
+    assert L.mstf_decode_attention_splits(4096, 128, 256, 4) == 8
+    assert L.mstf_decode_attention_splits(4096, 128, 1024, 4) == 2       # 16384 blocks: four per wavefront
     # workspace sizes are pure host arithmetic
     assert L.mstf_compress_workspace_bytes(64, 4096, 128) >= 64 * 64 * 4 + 64 * 4
     assert L.mstf_value_spmv_workspace_bytes(128, 4096, 256, 4, 1) % 256 == 0
