@@ -18,9 +18,10 @@
  *   kernel_quant/compression_quant.py:7-529      quantised producer
  *   kernel_quant/csrc/SpMM_Kernel_Quant.cuh:35-262   quantised consumer
  *
- * Parity status of each function is listed in oracle/README.md.  Parity unpinned: the exact fp16 bit patterns
- * the Triton producer emits for a tile's scale / zero-point (no reference fixture fixes its intermediate
- * precision); every other function is pinned by independent checks.
+ * Parity status of each function is listed in oracle/README.md.  Every function is pinned by independent checks;
+ * both producers (fp16 and 2-bit) also by arrays that the reference's own Triton programs wrote under Triton's
+ * interpreter (tests/golden/ref_fp16.npz, ref_quant.npz).  Parity unpinned: the 4- and 8-bit widths of the quantised
+ * producer, which the reference does not have (closed form and error bound only).
  */
 #include <math.h>
 #include <stdint.h>
@@ -361,8 +362,11 @@ void orc_dense_masked_attention(const h16* q, const h16* Kp, const h16* Vp, int 
  *   scale = (max-min)/(2^bit-1), 1 if 0 or empty; zero = floor(-min/scale+0.5)   (:49-57)
  *   code  = clamp(floor(v/scale+0.5)+zero, 0, 2^bit-1)   (:143-145) using the fp16-stored scale/zero (:134-135)
  *   code j of a tile -> bits bit*(j%cap) of word j/cap    (:148-152)
- * scale/zero are computed in fp32 from the fp16 min/max and rounded once to fp16
- * (the exact intermediate precision of the Triton original is not pinned).
+ * scale/zero are computed in fp32 from the fp16 min/max, zero from the unrounded fp32 scale, and each is rounded
+ * once to fp16 on the store: tl.min / tl.max widen sub-32-bit floats to fp32 before reducing, so the whole chain of
+ * :41-57 is fp32 arithmetic in Triton.  Pinned bit for bit (bit = 2) by arrays the reference's own programs wrote
+ * under Triton's interpreter (tests/golden/ref_quant.npz).  bit = 4 / 8 are extensions of this build (the reference
+ * producer hard-codes 2): same formulas with 2^bit - 1 steps, pinned by closed form and error bound only.
  * packed may be NULL to size it. returns total uint32 words. */
 uint64_t orc_compress_quant(const h16* x, int B, int M, int N, int is_value, int bit, uint64_t* bmp, uint32_t* counts,
                             uint32_t* units, uint32_t* tile_off, uint32_t* packed, uint64_t packed_cap, h16* scales,

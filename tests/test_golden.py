@@ -70,3 +70,55 @@ def test_quant_producer_reproduces_the_fixture(bit):
             want = q["%s%d_%s" % (pre, bit, name)]
             a = u16(a) if a.dtype == np.float16 else a
             assert np.array_equal(a, want), name
+
+
+# ------------------------------------------------------------------ fixtures written by the reference's own programs
+# ref_quant.npz / ref_fp16.npz come from tests/golden/make_ref_fixtures.py: the reference's @triton.jit producers
+# (kernel_quant/compression_quant.py:7-157, 267-422; kernel/compression.py:8-247) executed by Triton's interpreter
+# on CPU tensors.  They pin the intermediate precision of scale / zero (tl.min / tl.max widen fp16 to fp32, so the
+# whole chain runs in fp32 and is rounded once on the store) and the packed codes, bit for bit.
+REF_CASES = [("kat_k", "Kp", 0), ("kat_v", "Vp", 1), ("rnd_k", None, 0), ("rnd_v", None, 1)]
+
+
+def _ref_input(rq, pruned):
+    return f16(load("kat_fp16.npz")[pruned]) if pruned else f16(rq["rnd_x"])
+
+
+@pytest.mark.parametrize("case,pruned,is_value", REF_CASES)
+def test_quant_producer_matches_reference_triton_programs(case, pruned, is_value):
+    rq = load("ref_quant.npz")
+    x = _ref_input(rq, pruned)
+    got = orc.compress_quant(x, is_value, 2)
+    for name, a in zip(["bmp", "tile_off", "packed", "counts", "units", "scales", "zeros"], got):
+        a = u16(a) if a.dtype == np.float16 else a
+        assert np.array_equal(a, rq["%s_%s" % (case, name)]), name
+
+
+@pytest.mark.parametrize("case,pruned,is_value", REF_CASES)
+def test_fp16_producer_matches_reference_triton_programs(case, pruned, is_value):
+    rf = load("ref_fp16.npz")
+    x = _ref_input(rf, pruned)
+    bmp, idx, nz, off = orc.compress(x, is_value)
+    assert np.array_equal(bmp, rf[case + "_bmp"]) and np.array_equal(idx, rf[case + "_idx"])
+    assert np.array_equal(u16(nz), rf[case + "_nz"])
+    # nz_off is the caller's running total in 16-byte units (models/llama_mustafar_kernel.py:450-452)
+    assert np.array_equal(off, np.concatenate([[0], np.cumsum(idx[:-1, -1] // 4)]))
+
+
+def test_reference_fixture_separates_the_candidate_precisions():
+    """The fixture must be able to tell an fp16 chain from the fp32 one: a fair share of its tiles round differently."""
+    rq = load("ref_quant.npz")
+    x = f16(rq["rnd_x"])
+    n_diff = n = 0
+    for b in range(x.shape[0]):
+        for t in range(x.shape[1]):
+            for h in range(2):
+                v = x[b, t, h * 64:(h + 1) * 64]
+                v = v[v != 0]
+                if v.size < 2 or not np.isfinite(np.float16(v.max() - v.min())):
+                    continue
+                chain16 = np.float16(np.float16(v.max() - v.min()) / np.float16(3))
+                once32 = np.float16((np.float32(v.max()) - np.float32(v.min())) / np.float32(3))
+                n += 1
+                n_diff += chain16 != once32
+    assert n > 300 and n_diff > 0.1 * n

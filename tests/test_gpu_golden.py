@@ -75,3 +75,35 @@ def test_quant_producer_reproduces_the_fixture(bit):
             a = t.cpu().numpy()
             a = a.view(np.uint16) if a.dtype == np.float16 else a
             assert np.array_equal(a, want["%s%d_%s" % (pre, bit, name)]), name
+
+
+# Fixtures written by the reference's own Triton producers (tests/golden/make_ref_fixtures.py, Triton interpreter on
+# CPU tensors): the HIP producers must reproduce every array bit for bit.
+REF_CASES = [("kat_k", "Kp", False), ("kat_v", "Vp", True), ("rnd_k", None, False), ("rnd_v", None, True)]
+
+
+def _ref_input(r, pruned):
+    return gpu_f16(load("kat_fp16.npz")[pruned]) if pruned else gpu_f16(r["rnd_x"])
+
+
+@pytest.mark.parametrize("case,pruned,is_value", REF_CASES)
+def test_quant_producer_matches_reference_triton_programs(case, pruned, is_value):
+    from mustafar_amd import compression_quant as cq
+    rq = load("ref_quant.npz")
+    x = _ref_input(rq, pruned)
+    got = cq.convert_value_batched_quant(x) if is_value else cq.convert_key_batched_quant(x, return_metadata=True)
+    for name, t in zip(["bmp", "tile_off", "packed", "counts", "units", "scales", "zeros"], got):
+        a = t.cpu().numpy()
+        a = a.view(np.uint16) if a.dtype == np.float16 else a
+        assert np.array_equal(a, rq["%s_%s" % (case, name)]), name
+
+
+@pytest.mark.parametrize("case,pruned,is_value", REF_CASES)
+def test_fp16_producer_matches_reference_triton_programs(case, pruned, is_value):
+    from mustafar_amd import compression as cf
+    rf = load("ref_fp16.npz")
+    x = _ref_input(rf, pruned)
+    bmp, idx, nzs = cf.convert_value_batched(x) if is_value else cf.convert_key_batched(x)
+    assert np.array_equal(bmp.cpu().numpy(), rf[case + "_bmp"])
+    assert np.array_equal(idx.cpu().numpy(), rf[case + "_idx"])
+    assert np.array_equal(np.concatenate([bits(t) for t in nzs]), rf[case + "_nz"])

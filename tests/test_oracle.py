@@ -298,11 +298,12 @@ def test_quant_closed_forms_and_roundtrip_bound(bit, is_value):
             if vals.size == 0:
                 assert scales[b, t] == 1 and zeros[b, t] == 0
                 continue
-            sc = np.float32(vals.max() - vals.min()) / np.float32(maxq)
-            sc = np.float32(1.0) if sc == 0 else sc
-            zp = np.floor(-vals.min() / sc + np.float32(0.5))
-            assert scales[b, t] == np.float16(sc) and zeros[b, t] == np.float16(zp)
+            # scale / zero bit patterns: held to the reference's own Triton programs in tests/test_golden.py
+            # (ref_quant.npz); here only what the mathematics fixes: the range is covered by maxq steps
             s16, z16 = np.float32(scales[b, t]), np.float32(zeros[b, t])
+            rng_ = np.float32(vals.max() - vals.min())
+            assert (rng_ == 0 and s16 == 1) or abs(s16 * maxq - rng_) <= 2.0 ** -10 * rng_ + 1e-7
+            assert abs(z16 + vals.min() / s16) <= 0.5 + 2.0 ** -10 * abs(z16) + 1e-3
             for j, v in enumerate(vals):
                 code = _unpack_py(packed, int(toff[b, t]), j, bit)
                 want = int(min(max(np.floor(v / s16 + np.float32(0.5)) + z16, 0), maxq))
