@@ -40,7 +40,8 @@ enum {
     MSTF_EALIGN = -2,       /* a pointer is not aligned as required */
     MSTF_EUNSUPPORTED = -3, /* shape outside what the kernels cover (e.g. head_dim != 128) */
     MSTF_EWORKSPACE = -4,   /* workspace missing or too small */
-    MSTF_ELAUNCH = -5       /* HIP reported an error at launch; see mstf_last_hip_error() */
+    MSTF_ELAUNCH = -5,      /* HIP reported an error at launch; see mstf_last_hip_error() */
+    MSTF_ETOOLARGE = -6     /* the problem needs more scratch than the library's fixed buffer holds */
 };
 
 const char* mstf_strerror(int code);
@@ -171,6 +172,22 @@ int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, const mstf_ha
                               const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out,
                               float* lse_out, int tokens, int head_dim, int Bq, int groups, void* workspace,
                               size_t workspace_bytes);
+/* mstf_decode_attention_f16 for callers that cannot allocate or hand over a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The split partials live
+ * in a device array of MSTF_STATIC_SCRATCH_BYTES that is part of the library image: each GPU the library runs on holds
+ * one copy until the process ends, and every call on a GPU uses that GPU's copy.  Same arguments, results and checks
+ * as mstf_decode_attention_f16 without the workspace pair; a problem whose partials
+ * (mstf_decode_attention_workspace_bytes) exceed the buffer is refused with MSTF_ETOOLARGE before anything is
+ * launched (4096 tokens fit up to Bq = 1008 query rows; at the headline shape - 256 rows - up to 15872 tokens).  Calls
+ * no hipMalloc / hipFree or other allocating routine; the first call on a device looks the array's address up
+ * (hipGetSymbolAddress, with that device current - make that first call outside a graph capture).  Nothing has to be
+ * cleared between calls: the kernels write every partial they later read.  Calls that overlap on one GPU (two streams,
+ * two threads) share the buffer and race: serialise them, or use the workspace form. */
+#define MSTF_STATIC_SCRATCH_BYTES ((size_t)4 << 20)
+int mstf_decode_attention_static_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                                     const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                                     const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q,
+                                     mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq, int groups);
 /* The two phases of mstf_decode_attention_f16 as separate calls, for a caller that shards the cached
  * tokens (each shard runs `partial` on its tokens, the (max, sum, output) triples are then combined).
  * partial: per token split s and query row: workspace = float part_o[Bq][ns][head_dim] followed by

@@ -51,6 +51,7 @@ SIGNATURES = {
     "mstf_decode_attention_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mstf_decode_attention_splits": (_i, [_i, _i, _i, _i]),
     "mstf_decode_attention_f16": (_i, [_vp] * 12 + [_i, _i, _i, _i, _vp, _sz]),
+    "mstf_decode_attention_static_f16": (_i, [_vp] * 12 + [_i, _i, _i, _i]),
     "mstf_decode_attention_partial_f16": (_i, [_vp] * 10 + [_i, _i, _i, _i, _vp, _sz]),
     "mstf_decode_attention_merge_f16": (_i, [_vp, _vp, _sz, _vp, _vp, _i, _i, _i, _i]),
     "mstf_decode_attention_window_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),

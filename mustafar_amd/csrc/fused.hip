@@ -14,6 +14,8 @@
 // merge kernel.  Scores and probabilities never touch HBM.
 #include "fused_common.hpp"
 
+#include <atomic>
+
 namespace mstf {
 
 // grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns the bpw consecutive token
@@ -490,6 +492,7 @@ extern "C" size_t mstf_decode_attention_workspace_bytes(int tokens, int head_dim
 }
 
 // Shared argument checks of the fused entry points.
+constexpr size_t kWorkspaceIsOurs = ~(size_t)0;
 static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, const void* k_nz_off, const void* v_bmp,
                         const void* v_nz, const void* v_idx, const void* v_nz_off, const void* q, int tokens,
                         int head_dim, int Bq, int groups, const void* workspace, size_t workspace_bytes)
@@ -501,6 +504,7 @@ static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, 
         !aligned_to(k_idx, 4) || !aligned_to(v_idx, 4) || !aligned_to(k_nz_off, 4) || !aligned_to(v_nz_off, 4) ||
         !aligned_to(q, 16))
         return MSTF_EALIGN;
+    if (workspace_bytes == kWorkspaceIsOurs) return MSTF_OK;  // the library's own buffer: nothing of the caller's to check
     const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
@@ -626,6 +630,63 @@ extern "C" int mstf_decode_attention_f16(void* stream, const uint64_t* k_bmp, co
                                            groups);
 }
 
+
+// ------------------------------------------------------------------ the entry point that allocates nothing
+// mstf_decode_attention_f16 with the split partials in a buffer the library itself holds: a file-scope device array
+// (one copy per GPU, held until the process ends).  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address it yields - looked up once per device, with that device current - is what the
+// kernels get.
+constexpr size_t kStaticScratchBytes = MSTF_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kStaticMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kStaticMaxDevices];
+
+static int static_scratch(void** ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) {
+        set_last_hip_error((int)(e != hipSuccess ? e : hipErrorInvalidDevice));
+        return MSTF_ELAUNCH;
+    }
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_last_hip_error((int)(e != hipSuccess ? e : hipErrorInvalidSymbol));
+            return MSTF_ELAUNCH;
+        }
+        g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+    }
+    *ptr = p;
+    return MSTF_OK;
+}
+
+extern "C" int mstf_decode_attention_static_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                                const uint32_t* k_idx, const uint32_t* k_nz_off, const uint64_t* v_bmp,
+                                                const mstf_half* v_nz, const uint32_t* v_idx, const uint32_t* v_nz_off,
+                                                const mstf_half* q, mstf_half* out, float* lse_out, int tokens,
+                                                int head_dim, int Bq, int groups)
+{
+    if (!out) return MSTF_EINVAL;
+    // sizes first, on the host alone: a problem whose partials do not fit is refused before anything touches the GPU
+    if (tokens <= 0 || Bq <= 0 || groups <= 0 || Bq % groups != 0) return MSTF_EINVAL;
+    if (head_dim != kFusedD || tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    const size_t need = mstf_decode_attention_workspace_bytes(tokens, head_dim, Bq, groups);
+    if (need == 0 || need > kStaticScratchBytes) return MSTF_ETOOLARGE;
+    void* ws = nullptr;
+    int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, tokens, head_dim, Bq, groups,
+                          nullptr, kWorkspaceIsOurs);
+    if (rc != MSTF_OK) return rc;
+    if (!aligned_to(out, 2) || (lse_out && !aligned_to(lse_out, 4))) return MSTF_EALIGN;
+    if ((rc = static_scratch(&ws)) != MSTF_OK) return rc;
+    // every split slot of every row is written by the partial kernel before the merge reads it: nothing to clear
+    const int write_final = (splits_of(tokens, Bq, groups) == 1 && !lse_out) ? 1 : 0;
+    rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, out, tokens,
+                       head_dim, Bq, groups, ws, write_final);
+    if (rc != MSTF_OK || write_final) return rc;
+    return merge_splits(as_stream(stream), ws, out, lse_out, splits_of(tokens, Bq, groups), head_dim, Bq);
+}
 
 extern "C" size_t mstf_decode_attention_window_workspace_bytes(int tokens, int max_window, int head_dim, int Bq,
                                                                int groups)

@@ -17,6 +17,9 @@ extern "C" const char* mstf_strerror(int code)
         case MSTF_EUNSUPPORTED: return "shape not supported by the gfx950 kernels";
         case MSTF_EWORKSPACE: return "workspace missing or too small";
         case MSTF_ELAUNCH: return "HIP kernel launch failed (see mstf_last_hip_error)";
+        case MSTF_ETOOLARGE:
+            return "the problem needs more scratch memory than the library's fixed buffer holds (use the entry point "
+                   "that takes a workspace)";
         default: return "unknown error code";
     }
 }

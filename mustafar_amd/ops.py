@@ -194,6 +194,21 @@ def decode_attention(ck, cv, q, groups, out=None, lse=None):
     return o
 
 
+def decode_attention_static(ck, cv, q, groups, out=None, lse=None):
+    """decode_attention through the entry point that uses the library's own fixed scratch buffer: no workspace is
+    passed and nothing is allocated by the library (calls on one GPU must not overlap)."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    D = ck.head_dim
+    Bq = q.numel() // D
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    check(lib().mstf_decode_attention_static_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
+                                                 ck.nz_off.data_ptr(), cv.bmp.data_ptr(), cv.nz.data_ptr(),
+                                                 cv.idx.data_ptr(), cv.nz_off.data_ptr(), q.data_ptr(), o.data_ptr(),
+                                                 lse.data_ptr() if lse is not None else None, ck.tokens, D, Bq, groups),
+          "mstf_decode_attention_static_f16")
+    return o
+
+
 def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, lse=None, win_len_dev=None):
     """Attention of one decode step over [compressed tokens | dense window] under one softmax, three launches.
 

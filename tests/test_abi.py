@@ -45,7 +45,7 @@ def test_binding_table_matches_header():
 def test_error_strings_and_version(lib):
     lib.mstf_strerror.restype = ctypes.c_char_p
     assert lib.mstf_strerror(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6):
         assert lib.mstf_strerror(code) and lib.mstf_strerror(code) != lib.mstf_strerror(-99)
     assert lib.mstf_version() >= 100
 
@@ -66,6 +66,9 @@ def test_argument_validation_returns_before_any_launch(lib):
     assert L.mstf_compress_proj_f16(None, ctypes.byref(src), 0, 64, 128, 89, None, None, None, None, None, 0, None, 0) == -1
     assert L.mstf_append_proj_f16(None, ctypes.byref(src), 1, 64, 128, 89, None, None, None, None, None, None, None, 0) == -1
     assert L.mstf_decode_attention_f16(None, *([None] * 11), 64, 128, 4, 4, None, 0) == -1
+    # the entry point on the library's fixed scratch buffer refuses, on the host, what does not fit into it
+    assert L.mstf_decode_attention_static_f16(None, *([256] * 10), None, 4096, 128, 1012, 4) == -6
+    assert L.mstf_decode_attention_static_f16(None, *([None] * 11), 4096, 128, 256, 4) == -1
     assert L.mstf_decode_attention_splits(4096, 128, 256, 4) == 8
     assert L.mstf_decode_attention_splits(4096, 128, 1024, 4) == 2       # 16384 blocks: four per wavefront
     # workspace sizes are pure host arithmetic
