@@ -7,13 +7,9 @@ import torch
 
 from oracle import oracle as orc
 
+from _metrics import rel_err   # row metric and element-wise allclose(rtol, atol = rtol * rms) in one number
+
 pytestmark = pytest.mark.gpu
-
-
-def rel_rowmax(a, b):
-    a = a.astype(np.float64).reshape(-1, a.shape[-1])
-    b = b.astype(np.float64).reshape(-1, b.shape[-1])
-    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
 @pytest.mark.parametrize("fused,pooled,window_kernel", [(False, False, False), (True, False, False), (True, True, False),
@@ -45,7 +41,7 @@ def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled, window
             Kf[:, :Lc_before] = orc.prune_rows(np.ascontiguousarray(Kf[:, :Lc_before]), 89)
             Vf[:, :Lc_before] = orc.prune_rows(np.ascontiguousarray(Vf[:, :Lc_before]), 89)
             _, _, ref = orc.dense_masked_attention(Q[t], Kf, Vf, g)
-            assert rel_rowmax(out.cpu().numpy().reshape(-1, D), ref) < 2e-3, (t, pos)
+            assert rel_err(out.cpu().numpy().reshape(-1, D), ref) < 2e-3, (t, pos)
             checked += 1
     assert cache.kv_len == total and cache.compressed_length == 768      # two appends happened
     assert cache.k_win.shape[2] == total - 768
@@ -145,7 +141,7 @@ def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
             Kf[:, :Lc_before] = dequantised(K, Lc_before, 0)
             Vf[:, :Lc_before] = dequantised(V, Lc_before, 1)
             _, _, ref = orc.dense_masked_attention(Q[t], Kf, Vf, g)
-            assert rel_rowmax(out.cpu().numpy().reshape(-1, D), ref) < 1e-2, (t, pos)
+            assert rel_err(out.cpu().numpy().reshape(-1, D), ref) < 1e-2, (t, pos)
             checked += 1
     assert cache.compressed_length == 512 and cache.kv_len == total and checked >= 6
     # per-tile arrays equal a one-shot quantisation; the packed words are the same words, chunk by chunk

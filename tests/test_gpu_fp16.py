@@ -9,6 +9,8 @@ import torch
 
 from oracle import oracle as orc
 
+from _metrics import check_chain, rel_err   # row metric and element-wise allclose(rtol, atol = rtol * rms) in one number
+
 pytestmark = pytest.mark.gpu
 
 RTOL = 2e-3  # fp16 tolerance of the north-star metric
@@ -20,14 +22,6 @@ def dev():
 
 def to_gpu(a):
     return torch.from_numpy(np.ascontiguousarray(a)).to(dev())
-
-
-def rel_rowmax(a, b):
-    """max |a-b| per row divided by max |b| of the row (rows = all leading axes)."""
-    a = a.astype(np.float64).reshape(-1, a.shape[-1])
-    b = b.astype(np.float64).reshape(-1, b.shape[-1])
-    den = np.maximum(np.abs(b).max(-1), 1e-30)
-    return (np.abs(a - b).max(-1) / den).max()
 
 
 def special_inputs(seed, B, M, D=128):
@@ -125,7 +119,7 @@ def test_reference_api_convert_and_formulation():
                                                     groups)
     assert tuple(att.shape) == (Bq, 8, Lc) and att.dtype == torch.float16
     C, Cf = orc.key_spmv(rb, rnz, ri, roff, padded_query.cpu().numpy(), Lc, D, groups)
-    assert rel_rowmax(att.cpu().numpy(), Cf) < RTOL
+    assert rel_err(att.cpu().numpy(), Cf) < RTOL
     assert not att[:, 1].any()          # zero query rows give zero scores
 
     P = orc.scale_softmax(C[:, 0], D)
@@ -136,7 +130,7 @@ def test_reference_api_convert_and_formulation():
     assert tuple(out.shape) == (Bq, 8, D)
     vb, vi, vnz, voff = orc.compress(Vp, 1)
     O, Of = orc.value_spmv(vb, vnz, vi, voff, padded_score.cpu().numpy(), D, Lc, groups)
-    assert rel_rowmax(out.cpu().numpy()[:, 0], Of[:, 0]) < RTOL
+    assert rel_err(out.cpu().numpy()[:, 0], Of[:, 0]) < RTOL
     assert not out[:, 1:].any()
 
     with pytest.raises(RuntimeError):
@@ -168,19 +162,17 @@ def test_decode_attention_against_dense_masked_oracle(groups, Bkv, Lc, sparsity)
     ck = ops.compress(to_gpu(K), False, kth=kth)
     cv = ops.compress(to_gpu(V), True, kth=kth)
     s = ops.key_spmv(ck, to_gpu(q).view(Bq, 1, D), groups)
-    assert rel_rowmax(s.cpu().numpy()[:, 0], sc_ref) < RTOL
     p = ops.scale_softmax(s, D)
-    assert rel_rowmax(p.cpu().numpy()[:, 0], pr_ref) < RTOL
     o = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o.cpu().numpy()[:, 0], out_ref) < RTOL
+    check_chain(RTOL, sc_ref, pr_ref, out_ref, Vp, groups, s=s[:, 0], p=p[:, 0], o=o[:, 0])
     # and each product separately against the fp32 sums of the oracle fed the same inputs
     kb = orc.compress(Kp, 0)
     _, Cf = orc.key_spmv(kb[0], kb[2], kb[1], kb[3], q.reshape(Bq, 1, D), Lc, D, groups)
-    assert rel_rowmax(s.cpu().numpy(), Cf) < 1e-3
+    assert rel_err(s.cpu().numpy(), Cf) < 1e-3
     vb = orc.compress(Vp, 1)
     _, Of = orc.value_spmv(vb[0], vb[2], vb[1], vb[3], pr_ref.reshape(Bq, 1, Lc), D, Lc, groups)
     o2 = ops.value_spmv(cv, to_gpu(pr_ref).view(Bq, 1, Lc), groups)
-    assert rel_rowmax(o2.cpu().numpy(), Of) < 1e-3
+    assert rel_err(o2.cpu().numpy(), Of) < 1e-3
 
 
 def test_softmax_strided_and_inplace():
@@ -190,12 +182,12 @@ def test_softmax_strided_and_inplace():
     ref = orc.scale_softmax(s, 128)
     g = to_gpu(s)
     p = ops.scale_softmax(g, 128)
-    assert rel_rowmax(p.cpu().numpy(), ref) < 1e-3
+    assert rel_err(p.cpu().numpy(), ref) < 1e-3
     big = torch.zeros((6, 1200), dtype=torch.float16, device=dev())
     big[:, :1000] = g
     view = big[:, :1000]
     ops.scale_softmax(view, 128, out=view)      # strided rows, in place
-    assert rel_rowmax(view.cpu().numpy(), ref) < 1e-3
+    assert rel_err(view.cpu().numpy(), ref) < 1e-3
 
 
 def test_special_bitmaps():
@@ -272,9 +264,7 @@ def test_config0_shape_against_oracle():
         assert np.array_equal(c.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
     qg = to_gpu(q)
     s = ops.key_spmv(ck, qg.view(heads, 1, D), groups)
-    assert rel_rowmax(s.cpu().numpy()[:, 0], s_ref) < RTOL
     p = ops.scale_softmax(s, D)
-    assert rel_rowmax(p.cpu().numpy()[:, 0], p_ref) < RTOL
     o = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o.cpu().numpy()[:, 0], o_ref) < RTOL
-    assert rel_rowmax(ops.decode_attention(ck, cv, qg, groups).cpu().numpy(), o_ref) < RTOL
+    check_chain(RTOL, s_ref, p_ref, o_ref, Vp, groups, s=s[:, 0], p=p[:, 0], o=o[:, 0],
+                fused=ops.decode_attention(ck, cv, qg, groups))

@@ -1,20 +1,31 @@
-"""Size-independent properties at the headline size (batch 8 x 8 KV heads, 4096 tokens, 70 %), where the CPU
-oracle would take minutes: the checker here is plain torch on the device - kthvalue pruning, fp32 matmuls - which
-shares no code with the kernels under test.
+"""Size-independent properties at the full sizes of the benchmark configurations, where the CPU oracle would take
+minutes: the checker here is plain torch on the device - kthvalue pruning, fp32 matmuls, the quantiser's closed form -
+which shares no code with the kernels under test.
+
+  configs[1]  batch 8 x 8 KV heads (64 heads), 4096 tokens, 70 % and 50 %: formats, three-launch and fused attention
+  configs[2]  batch 16 x 8 KV heads (128 heads), 4096 tokens, 50 / 70 / 90 %: formats of both compressors
+  configs[3]  batch 32 x 8 KV heads (256 heads), 4096 tokens, 70 %, 2- and 4-bit codes: producer arrays against the
+              closed form, three-launch and fused quantised attention against dense attention on the dequantised cache
 
   * format invariants of the compressed cache (padding rule, offsets, popcounts) and checksums of its content
     against the torch-pruned dense tensor;
-  * fused and three-launch sparse decode attention against dense masked attention on the torch-pruned tensors,
-    2e-3 relative to the row maximum (the north-star tolerance).
+  * sparse decode attention against dense masked attention on the torch-pruned tensors: 2e-3 (fp16) / 1e-2
+    (quantised), row metric end to end and element-wise from the scores the GPU produced.
 """
 import math
 
 import pytest
 import torch
 
+from _metrics import elem_err, rel_err, row_err
+
 pytestmark = pytest.mark.gpu
 
-BKV, L, D, GROUPS, KTH = 64, 4096, 128, 4, 89
+L, D, GROUPS = 4096, 128, 4
+KTH = 89          # 70 %
+# (KV heads, pruning rank): configs[1] at 70 % / 50 %, configs[2] at 50 / 70 / 90 %
+FORMAT_CASES = [(64, 89), (64, 64), (128, 64), (128, 89), (128, 115)]
+ATTENTION_CASES = [(64, 89), (64, 64), (128, 89)]
 
 
 def popcount64(x):
@@ -33,25 +44,42 @@ def torch_prune(x, kth):
     return torch.where(a >= thr, x, torch.zeros_like(x))
 
 
-@pytest.fixture(scope="module")
+_DATA = {}
+
+
+def make_data(bkv, kth):
+    """Seeded K (two outlier channels), V, q and their torch-pruned forms; the latest case stays cached."""
+    key = (bkv, kth)
+    if key not in _DATA:
+        _DATA.clear()
+        torch.cuda.empty_cache()
+        dev = torch.device("cuda:0")
+        g = torch.Generator(device=dev)
+        g.manual_seed(4096 + bkv + kth)
+        K = torch.randn((bkv, L, D), generator=g, device=dev).half()
+        V = torch.randn((bkv, L, D), generator=g, device=dev).half()
+        K[:, :, 5] *= 10
+        K[:, :, 77] *= 10
+        q = torch.randn((bkv * GROUPS, D), generator=g, device=dev).half()
+        _DATA[key] = (K, V, q, torch_prune(K, kth), torch_prune(V, kth))
+    return _DATA[key]
+
+
+@pytest.fixture()
 def data():
-    dev = torch.device("cuda:0")
-    g = torch.Generator(device=dev)
-    g.manual_seed(4096)
-    K = torch.randn((BKV, L, D), generator=g, device=dev).half()
-    V = torch.randn((BKV, L, D), generator=g, device=dev).half()
-    K[:, :, 5] *= 10
-    K[:, :, 77] *= 10
-    q = torch.randn((BKV * GROUPS, D), generator=g, device=dev).half()
-    return K, V, q, torch_prune(K, KTH), torch_prune(V, KTH)
+    return make_data(64, KTH)
+
+
+BKV = 64
 
 
 @pytest.mark.parametrize("is_value", [0, 1])
-def test_format_invariants_and_checksums(data, is_value):
+@pytest.mark.parametrize("BKV,kth", FORMAT_CASES)
+def test_format_invariants_and_checksums(BKV, kth, is_value):
     from mustafar_amd import ops
-    K, V, _, Kp, Vp = data
+    K, V, _, Kp, Vp = make_data(BKV, kth)
     x, xp = (V, Vp) if is_value else (K, Kp)
-    c = ops.compress(x, bool(is_value), kth=KTH)
+    c = ops.compress(x, bool(is_value), kth=kth)
     T = L * D // 64
     assert c.bmp.shape == (BKV, T) and c.idx.shape == (BKV, T + 1)
     pop = popcount64(c.bmp)
@@ -83,48 +111,142 @@ def test_format_invariants_and_checksums(data, is_value):
     assert int((nz != 0).sum()) == int(pop.sum())
 
 
+def scaled(s):
+    """fp16(s / sqrt(d)) by true division: torch divides a device tensor by a host scalar as a multiplication with the
+    rounded reciprocal, which rounds a few results differently; the divisor therefore goes in as a tensor."""
+    return torch.div(s.float(), torch.tensor(math.sqrt(D), dtype=torch.float32, device=s.device)).half()
+
+
 def dense_masked_attention(q, Kp, Vp, groups=GROUPS):
     """The reference's dense path on pruned tensors (models/llama_mustafar_Kt_Mag_Vt_Mag.py:836-1026): fp16 scores with
     fp32 accumulation, / sqrt(d) in fp16, fp32 softmax rounded to fp16, fp32-accumulated P.V rounded to fp16."""
     bkv, length = Kp.shape[0], Kp.shape[1]
     qh = q.view(bkv, groups, D).float()
     s = torch.einsum("bgd,bld->bgl", qh, Kp.float()).half()
-    w = (s / math.sqrt(D)).float()
+    w = scaled(s).float()
     p = torch.softmax(w, -1).half()
     o = torch.einsum("bgl,bld->bgd", p.float(), Vp.float()).half()
     return s.view(-1, length), p.view(-1, length), o.view(-1, D)
 
 
-def rel_rowmax(a, b):
-    a, b = a.double(), b.double()
-    return float(((a - b).abs().amax(-1) / b.abs().amax(-1).clamp_min(1e-30)).max())
+def continue_from_scores(s, Vp, groups=GROUPS):
+    """The dense path continued from given fp16 scores [Bq, L]: probabilities and output as the reference rounds them."""
+    bkv, length = Vp.shape[0], Vp.shape[1]
+    w = scaled(s).float()
+    p = torch.softmax(w, -1).half()
+    o = torch.einsum("bgl,bld->bgd", p.view(bkv, groups, length).float(), Vp.float()).half()
+    return p, o.view(-1, D)
 
 
-def test_decode_attention_full_size(data):
+def check_chain(tol, refs, Vp, s, p=None, o=None, fused=None, groups=GROUPS):
+    """Scores: both metrics against the checker's.  Everything behind the scores: the row metric end to end, and both
+    metrics against the checker continued from the GPU's own scores / probabilities (two correct summation orders round
+    about one score in a thousand to neighbouring fp16 values, and one ulp of an outlier-sized score moves that
+    token's probability by up to 2 %)."""
+    s_ref, p_ref, o_ref = refs
+    assert rel_err(s, s_ref) < tol, (row_err(s, s_ref), elem_err(s, s_ref))
+    p_cont, o_cont = continue_from_scores(s, Vp, groups)
+    if p is not None:
+        assert row_err(p, p_ref) < tol and rel_err(p, p_cont) < tol, (row_err(p, p_ref), elem_err(p, p_cont))
+    if o is not None:
+        bkv, length = Vp.shape[0], Vp.shape[1]
+        want = torch.einsum("bgl,bld->bgd", p.view(bkv, groups, length).float(), Vp.float()).half().view(-1, D)
+        assert row_err(o, o_ref) < tol and rel_err(o, want) < tol, (row_err(o, o_ref), elem_err(o, want))
+    if fused is not None:
+        assert row_err(fused, o_ref) < tol and rel_err(fused, o_cont) < tol, (row_err(fused, o_ref),
+                                                                              elem_err(fused, o_cont))
+
+
+@pytest.mark.parametrize("BKV,kth", ATTENTION_CASES)
+def test_decode_attention_full_size(BKV, kth):
     from mustafar_amd import ops
-    K, V, q, Kp, Vp = data
-    s_ref, p_ref, o_ref = dense_masked_attention(q, Kp, Vp)
-    ck = ops.compress(K, False, kth=KTH)
-    cv = ops.compress(V, True, kth=KTH)
+    K, V, q, Kp, Vp = make_data(BKV, kth)
+    refs = dense_masked_attention(q, Kp, Vp)
+    s_ref, p_ref, o_ref = refs
+    ck = ops.compress(K, False, kth=kth)
+    cv = ops.compress(V, True, kth=kth)
     Bq = BKV * GROUPS
     s = ops.key_spmv(ck, q.view(Bq, 1, D), GROUPS)
-    assert rel_rowmax(s[:, 0], s_ref) < 2e-3
     p = ops.scale_softmax(s, D)
-    assert rel_rowmax(p[:, 0], p_ref) < 2e-3
     o = ops.value_spmv(cv, p, GROUPS)
-    assert rel_rowmax(o[:, 0], o_ref) < 2e-3
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=q.device)
     of = ops.decode_attention(ck, cv, q, GROUPS, lse=lse)
-    assert rel_rowmax(of, o_ref) < 2e-3
+    check_chain(2e-3, refs, Vp, s[:, 0], p[:, 0], o[:, 0], of)
     # (max, sum) of the scaled scores
-    w = (s_ref / math.sqrt(D)).float()
+    w = scaled(s_ref).float()
     m_ref = w.amax(-1)
     assert float((lse[:, 0] - m_ref).abs().max()) <= 2e-2 * max(float(m_ref.abs().max()), 1.0)
     l_ref = torch.exp(w - m_ref[:, None]).sum(-1)
     assert float((lse[:, 1] * torch.exp(lse[:, 0] - m_ref) - l_ref).abs().max()) <= 5e-3 * float(l_ref.max())
     # linearity of the value product in the probabilities: P -> 0.5 P halves the output exactly (power of two)
     o_half = ops.value_spmv(cv, (p * 0.5).contiguous(), GROUPS)
-    assert torch.equal(o_half.float() * 2, o.float()) or rel_rowmax(o_half[:, 0] * 2, o[:, 0]) < 1e-3
+    assert torch.equal(o_half.float() * 2, o.float()) or rel_err(o_half[:, 0] * 2, o[:, 0]) < 1e-3
+
+
+# ------------------------------------------------------------------ configs[3]: quantised cache, 256 heads x 4096 tokens
+def torch_quantise(xp, is_value, bit):
+    """The producer's closed form (kernel_quant/compression_quant.py:41-57, 143-145) and the consumer's dequantisation
+    (kernel_quant/csrc/SpMM_Kernel_Quant.cuh:238-240) with torch operators on [B, L, D] pruned values: per 64-element
+    tile fp32 scale / zero-point rounded to fp16, codes, and the dequantised dense tensor (mode 0)."""
+    B, length, _ = xp.shape
+    if is_value:
+        tiles = xp.view(B, length // 64, 64, 2, 64).permute(0, 1, 3, 2, 4)      # [b, blk, half, tok, ch]
+    else:
+        tiles = xp.view(B, length // 64, 64, D).permute(0, 1, 3, 2)             # [b, blk, ch, tok]
+    tiles = tiles.reshape(B, -1, 64).float()
+    nz = tiles != 0
+    maxq = float((1 << bit) - 1)
+    inf = torch.tensor(float("inf"), device=xp.device)
+    mn = torch.where(nz, tiles, inf).amin(-1)
+    mx = torch.where(nz, tiles, -inf).amax(-1)
+    any_nz = nz.any(-1)
+    scale = torch.div(mx - mn, torch.tensor(maxq, device=xp.device))     # tensor divisor: true division
+    scale = torch.where(any_nz & (scale != 0), scale, torch.ones_like(scale))
+    zero = torch.where(any_nz, torch.floor(-mn / scale + 0.5), torch.zeros_like(scale))
+    s16, z16 = scale.half(), zero.half()
+    sf, zf = s16.float()[..., None], z16.float()[..., None]
+    code = (torch.floor(tiles / sf + 0.5) + zf).clamp(0, maxq)
+    deq = torch.where(nz, ((code - zf) * sf), torch.zeros_like(tiles)).half()
+    if is_value:
+        dense = deq.view(B, length // 64, 2, 64, 64).permute(0, 1, 3, 2, 4).reshape(B, length, D)
+    else:
+        dense = deq.view(B, length // 64, D, 64).permute(0, 1, 3, 2).reshape(B, length, D)
+    return s16, z16, dense.contiguous()
+
+
+@pytest.mark.parametrize("bit", [2, 4])
+def test_quantised_decode_attention_full_size(bit):
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    from mustafar_amd import ops
+    bkv = 256
+    K, V, q, Kp, Vp = make_data(bkv, KTH)
+    Bq, cap = bkv * GROUPS, 32 // bit
+    kq = cq.convert_key_batched_quant(Kp, return_metadata=True, bit=bit)
+    vq = cq.convert_value_batched_quant(Vp, bit=bit)
+    ks, kz, Kd = torch_quantise(Kp, False, bit)
+    vs, vz, Vd = torch_quantise(Vp, True, bit)
+    # producer arrays at the full size: scales / zero-points bit for bit, counts = popcounts, offsets = running units
+    for got, (s16, z16) in ((kq, (ks, kz)), (vq, (vs, vz))):
+        assert torch.equal(got[5].view(torch.int16), s16.view(torch.int16))
+        assert torch.equal(got[6].view(torch.int16), z16.view(torch.int16))
+        pop = popcount64(got[0])
+        assert torch.equal(got[3].to(torch.int64), pop) and torch.equal(got[4].to(torch.int64), (pop + cap - 1) // cap)
+        units = got[4].to(torch.int64).view(-1)
+        assert torch.equal(got[1].to(torch.int64).view(-1)[1:], torch.cumsum(units, 0)[:-1]) and int(got[1].view(-1)[0]) == 0
+        assert got[2].numel() == int(units.sum())
+    del K, V
+    refs = dense_masked_attention(q, Kd, Vd)
+    qp = torch.zeros((Bq, 8, D), dtype=torch.float16, device=q.device)
+    qp[:, 0] = q
+    s = mpq.mustafar_key_formulation_quant_meta(kq[0], kq[2], kq[1], kq[3], kq[4], kq[5], kq[6], qp, L, D, Bq, GROUPS,
+                                                bit, cap)[:, 0].contiguous()
+    p = ops.scale_softmax(s, D)
+    o = mpq.mustafar_value_formulation_quant_decode_n1(vq[0], vq[2], vq[1], vq[3], vq[4], vq[5], vq[6], p, None, D, L, Bq,
+                                                       GROUPS, bit, cap)
+    of = mpq.decode_attention_quant(kq, vq, q, GROUPS, bit)
+    check_chain(1e-2, refs, Vd, s, p, o, of)
+    _DATA.clear()
 
 
 @pytest.mark.parametrize("bkv,blocks,groups", [(140, 31, 4), (150, 56, 2), (40, 112, 8), (600, 64, 1), (8, 2048, 4)])
@@ -154,23 +276,23 @@ def test_decode_attention_many_blocks(bkv, blocks, groups):
     # of its own; the fused kernel keeps un-normalised weights (<= 1) in fp16 and normalises in fp32.  So the fused
     # output is held to 2e-3 against the same attention with fp32 probabilities, and to a looser bound against the
     # reference formula for the long case; the three-launch path, which rounds as the reference does, is held to it.
-    w = (s_ref / math.sqrt(D)).float()
+    w = scaled(s_ref).float()
     Vp = torch_prune(V, KTH)
     o_exact = torch.einsum("bgl,bld->bgd", torch.softmax(w, -1).view(bkv, groups, length), Vp.float()).half().view(-1, D)
-    assert rel_rowmax(o, o_exact) < 2e-3
+    assert rel_err(o, o_exact) < 2e-3
     tol_ref = 2e-3 if length <= 32768 else 4e-3
-    assert rel_rowmax(o, o_ref) < tol_ref
+    assert rel_err(o, o_ref) < tol_ref
     m_ref = w.amax(-1)
     assert float((lse[:, 0] - m_ref).abs().max()) <= 2e-2 * max(float(m_ref.abs().max()), 1.0)
     l_ref = torch.exp(w - m_ref[:, None]).sum(-1)
     assert float((lse[:, 1] * torch.exp(lse[:, 0] - m_ref) - l_ref).abs().max()) <= 5e-3 * float(l_ref.max())
     o2 = ops.decode_attention(ck, cv, q, groups)            # route without (max, sum) output
-    assert rel_rowmax(o2, o_exact) < 2e-3
+    assert rel_err(o2, o_exact) < 2e-3
     # the three-launch path on the same cache
     p = ops.scale_softmax(ops.key_spmv(ck, q.view(Bq, 1, D), groups), D)
     o3 = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o3[:, 0], o_ref) < 2e-3
-    assert rel_rowmax(o, o3[:, 0]) < tol_ref
+    assert rel_err(o3[:, 0], o_ref) < 2e-3
+    assert rel_err(o, o3[:, 0]) < tol_ref
 
 
 def test_compress_twice_is_idempotent(data):

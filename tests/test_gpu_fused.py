@@ -6,13 +6,9 @@ import torch
 
 from oracle import oracle as orc
 
+from _metrics import check_chain, rel_err   # row metric and element-wise allclose(rtol, atol = rtol * rms) in one number
+
 pytestmark = pytest.mark.gpu
-
-
-def rel_rowmax(a, b):
-    a = a.astype(np.float64).reshape(-1, a.shape[-1])
-    b = b.astype(np.float64).reshape(-1, b.shape[-1])
-    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
 @pytest.mark.parametrize("groups,Bkv,Lc,sparsity", [(4, 2, 1024, 0.7), (4, 3, 64, 0.7), (1, 4, 576, 0.5),
@@ -32,9 +28,10 @@ def test_fused_decode_attention(groups, Bkv, Lc, sparsity):
     qg = torch.from_numpy(q).to(dev)
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
     o = ops.decode_attention(ck, cv, qg, groups, lse=lse)
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3
+    s = ops.key_spmv(ck, qg.view(Bq, 1, D), groups)
+    check_chain(2e-3, sc_ref, pr_ref, out_ref, Vp, groups, s=s[:, 0], fused=o)
     o2 = ops.decode_attention(ck, cv, qg, groups)            # route without (max, sum) output
-    assert rel_rowmax(o2.cpu().numpy(), out_ref) < 2e-3
+    check_chain(2e-3, sc_ref, pr_ref, out_ref, Vp, groups, s=s[:, 0], fused=o2)
     # (max, sum) against the oracle's scaled scores
     w = (sc_ref.astype(np.float32) / np.float32(np.sqrt(128.0))).astype(np.float16).astype(np.float32)
     m_ref = w.max(-1)
@@ -43,10 +40,9 @@ def test_fused_decode_attention(groups, Bkv, Lc, sparsity):
     assert np.abs(got[:, 0] - m_ref).max() <= 2e-2 * np.maximum(np.abs(m_ref).max(), 1)
     assert np.abs(got[:, 1] * np.exp(got[:, 0] - m_ref) - l_ref).max() <= 5e-3 * l_ref.max()
     # and against the three-launch path
-    s = ops.key_spmv(ck, qg.view(Bq, 1, D), groups)
     p = ops.scale_softmax(s, D)
     o3 = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o.cpu().numpy(), o3.cpu().numpy()[:, 0]) < 2e-3
+    assert rel_err(o.cpu().numpy(), o3.cpu().numpy()[:, 0]) < 2e-3
 
 
 def test_partial_then_merge_equals_fused():
@@ -75,7 +71,7 @@ def test_partial_then_merge_equals_fused():
     M = ml[:, :, 0].max(1, keepdims=True)
     f = np.exp(ml[:, :, 0] - M)
     host = (f[:, :, None] * po).sum(1) / (f * ml[:, :, 1]).sum(1, keepdims=True)
-    assert rel_rowmax(o.cpu().numpy(), host) < 1e-3
+    assert rel_err(o.cpu().numpy(), host) < 1e-3
 
 
 @pytest.mark.parametrize("groups,Bkv,Lc,Lw", [(4, 2, 512, 300), (8, 1, 256, 64), (1, 3, 0, 257), (4, 2, 0, 1), (2, 2, 1024, 511)])
@@ -104,7 +100,7 @@ def test_decode_attention_with_dense_window(groups, Bkv, Lc, Lw):
     vw[:, :Lw] = torch.from_numpy(np.ascontiguousarray(V[:, Lc:])).to(dev)
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev)
     o = ops.decode_attention_window(ck, cv, torch.from_numpy(q).to(dev), kw, vw, Lw, groups, lse=lse)
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3
+    assert rel_err(o.cpu().numpy(), out_ref) < 2e-3
     # the same with the length read on the device and the launch sized for the whole buffer
     wl = torch.tensor([Lw], dtype=torch.int32, device=dev)
     o_dev = ops.decode_attention_window(ck, cv, torch.from_numpy(q).to(dev), kw, vw, cap, groups, win_len_dev=wl)

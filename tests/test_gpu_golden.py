@@ -6,6 +6,8 @@ import numpy as np
 import pytest
 import torch
 
+from _metrics import check_chain, rel_err   # row metric and element-wise allclose(rtol, atol = rtol * rms) in one number
+
 pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -21,11 +23,6 @@ def gpu_f16(a):
 
 def bits(t):
     return t.cpu().numpy().view(np.uint16)
-
-
-def rel_rowmax(a, b):
-    a, b = a.astype(np.float64), b.astype(np.float64)
-    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
 @pytest.mark.parametrize("fused_prune", [True, False])
@@ -54,12 +51,11 @@ def test_attention_reproduces_the_fixture():
     ck = ops.compress(gpu_f16(g["K"]), False, kth=kth)
     cv = ops.compress(gpu_f16(g["V"]), True, kth=kth)
     s = ops.key_spmv(ck, q.view(Bq, 1, D), groups)
-    assert rel_rowmax(s[:, 0].cpu().numpy(), want_s) < 2e-3
     p = ops.scale_softmax(s, D)
-    assert rel_rowmax(p[:, 0].cpu().numpy(), want_p) < 2e-3
     o = ops.value_spmv(cv, p, groups)
-    assert rel_rowmax(o[:, 0].cpu().numpy(), want_o) < 2e-3
-    assert rel_rowmax(ops.decode_attention(ck, cv, q, groups).cpu().numpy(), want_o) < 2e-3
+    Vp = ops.prune_rows(gpu_f16(g["V"]).view(-1, 128), kth).view(-1, want_s.shape[1], 128).cpu().numpy()
+    check_chain(2e-3, want_s, want_p, want_o, Vp, groups, s=s[:, 0], p=p[:, 0], o=o[:, 0],
+                fused=ops.decode_attention(ck, cv, q, groups))
 
 
 @pytest.mark.parametrize("bit", [2, 4])

@@ -12,6 +12,8 @@ import torch
 
 from oracle import oracle as orc
 
+from _metrics import check_chain, rel_err   # row metric and element-wise allclose(rtol, atol = rtol * rms) in one number
+
 pytestmark = pytest.mark.gpu
 
 QTOL = 1e-2  # tolerance of the north-star metric for 4-bit and 2-bit non-zeros
@@ -23,12 +25,6 @@ def dev():
 
 def to_gpu(a):
     return torch.from_numpy(np.ascontiguousarray(a)).to(dev())
-
-
-def rel_rowmax(a, b):
-    a = a.astype(np.float64).reshape(-1, a.shape[-1])
-    b = b.astype(np.float64).reshape(-1, b.shape[-1])
-    return (np.abs(a - b).max(-1) / np.maximum(np.abs(b).max(-1), 1e-30)).max()
 
 
 def pruned(seed, B, M, kth=89):
@@ -87,7 +83,7 @@ def test_quant_formulations_reference_api(bit, dequant_mode):
     assert torch.equal(att, att_meta)
     C, Cf = orc.spmv_quant(rk[0], rk[2], rk[1], rk[5], rk[6], padded_query.cpu().numpy(), 0, Lc, D, groups, bit,
                            dequant_mode)
-    assert rel_rowmax(att.cpu().numpy()[:, 0], Cf[:, 0]) < 2e-3
+    assert rel_err(att.cpu().numpy()[:, 0], Cf[:, 0]) < 2e-3
     assert not att[:, 1:].any()
 
     P = orc.scale_softmax(C[:, 0], D)
@@ -98,11 +94,11 @@ def test_quant_formulations_reference_api(bit, dequant_mode):
     assert tuple(out.shape) == (Bq, 8, D)
     O, Of = orc.spmv_quant(rv[0], rv[2], rv[1], rv[5], rv[6], padded_score.cpu().numpy(), 1, Lc, D, groups, bit,
                            dequant_mode)
-    assert rel_rowmax(out.cpu().numpy()[:, 0], Of[:, 0]) < 2e-3
+    assert rel_err(out.cpu().numpy()[:, 0], Of[:, 0]) < 2e-3
     n1 = mq.mustafar_value_formulation_quant_decode_n1(vb, vp, vo, vc, vu, vs, vz, to_gpu(P), ws, D, Lc, Bq, groups,
                                                        bit, cap, dequant_mode)
     assert tuple(n1.shape) == (Bq, D)
-    assert rel_rowmax(n1.cpu().numpy(), Of[:, 0]) < 2e-3
+    assert rel_err(n1.cpu().numpy(), Of[:, 0]) < 2e-3
     with pytest.raises(RuntimeError):
         mq.mustafar_key_formulation_quant(kb, kp, ko, ks.float(), kz, padded_query, Lc, D, Bq, groups, bit, cap)
     with pytest.raises(RuntimeError):   # capacity must be 32 // bit
@@ -135,12 +131,10 @@ def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc
     qg = to_gpu(q).view(Bq, 1, D)
     assert L.mstf_key_spmv_quant(st, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), None, None, ks.data_ptr(),
                                  kz.data_ptr(), qg.data_ptr(), s.data_ptr(), Lc, D, Bq, groups, 1, bit, cap, 0) == 0
-    assert rel_rowmax(s.cpu().numpy()[:, 0], sc_ref) < QTOL
     p = ops.scale_softmax(s, D)
     o = mq.mustafar_value_formulation_quant_decode_n1(vb, vp, vo, vc, vu, vs, vz, p.view(Bq, Lc), None, D, Lc, Bq,
                                                       groups, bit, cap)
-    assert rel_rowmax(p.cpu().numpy()[:, 0], pr_ref) < QTOL
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
+    check_chain(QTOL, sc_ref, pr_ref, out_ref, Vd, groups, s=s[:, 0], p=p[:, 0], o=o)
     # the quantisation itself stays within half a step of the fp16 cache
     err = np.abs(Kd.astype(np.float32) - np.where(Kp != 0, Kp, 0).astype(np.float32))
     step = np.repeat(rk[5].astype(np.float32).reshape(Bkv, Lc // 64, D), 64, axis=1)   # key tile = 64 tokens x 1 channel
@@ -219,22 +213,22 @@ def test_fused_quant_decode_attention(bit, groups, Bkv, Lc):
     Kd = np.stack([orc.decode_quant(kr[0], kr[2], kr[1], kr[5], kr[6], b, Lc, D, 0, bit) for b in range(Bkv)])
     Vd = np.stack([orc.decode_quant(vr[0], vr[2], vr[1], vr[5], vr[6], b, Lc, D, 1, bit) for b in range(Bkv)])
     q = np.random.default_rng(bit + Lc).standard_normal((Bq, D)).astype(np.float16)
-    _, _, out_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
+    sc_ref, pr_ref, out_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
     lse = torch.empty((Bq, 2), dtype=torch.float32, device=dev())
     o = mpq.decode_attention_quant(kq, vq, to_gpu(q), groups, bit, lse=lse)
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < 2e-3      # the cache is the same dequantised one: fp16 accuracy
     o2 = mpq.decode_attention_quant(kq, vq, to_gpu(q), groups, bit)
-    assert torch.equal(o, o2) or rel_rowmax(o2.cpu().numpy(), o.cpu().numpy()) < 1e-3
+    assert torch.equal(o, o2) or rel_err(o2.cpu().numpy(), o.cpu().numpy()) < 1e-3
     # three-launch path
     qp = np.zeros((Bq, 8, D), np.float16)
     qp[:, 0] = q
     s = mpq.mustafar_key_formulation_quant_meta(kq[0], kq[2], kq[1], kq[3], kq[4], kq[5], kq[6], to_gpu(qp), Lc, D, Bq,
                                                 groups, bit, 32 // bit)[:, 0].contiguous()
+    # the cache is the same dequantised one on both sides: fp16 accuracy, well inside the 1e-2 of the quantised path
+    check_chain(2e-3, sc_ref, pr_ref, out_ref, Vd, groups, s=s, fused=o)
     p = ops.scale_softmax(s, D)
     o3 = mpq.mustafar_value_formulation_quant_decode_n1(vq[0], vq[2], vq[1], vq[3], vq[4], vq[5], vq[6], p, None, D, Lc,
                                                         Bq, groups, bit, 32 // bit)
-    assert rel_rowmax(o.cpu().numpy(), o3.cpu().numpy()) < 2e-3
+    assert rel_err(o.cpu().numpy(), o3.cpu().numpy()) < 2e-3
 
 
 def test_quant_c_abi_rejects_bad_arguments():
@@ -278,7 +272,7 @@ def test_quant_decode_attention_with_dense_window(bit, groups, Bkv, Lc, Lw):
     kw[:, :Lw] = to_gpu(K[:, Lc:])
     vw[:, :Lw] = to_gpu(V[:, Lc:])
     o = mpq.decode_attention_window_quant(kq, vq, to_gpu(q), kw, vw, Lw, groups, bit)
-    assert rel_rowmax(o.cpu().numpy(), out_ref) < QTOL
+    assert rel_err(o.cpu().numpy(), out_ref) < QTOL
     wl = torch.tensor([Lw], dtype=torch.int32, device=dev())
     o_dev = mpq.decode_attention_window_quant(kq, vq, to_gpu(q), kw, vw, cap, groups, bit, win_len_dev=wl)
     assert torch.equal(o_dev, o)
