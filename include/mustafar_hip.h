@@ -281,6 +281,36 @@ int mstf_decode_attention_window_quant(void* stream, const uint64_t* k_bmp, cons
                                        int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
                                        int dequant_mode, void* workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------------------------ group-32 scale / zero option
+ * No counterpart in the reference's kernels: its harness carries GROUP_SIZE = 32 (benchmark/mem_spd_test_quant.py:33,
+ * 104) but the producer quantises per 64-element tile (kernel_quant/compression_quant.py:47-57, 209-210).  With
+ * group_size 32 every tile has two (scale, zero) pairs, scales / zeros are fp16 [B][T][2] (4-byte aligned), pair g
+ * serves the elements 32g .. 32g+31 of the tile and is computed from the minimum and maximum of that half's kept
+ * elements by the formulas above; bitmaps, counts, units, tile_off and the rank-ordered packing of the codes are
+ * unchanged (the first popcount(upper bitmap half) codes of a tile belong to pair 0).  group_size 64 is the layout of
+ * the entry points above.  Otherwise the arguments are those of mstf_compress_{key,value}_quant (is_value picks the
+ * tile orientation), mstf_key_spmv_quant, mstf_value_spmv_quant and mstf_decode_attention_quant, without the unused
+ * counts / units of the consumers. */
+int mstf_compress_quant_grouped(void* stream, const mstf_half* x, int is_value, int B, int M, int N, int kth, int bit,
+                                int group_size, uint64_t* bmp, uint32_t* tile_off, uint32_t* counts, uint32_t* units,
+                                mstf_half* scales, mstf_half* zeros, uint64_t* total_words, uint32_t* packed,
+                                uint64_t packed_capacity_words, void* workspace, size_t workspace_bytes);
+int mstf_key_spmv_quant_grouped(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                                const mstf_half* scales, const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M,
+                                int K, int Bq, int groups, int n_rows, int bit, int capacity, int dequant_mode,
+                                int group_size);
+int mstf_value_spmv_quant_grouped(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                                  const mstf_half* scales, const mstf_half* zeros, const mstf_half* P, mstf_half* C, int M,
+                                  int K, int Bq, int groups, int n_rows, int bit, int capacity, int dequant_mode,
+                                  int group_size, void* workspace, size_t workspace_bytes);
+int mstf_decode_attention_quant_grouped(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                        const uint32_t* k_tile_off, const mstf_half* k_scales, const mstf_half* k_zeros,
+                                        const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+                                        const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q,
+                                        mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq, int groups,
+                                        int bit, int capacity, int dequant_mode, int group_size, void* workspace,
+                                        size_t workspace_bytes);
+
 
 #ifdef __cplusplus
 }

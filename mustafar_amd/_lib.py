@@ -66,6 +66,11 @@ SIGNATURES = {
     "mstf_value_spmv_quant": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _sz]),
     "mstf_decode_attention_quant": (_i, [_vp] * 14 + [_i, _i, _i, _i, _i, _i, _i, _vp, _sz]),
+    "mstf_compress_quant_grouped": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64,
+                                         _vp, _sz]),
+    "mstf_key_spmv_quant_grouped": (_i, [_vp] * 8 + [_i] * 9),
+    "mstf_value_spmv_quant_grouped": (_i, [_vp] * 8 + [_i] * 9 + [_vp, _sz]),
+    "mstf_decode_attention_quant_grouped": (_i, [_vp] * 14 + [_i] * 8 + [_vp, _sz]),
     "mstf_decode_attention_window_quant": (_i, [_vp] * 14 + [_i, _vp, _i, _vp, _vp] + [_i] * 7 + [_vp, _sz]),
 }
 

@@ -1,6 +1,7 @@
 """Drop-in for the reference's kernel_quant/compression_quant.py (convert_key_batched_quant :159-264,
 convert_value_batched_quant :425-529): same arguments and return tuples.  The reference hard-codes
-2-bit codes; `bit` is exposed here as an extra keyword (2, 4 or 8; capacity = 32 // bit).
+2-bit codes; `bit` is exposed here as an extra keyword (2, 4 or 8; capacity = 32 // bit), and `group_size`
+(64 = one scale / zero pair per tile as in the reference; 32 = two, scales and zeros then [B, T, 2]).
 
 inputs: [B, M, N] fp16 on the GPU, already pruned, M % 64 == 0.
 """
@@ -10,7 +11,7 @@ from . import ops
 from ._lib import check, lib
 
 
-def _convert(inputs, is_value, bit, kth=0):
+def _convert(inputs, is_value, bit, kth=0, group_size=64):
     assert inputs.is_cuda
     assert inputs.dim() == 3
     B, M, N = inputs.shape
@@ -25,32 +26,35 @@ def _convert(inputs, is_value, bit, kth=0):
     tile_off = torch.empty((B, T), dtype=torch.int32, device=dev)
     counts = torch.empty((B, T), dtype=torch.int32, device=dev)
     units = torch.empty((B, T), dtype=torch.int32, device=dev)
-    scales = torch.empty((B, T), dtype=torch.float16, device=dev)
-    zeros = torch.empty((B, T), dtype=torch.float16, device=dev)
+    if group_size not in (32, 64):
+        raise RuntimeError("group_size must be 32 or 64")
+    meta_shape = (B, T) if group_size == 64 else (B, T, 2)
+    scales = torch.empty(meta_shape, dtype=torch.float16, device=dev)
+    zeros = torch.empty(meta_shape, dtype=torch.float16, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
     ws = ops.workspace(dev, L.mstf_compress_quant_workspace_bytes(B, M, N))
-    fn = L.mstf_compress_value_quant if is_value else L.mstf_compress_key_quant
-    name = "mstf_compress_value_quant" if is_value else "mstf_compress_key_quant"
+    name = "mstf_compress_quant_grouped"
     st = torch.cuda.current_stream().cuda_stream
     # one pass with room for the worst case (every element kept: 64 // capacity words per tile), then the used
     # part is copied out so that the large buffer goes back to the allocator; the total is read once on the host, as
     # the reference's .item() does
     cap_words = B * T * (64 * int(bit) // 32)
     room = torch.empty((max(cap_words, 1),), dtype=torch.int32, device=dev)
-    check(fn(st, x.data_ptr(), B, M, N, int(kth), int(bit), bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(),
-             units.data_ptr(), scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,
-             ws.data_ptr(), ws.numel()), name)
+    check(L.mstf_compress_quant_grouped(st, x.data_ptr(), int(bool(is_value)), B, M, N, int(kth), int(bit), int(group_size),
+                                        bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(), units.data_ptr(),
+                                        scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,
+                                        ws.data_ptr(), ws.numel()), name)
     n = int(total.item())
     packed = room[:n].clone()
     return bmp, tile_off, packed, counts, units, scales, zeros
 
 
-def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2):
-    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit)
+def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2, group_size: int = 64):
+    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit, group_size=group_size)
     if return_metadata:
         return bmp, tile_off, packed, counts, units, scales, zeros
     return bmp, tile_off, packed, scales, zeros
 
 
-def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2):
-    return _convert(inputs, True, bit)
+def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2, group_size: int = 64):
+    return _convert(inputs, True, bit, group_size=group_size)

@@ -24,7 +24,7 @@ struct QSide {
 };
 
 // grid = (token splits, KV heads), kFusedWaves wavefronts; see decode_attention_kernel.
-template <int NM, int BIT>
+template <int NM, int BIT, bool G32>
 __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kernel(
     const uint64_t* __restrict__ k_bmp, const uint32_t* k_packed, const uint32_t* __restrict__ k_off,
     const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros, const uint64_t* __restrict__ v_bmp,
@@ -37,7 +37,8 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
     constexpr int kQLds = NM * 4 * D * 2;
     constexpr int kPRow = 64 * 2;
     constexpr int kPLds = NM * 4 * kPRow;
-    constexpr int kStage = q_lds_bytes<BIT>();  // image, zero slot, two word buffers, two metadata buffers
+    constexpr int kMetaBytes = meta_bytes<G32>();
+    constexpr int kStage = q_lds_bytes<BIT, G32>();  // image, zero slot, two word buffers, two metadata buffers
     constexpr int kNeed = kStage + kQLds + kPLds;
     constexpr int kPark = NM * 4 * D * 4 + 64;
     constexpr int kWaveLds = kNeed > kPark ? kNeed : kPark;
@@ -71,8 +72,11 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
 
     if (active) {
         const size_t tile0 = (size_t)kv * T + (size_t)tb * D;  // tile_off / scales / zeros / bmp are flat over [Bkv, T]
-        const QSide K = {k_bmp + tile0, k_packed, k_off + tile0, k_off_dma + tile0, k_scales + tile0, k_zeros + tile0};
-        const QSide V = {v_bmp + tile0, v_packed, v_off + tile0, v_off_dma + tile0, v_scales + tile0, v_zeros + tile0};
+        constexpr size_t kPairs = G32 ? 2 : 1;  // (scale, zero) pairs per tile
+        const QSide K = {k_bmp + tile0, k_packed, k_off + tile0, k_off_dma + tile0, k_scales + tile0 * kPairs,
+                         k_zeros + tile0 * kPairs};
+        const QSide V = {v_bmp + tile0, v_packed, v_off + tile0, v_off_dma + tile0, v_scales + tile0 * kPairs,
+                         v_zeros + tile0 * kPairs};
         if (lane < 4) reinterpret_cast<uint32_t*>(my + kImgBytes)[lane] = 0u;
         // word offsets at the stage boundaries of both sides by one vector load (lanes 0.. keys, 16.. values); the
         // block's last stage ends where its last tile's words end
@@ -92,15 +96,15 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             if (n == kKeySubs + kValSubs - 1) return endV;
             return start_of(n + 1);
         };
-        const MetaLane metaK = meta_lane(K.off_dma, K.scales, K.zeros, lane);
-        const MetaLane metaV = meta_lane(V.off_dma, V.scales, V.zeros, lane);
+        const MetaLanes metaK = meta_lanes<G32>(K.off_dma, K.scales, K.zeros, K.bmp, lane);
+        const MetaLanes metaV = meta_lanes<G32>(V.off_dma, V.scales, V.zeros, V.bmp, lane);
         const uint32_t lane4 = (uint32_t)lane * 4u;
         const uint32_t touch8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
         const uint32_t wordbuf_lds = lds_addr(wordbuf);
         // (no lane-dependent branches: every piece is issued with exec set by hand or from a clamped address)
         auto issue = [&](int n) {
             const QSide& S = n < kKeySubs ? K : V;
-            const MetaLane& ML = n < kKeySubs ? metaK : metaV;
+            const MetaLanes& ML = n < kKeySubs ? metaK : metaV;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             const uint32_t s = start_of(n);
             uint32_t nw = end_of(n) - s;
@@ -108,7 +112,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             words_issue_flat<F::kWordsMax / 64>(S.packed + s, nw, wordbuf_lds + (uint32_t)(n & 1) * F::kWordBuf,
                                                 (uint32_t)lane, lane4);
             // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane)
-            dma4(ML.at((uint32_t)t), metabuf + (n & 1) * kMetaBytes);
+            meta_issue<G32>(ML, (uint32_t)t, metabuf + (n & 1) * kMetaBytes);
             // pulls the stage's bitmaps into L2 ahead of the scalar loads of the expansion
             return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(S.bmp + t) + touch8);
         };
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         auto stage = [&](int n, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
             const QSide& S = n < kKeySubs ? K : V;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
-            dequant_stage<BIT>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
+            dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
                                lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), lane, mode);
             stage_img_exec<NM>(S.bmp + t, lbase, zaddr, waddr, wgroup, acc);
         };
@@ -170,11 +174,16 @@ static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp
                                 const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_off,
                                 const uint16_t* v_scales, const uint16_t* v_zeros, const _Float16* q, _Float16* out,
                                 float* part_o, float* part_ml, int tokens, int groups, int ns, int write_final, float sq,
-                                int mode)
+                                int mode, int group_size)
 {
-    hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, k_packed, k_off,
-                       k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q, out, part_o, part_ml,
-                       tokens, groups, tokens / 64, ns, write_final, sq, mode);
+    if (group_size == 32)
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
+                           k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
+                           out, part_o, part_ml, tokens, groups, tokens / 64, ns, write_final, sq, mode);
+    else
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
+                           k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
+                           out, part_o, part_ml, tokens, groups, tokens / 64, ns, write_final, sq, mode);
 }
 
 }  // namespace mstf
@@ -208,7 +217,8 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
                         const mstf_half* k_scales, const mstf_half* k_zeros, const uint64_t* v_bmp,
                         const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
                         const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
-                        int groups, int bit, int dequant_mode, void* workspace, int nst, int write_final)
+                        int groups, int bit, int dequant_mode, void* workspace, int nst, int write_final,
+                        int group_size = 64)
 {
     const int Bkv = Bq / groups, ns = fused_nsplit(tokens);
     float* part_o = reinterpret_cast<float*>(workspace);
@@ -223,7 +233,7 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
     const uint16_t* vz = reinterpret_cast<const uint16_t*>(v_zeros);
 #define MSTF_FQ(NMV, BITV)                                                                                             \
     launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, ks, kz, v_bmp, v_packed, v_tile_off, vs, vz, \
-                                   qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode)
+                                   qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode, group_size)
     if (groups <= 4) {
         if (bit == 2) MSTF_FQ(1, 2); else if (bit == 4) MSTF_FQ(1, 4); else MSTF_FQ(1, 8);
     } else {
@@ -233,15 +243,16 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
     return check_launch();
 }
 
-extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
-                                           const uint32_t* k_tile_off, const mstf_half* k_scales,
-                                           const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
-                                           const uint32_t* v_tile_off, const mstf_half* v_scales,
-                                           const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out,
-                                           int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
-                                           int dequant_mode, void* workspace, size_t workspace_bytes)
+static int decode_attention_quant_impl(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                       const uint32_t* k_tile_off, const mstf_half* k_scales, const mstf_half* k_zeros,
+                                       const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+                                       const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q,
+                                       mstf_half* out, float* lse_out, int tokens, int head_dim, int Bq, int groups,
+                                       int bit, int capacity, int dequant_mode, int group_size, void* workspace,
+                                       size_t workspace_bytes)
 {
     if (!out) return MSTF_EINVAL;
+    if (group_size != 64 && group_size != 32) return MSTF_EUNSUPPORTED;
     int rc = quant_check(k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
                          tokens, head_dim, Bq, groups, bit, capacity, dequant_mode);
     if (rc != MSTF_OK) return rc;
@@ -254,9 +265,37 @@ extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, 
     // with one split and no (max, sum) requested the kernel writes the final output itself
     const int write_final = (ns == 1 && !lse_out) ? 1 : 0;
     rc = quant_launch(st, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
-                      out, tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, ns, write_final);
+                      out, tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, ns, write_final, group_size);
     if (rc != MSTF_OK || write_final) return rc;
     return merge_splits(st, workspace, out, lse_out, ns, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_attention_quant(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                           const uint32_t* k_tile_off, const mstf_half* k_scales,
+                                           const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
+                                           const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                           const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, float* lse_out,
+                                           int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
+                                           int dequant_mode, void* workspace, size_t workspace_bytes)
+{
+    return decode_attention_quant_impl(stream, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off,
+                                       v_scales, v_zeros, q, out, lse_out, tokens, head_dim, Bq, groups, bit, capacity,
+                                       dequant_mode, 64, workspace, workspace_bytes);
+}
+
+extern "C" int mstf_decode_attention_quant_grouped(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                                   const uint32_t* k_tile_off, const mstf_half* k_scales,
+                                                   const mstf_half* k_zeros, const uint64_t* v_bmp,
+                                                   const uint32_t* v_packed, const uint32_t* v_tile_off,
+                                                   const mstf_half* v_scales, const mstf_half* v_zeros,
+                                                   const mstf_half* q, mstf_half* out, float* lse_out, int tokens,
+                                                   int head_dim, int Bq, int groups, int bit, int capacity,
+                                                   int dequant_mode, int group_size, void* workspace,
+                                                   size_t workspace_bytes)
+{
+    return decode_attention_quant_impl(stream, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off,
+                                       v_scales, v_zeros, q, out, lse_out, tokens, head_dim, Bq, groups, bit, capacity,
+                                       dequant_mode, group_size, workspace, workspace_bytes);
 }
 
 extern "C" int mstf_decode_attention_window_quant(

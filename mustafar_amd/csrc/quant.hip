@@ -18,7 +18,9 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits) { return (flo
 // ------------------------------------------------------------------------------- producer: count
 // grid = B * M/64 units, 64 threads.  Lane l owns tiles l and 64+l of the unit: bitmap, raw count,
 // units, scale, zero; tile_off gets the unit-local exclusive word offset, unit_tot the unit total.
-template <bool IS_VALUE>
+// G32: two (scale, zero) pairs per tile, pair g from the kept elements 32g .. 32g+31 of the tile; scales / zeros are
+// then [B][T][2].
+template <bool IS_VALUE, bool G32>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void quant_count_kernel(const _Float16* __restrict__ x, int M, int kth, int bit,
                                                          uint64_t* __restrict__ bmp, uint32_t* __restrict__ counts,
                                                          uint32_t* __restrict__ units, uint32_t* __restrict__ tile_off,
@@ -58,47 +60,62 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void qu
     uint32_t u[2];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        float mn = INFINITY, mx = -INFINITY;
+        constexpr int NG = G32 ? 2 : 1;
+        float mn[NG], mx[NG];
         const uint64_t m = bm[h];
         if (IS_VALUE) {
-            // tile (h, token = lane): the lane's own 64 channels, two per register
+            // tile (h, token = lane): the lane's own 64 channels, two per register; group g = registers 16g .. 16g+15
             typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
-            h2v_t mn2 = {(_Float16)INFINITY, (_Float16)INFINITY}, mx2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
 #pragma unroll
-            for (int j = 0; j < 32; j++) {
-                const h2v_t v = __builtin_bit_cast(h2v_t, r[32 * h + j]);
-                mn2 = __builtin_elementwise_min(mn2, v);
-                mx2 = __builtin_elementwise_max(mx2, v);
+            for (int g = 0; g < NG; g++) {
+                h2v_t mn2 = {(_Float16)INFINITY, (_Float16)INFINITY}, mx2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+#pragma unroll
+                for (int j = g * (32 / NG); j < (g + 1) * (32 / NG); j++) {
+                    const h2v_t v = __builtin_bit_cast(h2v_t, r[32 * h + j]);
+                    mn2 = __builtin_elementwise_min(mn2, v);
+                    mx2 = __builtin_elementwise_max(mx2, v);
+                }
+                mn[g] = fminf((float)mn2[0], (float)mn2[1]);
+                mx[g] = fmaxf((float)mx2[0], (float)mx2[1]);
             }
-            mn = fminf((float)mn2[0], (float)mn2[1]);
-            mx = fmaxf((float)mx2[0], (float)mx2[1]);
         } else {
-            // tile = channel 64h + lane over the 64 tokens: the half-slab back into LDS, the lane walks its column
+            // tile = channel 64h + lane over the 64 tokens: the half-slab back into LDS, the lane walks its column;
+            // group g = tokens 32g .. 32g+31
 #pragma unroll
             for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
             __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                float a = INFINITY, z = -INFINITY;
 #pragma unroll 8
-            for (int i = 0; i < 64; i++) {
-                const float v = (float)sh[i * (2 * kHalfRowDw) + lane];
-                mn = fminf(mn, v);
-                mx = fmaxf(mx, v);
+                for (int i = g * (64 / NG); i < (g + 1) * (64 / NG); i++) {
+                    const float v = (float)sh[i * (2 * kHalfRowDw) + lane];
+                    a = fminf(a, v);
+                    z = fmaxf(z, v);
+                }
+                mn[g] = a;
+                mx[g] = z;
             }
             __builtin_amdgcn_wave_barrier();
         }
         const uint32_t cnt = (uint32_t)__popcll(m);
-        float scale = 1.f, zero = 0.f;
-        if (cnt > 0) {
-            scale = (mx - mn) / maxq;
-            if (scale == 0.f) scale = 1.f;
-            zero = floorf(-mn / scale + 0.5f);
-        }
         const size_t ti = tile0 + (size_t)h * 64 + lane;
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            // an empty group leaves the minimum at +inf: scale 1, zero 0, as for an empty tile
+            float scale = 1.f, zero = 0.f;
+            if (mn[g] <= mx[g]) {
+                scale = (mx[g] - mn[g]) / maxq;
+                if (scale == 0.f) scale = 1.f;
+                zero = floorf(-mn[g] / scale + 0.5f);
+            }
+            scales[ti * NG + g] = (_Float16)scale;
+            zeros[ti * NG + g] = (_Float16)zero;
+        }
         bmp[ti] = m;
         counts[ti] = cnt;
         u[h] = (cnt + (uint32_t)cap - 1u) / (uint32_t)cap;
         units[ti] = u[h];
-        scales[ti] = (_Float16)scale;
-        zeros[ti] = (_Float16)zero;
     }
     uint32_t totA, totB;
     const uint32_t eA = wave_excl_scan(u[0], lane, totA);
@@ -142,7 +159,7 @@ __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restric
 // ------------------------------------------------------------------------------- producer: pack
 // grid = B * M/64 units, 64 threads; every lane quantises and packs its two tiles.  tile_off still holds the
 // unit-local offsets of the count kernel and is completed here with the unit's and the head's base.
-template <bool IS_VALUE>
+template <bool IS_VALUE, bool G32>
 __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restrict__ x, int M, int bit,
                                                         const uint64_t* __restrict__ bmp,
                                                         const uint32_t* __restrict__ units, uint32_t* tile_off,
@@ -172,9 +189,14 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
         const uint64_t off = (uint64_t)tile_off[ti] + ubase;
         tile_off[ti] = (uint32_t)off;
         if (off + units[ti] > capacity_words) continue;  // would not fit: leave untouched
-        float sc = (float)scales[ti];
-        const float zp = (float)zeros[ti];
-        if (sc == 0.f) sc = 1.f;
+        constexpr int NG = G32 ? 2 : 1;
+        float scg[NG], zpg[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            scg[g] = (float)scales[ti * NG + g];
+            zpg[g] = (float)zeros[ti * NG + g];
+            if (scg[g] == 0.f) scg[g] = 1.f;
+        }
         uint32_t cur = 0;
         int pos = 0;
         uint32_t w = 0;
@@ -185,6 +207,8 @@ __global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restri
             rem &= ~(0x8000000000000000ull >> i);
             const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
             const float v = (float)sh[e];
+            const float sc = (G32 && i >= 32) ? scg[NG - 1] : scg[0];   // the element's position picks the pair
+            const float zp = (G32 && i >= 32) ? zpg[NG - 1] : zpg[0];
             float q = floorf(v / sc + 0.5f) + zp;
             q = fminf(fmaxf(q, 0.f), maxq);
             cur |= (uint32_t)q << pos;
@@ -216,7 +240,7 @@ static size_t quant_ws_bytes(int B, int M)
     return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
 }
 
-template <bool IS_VALUE>
+template <bool IS_VALUE, bool G32>
 static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit, uint64_t* bmp,
                                uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,
                                mstf_half* zeros, uint64_t* total_words, uint32_t* packed, uint64_t cap_words, void* ws,
@@ -227,7 +251,7 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     if (cap_shift_of(bit) < 0) return MSTF_EUNSUPPORTED;
     if (N != kD || M % 64 != 0 || M / 64 > 8192 || (int64_t)B * (M / 64) > 0x7FFFFFFF) return MSTF_EUNSUPPORTED;
     if (!aligned_to(x, 16) || !aligned_to(bmp, 8) || !aligned_to(tile_off, 4) || !aligned_to(counts, 4) ||
-        !aligned_to(units, 4) || !aligned_to(scales, 2) || !aligned_to(zeros, 2) || !aligned_to(total_words, 8) ||
+        !aligned_to(units, 4) || !aligned_to(scales, G32 ? 4 : 2) || !aligned_to(zeros, G32 ? 4 : 2) || !aligned_to(total_words, 8) ||
         (packed && !aligned_to(packed, 4)))
         return MSTF_EALIGN;
     if (!ws || ws_bytes < quant_ws_bytes(B, M)) return MSTF_EWORKSPACE;
@@ -242,7 +266,7 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     uint32_t* head_base = reinterpret_cast<uint32_t*>(w + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     int rc;
-    hipLaunchKernelGGL(quant_count_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bit, bmp,
+    hipLaunchKernelGGL((quant_count_kernel<IS_VALUE, G32>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bit, bmp,
                        counts, units, tile_off, reinterpret_cast<_Float16*>(scales), reinterpret_cast<_Float16*>(zeros),
                        unit_tot);
     if ((rc = check_launch()) != MSTF_OK) return rc;
@@ -250,7 +274,7 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
                        head_base, total_words, nblk);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     if (packed) {
-        hipLaunchKernelGGL(quant_pack_kernel<IS_VALUE>, dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bit, bmp,
+        hipLaunchKernelGGL((quant_pack_kernel<IS_VALUE, G32>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bit, bmp,
                            units, tile_off, unit_base, head_base, reinterpret_cast<const _Float16*>(scales),
                            reinterpret_cast<const _Float16*>(zeros), packed, cap_words);
     } else {
@@ -271,13 +295,29 @@ extern "C" size_t mstf_compress_quant_workspace_bytes(int B, int M, int N)
     return quant_ws_bytes(B, M);
 }
 
+// group_size 64: one (scale, zero) pair per tile (the reference); 32: two, scales / zeros [B][T][2].
+template <bool IS_VALUE>
+static int compress_quant_group(int group_size, void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit,
+                                uint64_t* bmp, uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,
+                                mstf_half* zeros, uint64_t* total_words, uint32_t* packed, uint64_t cap_words, void* ws,
+                                size_t ws_bytes)
+{
+    if (group_size == 64)
+        return compress_quant_impl<IS_VALUE, false>(stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
+                                                    total_words, packed, cap_words, ws, ws_bytes);
+    if (group_size == 32)
+        return compress_quant_impl<IS_VALUE, true>(stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
+                                                   total_words, packed, cap_words, ws, ws_bytes);
+    return MSTF_EUNSUPPORTED;
+}
+
 extern "C" int mstf_compress_key_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit,
                                        uint64_t* bmp, uint32_t* tile_off, uint32_t* counts, uint32_t* units,
                                        mstf_half* scales, mstf_half* zeros, uint64_t* total_words, uint32_t* packed,
                                        uint64_t packed_capacity_words, void* workspace, size_t workspace_bytes)
 {
-    return compress_quant_impl<false>(stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
-                                      total_words, packed, packed_capacity_words, workspace, workspace_bytes);
+    return compress_quant_group<false>(64, stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
+                                       total_words, packed, packed_capacity_words, workspace, workspace_bytes);
 }
 
 extern "C" int mstf_compress_value_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit,
@@ -285,6 +325,19 @@ extern "C" int mstf_compress_value_quant(void* stream, const mstf_half* x, int B
                                          mstf_half* scales, mstf_half* zeros, uint64_t* total_words, uint32_t* packed,
                                          uint64_t packed_capacity_words, void* workspace, size_t workspace_bytes)
 {
-    return compress_quant_impl<true>(stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
-                                     total_words, packed, packed_capacity_words, workspace, workspace_bytes);
+    return compress_quant_group<true>(64, stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales, zeros,
+                                      total_words, packed, packed_capacity_words, workspace, workspace_bytes);
+}
+
+extern "C" int mstf_compress_quant_grouped(void* stream, const mstf_half* x, int is_value, int B, int M, int N, int kth,
+                                           int bit, int group_size, uint64_t* bmp, uint32_t* tile_off, uint32_t* counts,
+                                           uint32_t* units, mstf_half* scales, mstf_half* zeros, uint64_t* total_words,
+                                           uint32_t* packed, uint64_t packed_capacity_words, void* workspace,
+                                           size_t workspace_bytes)
+{
+    if (is_value)
+        return compress_quant_group<true>(group_size, stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales,
+                                          zeros, total_words, packed, packed_capacity_words, workspace, workspace_bytes);
+    return compress_quant_group<false>(group_size, stream, x, B, M, N, kth, bit, bmp, tile_off, counts, units, scales,
+                                       zeros, total_words, packed, packed_capacity_words, workspace, workspace_bytes);
 }

@@ -18,11 +18,19 @@ struct QFmt {
     static constexpr int kWordBuf = kWordsMax * 4 + 64;         // + room for the lanes past a tile's last word
 };
 constexpr int kImgBytes = kSubTiles * 128;   // fp16 image of a stage: 64 slots per tile
-constexpr int kMetaBytes = 256;              // 32 word offsets, 32 scales, 32 zero-points
-template <int BIT>
+// Staged metadata of a stage.  One (scale, zero) pair per tile: 32 word offsets, 32 scales, 32 zero-points (256 bytes,
+// one LDS-direct load).  Two pairs per tile (G32: pair g for the elements 32g .. 32g+31): 32 word offsets, 32 x 2
+// scales, 32 x 2 zero-points and the upper halves of the 32 bitmaps (their popcount is the number of codes that
+// belong to the first pair), 128 bytes each, two LDS-direct loads.
+template <bool G32>
+constexpr int meta_bytes()
+{
+    return G32 ? 512 : 256;
+}
+template <int BIT, bool G32 = false>
 constexpr int q_lds_bytes()
 {
-    return kImgBytes + 16 + 2 * QFmt<BIT>::kWordBuf + 2 * kMetaBytes;
+    return kImgBytes + 16 + 2 * QFmt<BIT>::kWordBuf + 2 * meta_bytes<G32>();
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t bits) { return (float)as_h((uint16_t)bits); }
@@ -48,60 +56,94 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, h2_t neg_bias, 
 // writes that word's values to the tile image.  Lanes past a tile's last word decode whatever follows in
 // the staged buffer into image slots no rank ever points to.
 //   meta  : LDS address of the staged metadata; words: LDS address of the staged words, word 0 = `start_word`
-template <int BIT>
+template <int BIT, bool G32 = false>
 __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uint32_t img, uint32_t start_word, int lane,
                                               int mode)
 {
     using F = QFmt<BIT>;
+    typedef short s2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int p = 0; p < F::kPasses; p++) {
         const uint32_t tl = (uint32_t)(p * F::kTilesPerPass + lane / F::kSlots);
         const uint32_t slot = (uint32_t)(lane % F::kSlots);
         const uint32_t off = lds_load_u32(meta + tl * 4u);
-        const uint32_t sc = lds_load_u16(meta + 128u + tl * 2u);
-        const uint32_t zp = lds_load_u16(meta + 192u + tl * 2u);
+        // sc / zp: the pair of the tile (low half) or, G32, both pairs (first in the low half)
+        const uint32_t sc = G32 ? lds_load_u32(meta + 128u + tl * 4u) : lds_load_u16(meta + 128u + tl * 2u);
+        const uint32_t zp = G32 ? lds_load_u32(meta + 256u + tl * 4u) : lds_load_u16(meta + 192u + tl * 2u);
+        // G32: the codes of this word that belong to the first pair, 0 .. kCap (codes are in rank order over the whole
+        // tile; the first popcount(upper bitmap half) of them sit in elements 0 .. 31)
+        int kb = F::kCap;
+        if (G32) {
+            const int c0 = __builtin_popcount(lds_load_u32(meta + 384u + tl * 4u));
+            kb = c0 - (int)slot * F::kCap;
+            kb = kb < 0 ? 0 : (kb > F::kCap ? F::kCap : kb);
+        }
         const uint32_t w = lds_load_u32(words + (off - start_word + slot) * 4u);
         const uint32_t dst = img + tl * 128u + slot * (uint32_t)(F::kCap * 2);
-        if ((zp & 0x7fffu) <= 0x6400u) {
+        const bool small_zero = G32 ? ((zp & 0x7fffu) <= 0x6400u && ((zp >> 16) & 0x7fffu) <= 0x6400u)
+                                    : ((zp & 0x7fffu) <= 0x6400u);
+        if (small_zero) {
             const _Float16 nb = (_Float16)(-1024.0f) - as_h((uint16_t)zp);  // exact: |zero| <= 1024
             const _Float16 sh = as_h((uint16_t)sc);
-            const h2_t neg_bias = {nb, nb};
-            const h2_t scale2 = {sh, sh};
+            const h2_t nb_a = {nb, nb};
+            const h2_t sc_a = {sh, sh};
+            uint32_t nb_b = 0u, sc_b = 0u, kb2 = 0u;
+            if (G32) {
+                const _Float16 nb1 = (_Float16)(-1024.0f) - as_h((uint16_t)(zp >> 16));
+                const _Float16 sh1 = as_h((uint16_t)(sc >> 16));
+                nb_b = as_u32(h2_t{nb1, nb1});
+                sc_b = as_u32(h2_t{sh1, sh1});
+                kb2 = (uint32_t)kb | ((uint32_t)kb << 16);
+            }
+            // dequantises codes 2n, 2n+1 of the word (held in bytes 0 and 2 of `codes`); G32: each of the two takes the
+            // first pair if its index is below kb - a packed 16-bit subtract and arithmetic shift give the halfword
+            // masks, two bit-field inserts the parameters
+            auto deq = [&](uint32_t codes, int n) -> uint32_t {
+                if (!G32) return dequant_pair(codes, nb_a, sc_a);
+                const s2_t d = __builtin_bit_cast(s2_t, (uint32_t)(2 * n) | ((uint32_t)(2 * n + 1) << 16)) -
+                               __builtin_bit_cast(s2_t, kb2);                       // < 0 <=> first pair
+                const uint32_t m = __builtin_bit_cast(uint32_t, (s2_t)(d >> 15));
+                const uint32_t nbx = (m & as_u32(nb_a)) | (~m & nb_b);
+                const uint32_t scx = (m & as_u32(sc_a)) | (~m & sc_b);
+                return dequant_pair(codes, as_h2(nbx), as_h2(scx));
+            };
             if (BIT == 2) {
                 // E[k % 4] holds code k in byte k / 4
                 const uint32_t e0 = w & 0x03030303u, e1 = (w >> 2) & 0x03030303u;
                 const uint32_t e2 = (w >> 4) & 0x03030303u, e3 = (w >> 6) & 0x03030303u;
                 u32x4_t lo, hi;
-                lo[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), neg_bias, scale2);  // codes 0, 1
-                lo[1] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c040c00u), neg_bias, scale2);  // codes 2, 3
-                lo[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), neg_bias, scale2);
-                lo[3] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c050c01u), neg_bias, scale2);
-                hi[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), neg_bias, scale2);
-                hi[1] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c060c02u), neg_bias, scale2);
-                hi[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), neg_bias, scale2);
-                hi[3] = dequant_pair(__builtin_amdgcn_perm(e3, e2, 0x0c070c03u), neg_bias, scale2);
+                lo[0] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), 0);  // codes 0, 1
+                lo[1] = deq(__builtin_amdgcn_perm(e3, e2, 0x0c040c00u), 1);  // codes 2, 3
+                lo[2] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), 2);
+                lo[3] = deq(__builtin_amdgcn_perm(e3, e2, 0x0c050c01u), 3);
+                hi[0] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), 4);
+                hi[1] = deq(__builtin_amdgcn_perm(e3, e2, 0x0c060c02u), 5);
+                hi[2] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), 6);
+                hi[3] = deq(__builtin_amdgcn_perm(e3, e2, 0x0c070c03u), 7);
                 *(MSTF_LDS u32x4_t*)(uintptr_t)dst = lo;
                 *(MSTF_LDS u32x4_t*)(uintptr_t)(dst + 16u) = hi;
             } else if (BIT == 4) {
                 // e0 holds codes 0, 2, 4, 6 in its bytes, e1 codes 1, 3, 5, 7
                 const uint32_t e0 = w & 0x0f0f0f0fu, e1 = (w >> 4) & 0x0f0f0f0fu;
                 u32x4_t v;
-                v[0] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), neg_bias, scale2);
-                v[1] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), neg_bias, scale2);
-                v[2] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), neg_bias, scale2);
-                v[3] = dequant_pair(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), neg_bias, scale2);
+                v[0] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c040c00u), 0);
+                v[1] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c050c01u), 1);
+                v[2] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c060c02u), 2);
+                v[3] = deq(__builtin_amdgcn_perm(e1, e0, 0x0c070c03u), 3);
                 *(MSTF_LDS u32x4_t*)(uintptr_t)dst = v;
             } else {
                 u32x2_t v;
-                v[0] = dequant_pair(__builtin_amdgcn_perm(w, w, 0x0c010c00u), neg_bias, scale2);
-                v[1] = dequant_pair(__builtin_amdgcn_perm(w, w, 0x0c030c02u), neg_bias, scale2);
+                v[0] = deq(__builtin_amdgcn_perm(w, w, 0x0c010c00u), 0);
+                v[1] = deq(__builtin_amdgcn_perm(w, w, 0x0c030c02u), 1);
                 *(MSTF_LDS u32x2_t*)(uintptr_t)dst = v;
             }
         } else {
 #pragma unroll 1
             for (int k = 0; k < F::kCap; k++) {
                 const uint32_t q = (w >> (k * BIT)) & ((1u << BIT) - 1u);
-                *(MSTF_LDS _Float16*)(uintptr_t)(dst + 2u * (uint32_t)k) = dequant_exact(q, sc, zp, mode);
+                const uint32_t sel = (G32 && k >= kb) ? 16u : 0u;
+                *(MSTF_LDS _Float16*)(uintptr_t)(dst + 2u * (uint32_t)k) =
+                    dequant_exact(q, (sc >> sel) & 0xffffu, (zp >> sel) & 0xffffu, mode);
             }
         }
     }
@@ -155,6 +197,42 @@ __device__ __forceinline__ MetaLane meta_lane(const uint32_t* off_dma, const uin
                      : lane < 48 ? reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(scales) + (lane - 32))
                                  : reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(zeros) + (lane - 48));
     m.shift = lane < 32 ? 2u : 1u;
+    return m;
+}
+// Two pairs per tile: two loads.  First: lanes 0..31 the word offsets, 32..63 the scales (4 bytes per tile).  Second:
+// lanes 0..31 the zero-points (4 bytes per tile), 32..63 the upper halves of the bitmaps (elements 0 .. 31 of a tile
+// are bits 63 .. 32, i.e. the second 4 bytes of the little-endian 8).
+struct MetaLanes {
+    MetaLane a, b;
+};
+__device__ __forceinline__ MetaLanes meta_lanes_g32(const uint32_t* off_dma, const uint16_t* scales, const uint16_t* zeros,
+                                                    const uint64_t* bmp, int lane)
+{
+    MetaLanes m;
+    const int l = lane & 31;
+    m.a.p0 = lane < 32 ? reinterpret_cast<const char*>(off_dma + l)
+                       : reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(scales) + l);
+    m.a.shift = 2u;
+    m.b.p0 = lane < 32 ? reinterpret_cast<const char*>(reinterpret_cast<const uint32_t*>(zeros) + l)
+                       : reinterpret_cast<const char*>(bmp + l) + 4;
+    m.b.shift = lane < 32 ? 2u : 3u;
+    return m;
+}
+// Issues the metadata of the stage starting at tile t (relative to the pointers the lanes were built from).
+template <bool G32>
+__device__ __forceinline__ void meta_issue(const MetaLanes& m, uint32_t t, char* metabuf)
+{
+    dma4(m.a.at(t), metabuf);
+    if (G32) dma4(m.b.at(t), metabuf + 256);
+}
+template <bool G32>
+__device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const uint16_t* scales, const uint16_t* zeros,
+                                                const uint64_t* bmp, int lane)
+{
+    if (G32) return meta_lanes_g32(off_dma, scales, zeros, bmp, lane);
+    MetaLanes m;
+    m.a = meta_lane(off_dma, scales, zeros, lane);
+    m.b = m.a;
     return m;
 }
 

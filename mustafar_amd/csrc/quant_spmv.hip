@@ -35,7 +35,7 @@ struct QCache {
 
 // Walks `nsubs` stages of 32 tiles with a two-deep pipeline (see walk_subs).  Tile indices are global
 // (KV head included): tile_off / scales / zeros / bmp are flat over [Bkv, T].
-template <int NM, int BIT, class TileOf, class StageW, class WAddrOf>
+template <int NM, int BIT, bool G32, class TileOf, class StageW, class WAddrOf>
 __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW stage_w, WAddrOf waddr_of, uint32_t wgroup,
                                             const QCache& c, char* my, int lane, int mode, f4_t (&acc)[NM])
 {
@@ -53,7 +53,8 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
         const uint32_t cnt = (uint32_t)__builtin_popcountll(c.bmp[t + kSubTiles - 1]);
         e = c.off[t + kSubTiles - 1] + ((cnt + (uint32_t)F::kCap - 1u) >> F::kCapShift);
     };
-    const MetaLane meta = meta_lane(c.off_dma, c.scales, c.zeros, lane);
+    constexpr int kMetaBytes = meta_bytes<G32>();
+    const MetaLanes meta = meta_lanes<G32>(c.off_dma, c.scales, c.zeros, c.bmp, lane);
     const uint32_t lane4 = (uint32_t)lane * 4u;
     const uint32_t touch8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
     const uint32_t wordbuf_lds = lds_addr(wordbuf);
@@ -64,8 +65,9 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
         nw = nw > (uint32_t)F::kWordsMax ? (uint32_t)F::kWordsMax : nw;  // never true for a well-formed cache
         words_issue_flat<F::kWordsMax / 64>(c.packed + uni(s), nw, wordbuf_lds + (uint32_t)(n & 1) * F::kWordBuf,
                                             (uint32_t)lane, lane4);
-        // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane)
-        dma4(meta.at((uint32_t)t), metabuf + (n & 1) * kMetaBytes);
+        // metadata: lanes 0..31 the word offsets, 32..47 the scales, 48..63 the zero-points (two per lane); two loads
+        // when a tile has two (scale, zero) pairs
+        meta_issue<G32>(meta, (uint32_t)t, metabuf + (n & 1) * kMetaBytes);
         stage_w(n);
         // pulls the stage's bitmaps into L2 ahead of the scalar loads of the expansion
         return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(c.bmp + t) + touch8);
@@ -89,7 +91,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
             t_nxt = tile_of(n + 2);
             bounds(t_nxt, s_nxt, e_nxt);
         }
-        dequant_stage<BIT>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
+        dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
                            lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, lane, mode);
         const uint64_t* bm = c.bmp + t_now;
         const uint32_t waddr = waddr_of(n);
@@ -100,7 +102,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
 
 // ------------------------------------------------------------------------------- key
 // One wavefront per (KV head, token block); see key_spmv_kernel.
-template <int NW, int BIT>
+template <int NW, int BIT, bool G32>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void key_spmv_quant_kernel(
     const uint64_t* __restrict__ bmp, const uint32_t* packed, const uint32_t* __restrict__ tile_off,
     const uint32_t* tile_off_dma, const uint16_t* scales, const uint16_t* zeros, const _Float16* Bm,
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
 {
     constexpr int NM = (NW + 3) / 4;
     constexpr int kMaxD = 128;
-    constexpr int kQ = q_lds_bytes<BIT>();
+    constexpr int kQ = q_lds_bytes<BIT, G32>();
     constexpr int kWaveLds = kQ + NM * 4 * kMaxD * 2;
     __shared__ __attribute__((aligned(16))) char lds[4][kWaveLds];
     const int lane = lane_id();
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
     for (int m = 0; m < NM; m++) acc[m] = f4_t{0.f, 0.f, 0.f, 0.f};
     const size_t tile0 = (size_t)kv * T + (size_t)tb * D;
     const uint32_t wrow = lds_addr(wl) + (uint32_t)(lane & 3) * (uint32_t)D * 2u;
-    walk_subs_q<NM, BIT>(
+    walk_subs_q<NM, BIT, G32>(
         D / kSubTiles, [=](int n) { return tile0 + (size_t)n * kSubTiles; },
         [=](int n) {
             if (n != 0) return;  // the query rows are staged once per task
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
 
 // ------------------------------------------------------------------------------- value
 // grid = (token splits, D/64 halves, KV heads); see value_spmv_kernel.
-template <int NW, int WAVES, int BIT>
+template <int NW, int WAVES, int BIT, bool G32>
 __global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
     const uint64_t* __restrict__ bmp, const uint32_t* packed, const uint32_t* __restrict__ tile_off,
     const uint32_t* tile_off_dma, const uint16_t* scales, const uint16_t* zeros, const _Float16* P,
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
     constexpr int NM = (NW + 3) / 4;
     constexpr int kWRow = kSubTiles * 2;
     constexpr int kWBuf = NM * 4 * kWRow;
-    constexpr int kQ = q_lds_bytes<BIT>();
+    constexpr int kQ = q_lds_bytes<BIT, G32>();
     constexpr int kNeed = kQ + 2 * kWBuf;
     constexpr int kWaveLds = kNeed > NW * 256 ? kNeed : NW * 256;  // the per-wave sums are parked here at the end
     __shared__ __attribute__((aligned(16))) char lds[WAVES][kWaveLds];
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
     constexpr int subs_per_blk = 64 / kSubTiles;
     const uint32_t wrow = lds_addr(wl) + (uint32_t)(lane & 3) * kWRow;
     const size_t thead = (size_t)kv * T + (size_t)half * 64;
-    walk_subs_q<NM, BIT>(
+    walk_subs_q<NM, BIT, G32>(
         (last - first) * subs_per_blk,
         [=](int n) { return thead + (size_t)(first + n / subs_per_blk) * D + (size_t)(n % subs_per_blk) * kSubTiles; },
         [=](int n) {
@@ -252,6 +254,7 @@ struct QArgs {
     const uint16_t* scales;
     const uint16_t* zeros;
     int mode;
+    int group_size;  // 64: one (scale, zero) pair per tile; 32: two
 };
 
 template <int NW, int BIT>
@@ -260,8 +263,12 @@ static void launch_key_q(hipStream_t st, const QArgs& a, const _Float16* Bm, _Fl
 {
     const int nblk = Lc / 64;
     const int ntasks = Bkv * nblk;
-    hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT>), dim3((ntasks + 3) / 4), dim3(256), 0, st, a.bmp, a.packed,
-                       a.tile_off, a.tile_off, a.scales, a.zeros, Bm, C, Lc, D, nblk, ntasks, rows_per_kv, row0, a.mode);
+    if (a.group_size == 32)
+        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, true>), dim3((ntasks + 3) / 4), dim3(256), 0, st, a.bmp, a.packed,
+                           a.tile_off, a.tile_off, a.scales, a.zeros, Bm, C, Lc, D, nblk, ntasks, rows_per_kv, row0, a.mode);
+    else
+        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, false>), dim3((ntasks + 3) / 4), dim3(256), 0, st, a.bmp, a.packed,
+                           a.tile_off, a.tile_off, a.scales, a.zeros, Bm, C, Lc, D, nblk, ntasks, rows_per_kv, row0, a.mode);
 }
 template <int NW>
 static void launch_key_q_bit(int bit, hipStream_t st, const QArgs& a, const _Float16* Bm, _Float16* C, int Lc, int D,
@@ -279,9 +286,14 @@ template <int NW, int WAVES, int BIT>
 static void launch_value_q(hipStream_t st, const ValuePlan& pl, const QArgs& a, const _Float16* P, _Float16* C,
                            float* part, int Lc, int D, int Bkv, int rows_per_kv, int row0)
 {
-    hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT>), dim3(pl.nsplit, D / 64, Bkv), dim3(WAVES * 64), 0, st,
-                       a.bmp, a.packed, a.tile_off, a.tile_off, a.scales, a.zeros, P, C, part, Lc, D, Lc / 64, pl.nbpw,
-                       pl.nsplit, rows_per_kv, row0, a.mode);
+    if (a.group_size == 32)
+        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, true>), dim3(pl.nsplit, D / 64, Bkv), dim3(WAVES * 64), 0,
+                           st, a.bmp, a.packed, a.tile_off, a.tile_off, a.scales, a.zeros, P, C, part, Lc, D, Lc / 64,
+                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode);
+    else
+        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, false>), dim3(pl.nsplit, D / 64, Bkv), dim3(WAVES * 64), 0,
+                           st, a.bmp, a.packed, a.tile_off, a.tile_off, a.scales, a.zeros, P, C, part, Lc, D, Lc / 64,
+                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode);
 }
 template <int NW, int WAVES>
 static void launch_value_q_bit(int bit, hipStream_t st, const ValuePlan& pl, const QArgs& a, const _Float16* P,
@@ -299,13 +311,12 @@ static void launch_value_q_bit(int bit, hipStream_t st, const ValuePlan& pl, con
 
 using namespace mstf;
 
-extern "C" int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
-                                   const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
-                                   const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq,
-                                   int groups, int n_rows, int bit, int capacity, int dequant_mode)
+static int key_spmv_quant_impl(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                               const mstf_half* scales, const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M,
+                               int K, int Bq, int groups, int n_rows, int bit, int capacity, int dequant_mode,
+                               int group_size)
 {
-    (void)counts;  // raw counts and units follow from the bitmaps; accepted for interface compatibility
-    (void)units;
+    if (group_size != 64 && group_size != 32) return MSTF_EUNSUPPORTED;
     int rc = check_quant_spmv(bmp, packed, tile_off, scales, zeros, Bm, C, M, K, Bq, groups, n_rows, bit, capacity,
                               dequant_mode);
     if (rc != MSTF_OK) return rc;
@@ -313,7 +324,7 @@ extern "C" int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint
     const int Bkv = Bq / groups, rows_per_kv = groups * n_rows;
     const _Float16* b = reinterpret_cast<const _Float16*>(Bm);
     _Float16* c = reinterpret_cast<_Float16*>(C);
-    const QArgs a = {bmp, packed, tile_off, scales, zeros, dequant_mode};
+    const QArgs a = {bmp, packed, tile_off, scales, zeros, dequant_mode, group_size};
     for (int row0 = 0; row0 < rows_per_kv;) {
         const int nw = pick_nw(rows_per_kv - row0);
         switch (nw) {
@@ -330,6 +341,26 @@ extern "C" int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint
     return MSTF_OK;
 }
 
+extern "C" int mstf_key_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                                   const uint32_t* counts, const uint32_t* units, const mstf_half* scales,
+                                   const mstf_half* zeros, const mstf_half* Bm, mstf_half* C, int M, int K, int Bq,
+                                   int groups, int n_rows, int bit, int capacity, int dequant_mode)
+{
+    (void)counts;  // raw counts and units follow from the bitmaps; accepted for interface compatibility
+    (void)units;
+    return key_spmv_quant_impl(stream, bmp, packed, tile_off, scales, zeros, Bm, C, M, K, Bq, groups, n_rows, bit, capacity,
+                               dequant_mode, 64);
+}
+
+extern "C" int mstf_key_spmv_quant_grouped(void* stream, const uint64_t* bmp, const uint32_t* packed,
+                                           const uint32_t* tile_off, const mstf_half* scales, const mstf_half* zeros,
+                                           const mstf_half* Bm, mstf_half* C, int M, int K, int Bq, int groups, int n_rows,
+                                           int bit, int capacity, int dequant_mode, int group_size)
+{
+    return key_spmv_quant_impl(stream, bmp, packed, tile_off, scales, zeros, Bm, C, M, K, Bq, groups, n_rows, bit, capacity,
+                               dequant_mode, group_size);
+}
+
 extern "C" size_t mstf_value_spmv_quant_workspace_bytes(int M, int K, int Bq, int groups, int n_rows)
 {
     if (M <= 0 || K <= 0 || Bq <= 0 || groups <= 0 || n_rows <= 0 || K % 64 != 0 || M % 64 != 0 || Bq % groups != 0)
@@ -337,14 +368,12 @@ extern "C" size_t mstf_value_spmv_quant_workspace_bytes(int M, int K, int Bq, in
     return value_workspace_bytes(M, K, Bq, groups, n_rows);
 }
 
-extern "C" int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed,
-                                     const uint32_t* tile_off, const uint32_t* counts, const uint32_t* units,
-                                     const mstf_half* scales, const mstf_half* zeros, const mstf_half* P, mstf_half* C,
-                                     int M, int K, int Bq, int groups, int n_rows, int bit, int capacity,
-                                     int dequant_mode, void* workspace, size_t workspace_bytes)
+static int value_spmv_quant_impl(void* stream, const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off,
+                                 const mstf_half* scales, const mstf_half* zeros, const mstf_half* P, mstf_half* C, int M,
+                                 int K, int Bq, int groups, int n_rows, int bit, int capacity, int dequant_mode,
+                                 int group_size, void* workspace, size_t workspace_bytes)
 {
-    (void)counts;
-    (void)units;
+    if (group_size != 64 && group_size != 32) return MSTF_EUNSUPPORTED;
     // M = head_dim, K = compressed tokens (the operator's GEMM naming)
     int rc = check_quant_spmv(bmp, packed, tile_off, scales, zeros, P, C, K, M, Bq, groups, n_rows, bit, capacity,
                               dequant_mode);
@@ -357,7 +386,7 @@ extern "C" int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const ui
     const _Float16* p = reinterpret_cast<const _Float16*>(P);
     _Float16* c = reinterpret_cast<_Float16*>(C);
     float* part = reinterpret_cast<float*>(workspace);
-    const QArgs a = {bmp, packed, tile_off, scales, zeros, dequant_mode};
+    const QArgs a = {bmp, packed, tile_off, scales, zeros, dequant_mode, group_size};
     for (int row0 = 0; row0 < rows_per_kv;) {
         const int nw = pick_nw(rows_per_kv - row0);
         const ValuePlan pl = plan_value(K, M, Bkv, nw);
@@ -377,4 +406,26 @@ extern "C" int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const ui
         row0 += nw;
     }
     return MSTF_OK;
+}
+
+extern "C" int mstf_value_spmv_quant(void* stream, const uint64_t* bmp, const uint32_t* packed,
+                                     const uint32_t* tile_off, const uint32_t* counts, const uint32_t* units,
+                                     const mstf_half* scales, const mstf_half* zeros, const mstf_half* P, mstf_half* C,
+                                     int M, int K, int Bq, int groups, int n_rows, int bit, int capacity,
+                                     int dequant_mode, void* workspace, size_t workspace_bytes)
+{
+    (void)counts;
+    (void)units;
+    return value_spmv_quant_impl(stream, bmp, packed, tile_off, scales, zeros, P, C, M, K, Bq, groups, n_rows, bit, capacity,
+                                 dequant_mode, 64, workspace, workspace_bytes);
+}
+
+extern "C" int mstf_value_spmv_quant_grouped(void* stream, const uint64_t* bmp, const uint32_t* packed,
+                                             const uint32_t* tile_off, const mstf_half* scales, const mstf_half* zeros,
+                                             const mstf_half* P, mstf_half* C, int M, int K, int Bq, int groups, int n_rows,
+                                             int bit, int capacity, int dequant_mode, int group_size, void* workspace,
+                                             size_t workspace_bytes)
+{
+    return value_spmv_quant_impl(stream, bmp, packed, tile_off, scales, zeros, P, C, M, K, Bq, groups, n_rows, bit, capacity,
+                                 dequant_mode, group_size, workspace, workspace_bytes);
 }

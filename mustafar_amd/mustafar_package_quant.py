@@ -6,11 +6,25 @@ Differences that do not change results: `split_k` and `value_tile_config` only s
 reference splits its launch (its tile64 / fused configurations address the wrong tiles); here the
 split is chosen by the library and both arguments are accepted and ignored.  `tile_counts` /
 `tile_units` are validated but not read: they follow from the bitmaps.
+
+An addition of this build: when `scales` / `zeros` are [B, T, 2] (as `convert_*_batched_quant(group_size=32)` return
+them) every operator here reads two (scale, zero) pairs per tile, pair g for the elements 32g .. 32g+31.
 """
 import torch
 
 from . import ops
 from ._lib import check, lib
+
+
+def _group_size(bmp, scales, zeros):
+    """64 for [B, T] scales (the reference), 32 for [B, T, 2]."""
+    if scales.shape != zeros.shape:
+        raise RuntimeError("scales and zeros must have the same shape.")
+    if scales.numel() == bmp.numel():
+        return 64
+    if scales.numel() == 2 * bmp.numel() and scales.shape[-1] == 2:
+        return 32
+    raise RuntimeError("scales must hold one or two entries per tile.")
 
 
 def _common_checks(B, tensors, int_names, half_names):
@@ -49,13 +63,11 @@ def _key(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, B,
     if B.numel() != Batch_Size * 8 * K_Global:
         raise RuntimeError("Tensor B must hold Batch_Size x 8 x K_Global elements.")
     C = torch.empty((Batch_Size, 8, M_Global), dtype=torch.float16, device=B.device)
-    check(lib().mstf_key_spmv_quant(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
-                                    tile_offsets.data_ptr(),
-                                    tile_counts.data_ptr() if tile_counts is not None else None,
-                                    tile_units.data_ptr() if tile_units is not None else None, scales.data_ptr(),
-                                    zeros.data_ptr(), B.data_ptr(), C.data_ptr(), int(M_Global), int(K_Global),
-                                    int(Batch_Size), int(num_key_value_groups), 8, int(bit), int(capacity),
-                                    int(dequant_mode)), "mustafar_key_formulation_quant")
+    check(lib().mstf_key_spmv_quant_grouped(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
+                                            tile_offsets.data_ptr(), scales.data_ptr(), zeros.data_ptr(), B.data_ptr(),
+                                            C.data_ptr(), int(M_Global), int(K_Global), int(Batch_Size),
+                                            int(num_key_value_groups), 8, int(bit), int(capacity), int(dequant_mode),
+                                            _group_size(bmp, scales, zeros)), "mustafar_key_formulation_quant")
     return C
 
 
@@ -85,11 +97,11 @@ def _value(bmp, NZ_quant, tile_offsets, tile_counts, tile_units, scales, zeros, 
     wsb = L.mstf_value_spmv_quant_workspace_bytes(int(M_Global), int(K_Global), int(Batch_Size),
                                                   int(num_key_value_groups), n_rows)
     ws = ops.workspace(P.device, wsb)
-    check(L.mstf_value_spmv_quant(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
-                                  tile_offsets.data_ptr(), tile_counts.data_ptr(), tile_units.data_ptr(),
-                                  scales.data_ptr(), zeros.data_ptr(), P.data_ptr(), C.data_ptr(), int(M_Global),
-                                  int(K_Global), int(Batch_Size), int(num_key_value_groups), n_rows, int(bit),
-                                  int(capacity), int(dequant_mode), ws.data_ptr(), ws.numel()), what)
+    check(L.mstf_value_spmv_quant_grouped(torch.cuda.current_stream().cuda_stream, bmp.data_ptr(), NZ_quant.data_ptr(),
+                                          tile_offsets.data_ptr(), scales.data_ptr(), zeros.data_ptr(), P.data_ptr(),
+                                          C.data_ptr(), int(M_Global), int(K_Global), int(Batch_Size),
+                                          int(num_key_value_groups), n_rows, int(bit), int(capacity), int(dequant_mode),
+                                          _group_size(bmp, scales, zeros), ws.data_ptr(), ws.numel()), what)
     return C
 
 
@@ -126,12 +138,15 @@ def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, d
     L = lib()
     o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
     ws = ops.workspace(q.device, L.mstf_decode_attention_workspace_bytes(tokens, D, Bq, num_key_value_groups))
-    check(L.mstf_decode_attention_quant(torch.cuda.current_stream().cuda_stream, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(),
-                                        ks.data_ptr(), kz.data_ptr(), vb.data_ptr(), vp.data_ptr(), vo.data_ptr(),
-                                        vs.data_ptr(), vz.data_ptr(), q.contiguous().data_ptr(), o.data_ptr(),
-                                        lse.data_ptr() if lse is not None else None, tokens, D, Bq,
-                                        int(num_key_value_groups), int(bit), 32 // int(bit), int(dequant_mode),
-                                        ws.data_ptr(), ws.numel()), "mstf_decode_attention_quant")
+    group_size = _group_size(kb, ks, kz)
+    if _group_size(vb, vs, vz) != group_size:
+        raise RuntimeError("key side and value side must use the same group size.")
+    check(L.mstf_decode_attention_quant_grouped(torch.cuda.current_stream().cuda_stream, kb.data_ptr(), kp.data_ptr(),
+                                                ko.data_ptr(), ks.data_ptr(), kz.data_ptr(), vb.data_ptr(), vp.data_ptr(),
+                                                vo.data_ptr(), vs.data_ptr(), vz.data_ptr(), q.contiguous().data_ptr(),
+                                                o.data_ptr(), lse.data_ptr() if lse is not None else None, tokens, D, Bq,
+                                                int(num_key_value_groups), int(bit), 32 // int(bit), int(dequant_mode),
+                                                group_size, ws.data_ptr(), ws.numel()), "mstf_decode_attention_quant")
     return o
 
 
@@ -151,6 +166,8 @@ def decode_attention_window_quant(key_side, value_side, q, k_win, v_win, win_len
         kb, ko, kp, ks, kz = five(key_side)
         vb, vo, vp, vs, vz = five(value_side)
         tokens = kb.shape[1] * 64 // D
+        if _group_size(kb, ks, kz) != 64 or _group_size(vb, vs, vz) != 64:
+            raise RuntimeError("the window entry point reads one scale / zero pair per tile (group_size 64).")
         ptrs = [kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), ks.data_ptr(), kz.data_ptr(), vb.data_ptr(), vp.data_ptr(),
                 vo.data_ptr(), vs.data_ptr(), vz.data_ptr()]
     else:

@@ -367,11 +367,16 @@ void orc_dense_masked_attention(const h16* q, const h16* Kp, const h16* Vp, int 
  * :41-57 is fp32 arithmetic in Triton.  Pinned bit for bit (bit = 2) by arrays the reference's own programs wrote
  * under Triton's interpreter (tests/golden/ref_quant.npz).  bit = 4 / 8 are extensions of this build (the reference
  * producer hard-codes 2): same formulas with 2^bit - 1 steps, pinned by closed form and error bound only.
- * packed may be NULL to size it. returns total uint32 words. */
-uint64_t orc_compress_quant(const h16* x, int B, int M, int N, int is_value, int bit, uint64_t* bmp, uint32_t* counts,
-                            uint32_t* units, uint32_t* tile_off, uint32_t* packed, uint64_t packed_cap, h16* scales,
-                            h16* zeros)
+ * packed may be NULL to size it. returns total uint32 words.
+ * group_size 32 (an option of this build, after the harness setting GROUP_SIZE = 32 of
+ * benchmark/mem_spd_test_quant.py:33,104, which the reference's producer never reads): scales / zeros are [B,T,2],
+ * pair g for the elements 32g .. 32g+31 of the tile, each pair from the minimum and maximum of its own kept elements
+ * by the same formulas; codes stay packed in rank order over the whole tile. */
+uint64_t orc_compress_quant_grouped(const h16* x, int B, int M, int N, int is_value, int bit, int group_size,
+                                    uint64_t* bmp, uint32_t* counts, uint32_t* units, uint32_t* tile_off,
+                                    uint32_t* packed, uint64_t packed_cap, h16* scales, h16* zeros)
 {
+    const int ngrp = 64 / group_size; /* 1 (the reference: one pair per 64-element tile) or 2 (group 32) */
     long T = (long)M * N / 64;
     int cap = 32 / bit;
     float maxq = (float)((1 << bit) - 1);
@@ -381,39 +386,48 @@ uint64_t orc_compress_quant(const h16* x, int B, int M, int N, int is_value, int
         for (long t = 0; t < T; t++) {
             uint64_t bits = 0;
             int cnt = 0;
-            float mn = INFINITY, mx = -INFINITY;
+            float mn[2] = {INFINITY, INFINITY}, mx[2] = {-INFINITY, -INFINITY};
+            int gcnt[2] = {0, 0};
             h16 vals[64];
+            int grp[64];
             for (int i = 0; i < 64; i++) {
                 h16 v = xb[is_value ? value_elem(M, N, t, i) : key_elem(M, N, t, i)];
                 if (nonzero_h(v)) {
+                    const int g = i / group_size; /* the group is a matter of the element's position in the tile */
                     bits |= 1ull << (63 - i);
                     float f = h2f(v);
-                    if (f < mn) mn = f;
-                    if (f > mx) mx = f;
+                    if (f < mn[g]) mn[g] = f;
+                    if (f > mx[g]) mx[g] = f;
+                    gcnt[g]++;
+                    grp[cnt] = g;
                     vals[cnt++] = v;
                 }
             }
-            float scale = 1.f, zero = 0.f;
-            if (cnt > 0) {
-                scale = (mx - mn) / maxq;
-                if (scale == 0.f) scale = 1.f;
-                zero = floorf(-mn / scale + 0.5f);
-            }
-            h16 sh = f2h(scale), zh = f2h(zero);
             long ti = (long)b * T + t;
+            h16 sh[2], zh[2];
+            for (int g = 0; g < ngrp; g++) {
+                float scale = 1.f, zero = 0.f;
+                if (gcnt[g] > 0) {
+                    scale = (mx[g] - mn[g]) / maxq;
+                    if (scale == 0.f) scale = 1.f;
+                    zero = floorf(-mn[g] / scale + 0.5f);
+                }
+                sh[g] = f2h(scale);
+                zh[g] = f2h(zero);
+                scales[ti * ngrp + g] = sh[g];
+                zeros[ti * ngrp + g] = zh[g];
+            }
             bmp[ti] = bits;
             counts[ti] = (uint32_t)cnt;
             uint32_t u = (uint32_t)((cnt + cap - 1) / cap);
             units[ti] = u;
             tile_off[ti] = (uint32_t)off;
-            scales[ti] = sh;
-            zeros[ti] = zh;
             if (packed) {
-                float sc = h2f(sh), zp = h2f(zh);
-                if (sc == 0.f) sc = 1.f; /* :137-138 */
                 for (uint32_t w = 0; w < u; w++)
                     if (off + w < packed_cap) packed[off + w] = 0;
                 for (int j = 0; j < cnt; j++) {
+                    float sc = h2f(sh[grp[j]]), zp = h2f(zh[grp[j]]);
+                    if (sc == 0.f) sc = 1.f; /* :137-138 */
                     float qf = floorf(h2f(vals[j]) / sc + 0.5f) + zp;
                     if (qf < 0.f) qf = 0.f;
                     if (qf > maxq) qf = maxq;
@@ -427,13 +441,23 @@ uint64_t orc_compress_quant(const h16* x, int B, int M, int N, int is_value, int
     return off;
 }
 
+uint64_t orc_compress_quant(const h16* x, int B, int M, int N, int is_value, int bit, uint64_t* bmp, uint32_t* counts,
+                            uint32_t* units, uint32_t* tile_off, uint32_t* packed, uint64_t packed_cap, h16* scales,
+                            h16* zeros)
+{
+    return orc_compress_quant_grouped(x, B, M, N, is_value, bit, 64, bmp, counts, units, tile_off, packed, packed_cap,
+                                      scales, zeros);
+}
+
 /* Consumer-side dequantised dense rebuild of batch entry b:
  * kernel_quant/csrc/SpMM_Kernel_Quant.cuh:204-242: j-th set bit (MSB first) takes code j;
  * dequant_mode 0: fp32 (q - zero) * scale then round to fp16 (:238-240);
  * dequant_mode 1: fp16 arithmetic hsub then hmul (:190-191). */
-void orc_decode_quant(const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off, const h16* scales,
-                      const h16* zeros, int b, int M, int N, int is_value, int bit, int dequant_mode, h16* dense)
+void orc_decode_quant_grouped(const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off, const h16* scales,
+                              const h16* zeros, int b, int M, int N, int is_value, int bit, int dequant_mode,
+                              int group_size, h16* dense)
 {
+    const int ngrp = 64 / group_size;
     long T = (long)M * N / 64;
     int cap = 32 / bit;
     uint32_t mask = (1u << bit) - 1u;
@@ -442,11 +466,12 @@ void orc_decode_quant(const uint64_t* bmp, const uint32_t* packed, const uint32_
         long ti = (long)b * T + t;
         uint64_t bits = bmp[ti];
         const uint32_t* w = packed + tile_off[ti];
-        float sc = h2f(scales[ti]), zp = h2f(zeros[ti]);
         int j = 0;
         while (bits) {
             int pos = __builtin_clzll(bits);
             bits &= ~(0x8000000000000000ull >> pos);
+            /* the element's position picks its (scale, zero) pair; codes stay in rank order over the whole tile */
+            float sc = h2f(scales[ti * ngrp + pos / group_size]), zp = h2f(zeros[ti * ngrp + pos / group_size]);
             uint32_t qv = (w[j / cap] >> ((j % cap) * bit)) & mask;
             h16 v;
             if (dequant_mode == 1)
@@ -457,6 +482,12 @@ void orc_decode_quant(const uint64_t* bmp, const uint32_t* packed, const uint32_
             j++;
         }
     }
+}
+
+void orc_decode_quant(const uint64_t* bmp, const uint32_t* packed, const uint32_t* tile_off, const h16* scales,
+                      const h16* zeros, int b, int M, int N, int is_value, int bit, int dequant_mode, h16* dense)
+{
+    orc_decode_quant_grouped(bmp, packed, tile_off, scales, zeros, b, M, N, is_value, bit, dequant_mode, 64, dense);
 }
 
 /* Q2/Q3 semantics: the K1/V1 products on the dequantised matrix. */

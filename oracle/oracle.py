@@ -34,6 +34,7 @@ def lib():
         _lib = ctypes.CDLL(_SO)
         _lib.orc_compress.restype = ctypes.c_uint64
         _lib.orc_compress_quant.restype = ctypes.c_uint64
+        _lib.orc_compress_quant_grouped.restype = ctypes.c_uint64
         _lib.orc_num_threads.restype = ctypes.c_int
     return _lib
 
@@ -154,36 +155,41 @@ def dense_masked_attention(q, Kp, Vp, groups):
 
 
 # ----------------------------------------------------------- quant format
-def compress_quant(x, is_value, bit=2):
+def compress_quant(x, is_value, bit=2, group_size=64):
     """convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529).
 
     Returns (bmp int64 [B,T], tile_off int32 [B,T], packed int32 flat, counts int32, units int32,
-    scales fp16, zeros fp16)."""
+    scales fp16, zeros fp16); scales / zeros are [B,T] for group_size 64 (the reference) and [B,T,2] for 32."""
     x = _c(x, np.float16)
     B, M, N = x.shape
     T = M * N // 64
+    assert group_size in (32, 64)
     bmp = np.empty((B, T), np.uint64)
     counts = np.empty((B, T), np.uint32)
     units = np.empty((B, T), np.uint32)
     toff = np.empty((B, T), np.uint32)
-    scales = np.empty((B, T), np.float16)
-    zeros = np.empty((B, T), np.float16)
-    a = (ctypes.c_int(B), ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(int(is_value)), ctypes.c_int(bit))
-    total = lib().orc_compress_quant(_p(x), *a, _p(bmp), _p(counts), _p(units), _p(toff), None, ctypes.c_uint64(0),
-                                     _p(scales), _p(zeros))
+    shape = (B, T) if group_size == 64 else (B, T, 2)
+    scales = np.empty(shape, np.float16)
+    zeros = np.empty(shape, np.float16)
+    a = (ctypes.c_int(B), ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(int(is_value)), ctypes.c_int(bit),
+         ctypes.c_int(group_size))
+    fn = lib().orc_compress_quant_grouped
+    total = fn(_p(x), *a, _p(bmp), _p(counts), _p(units), _p(toff), None, ctypes.c_uint64(0), _p(scales), _p(zeros))
     packed = np.zeros((int(total),), np.uint32)
-    lib().orc_compress_quant(_p(x), *a, _p(bmp), _p(counts), _p(units), _p(toff), _p(packed),
-                             ctypes.c_uint64(int(total)), _p(scales), _p(zeros))
+    fn(_p(x), *a, _p(bmp), _p(counts), _p(units), _p(toff), _p(packed), ctypes.c_uint64(int(total)), _p(scales),
+       _p(zeros))
     return (bmp.view(np.int64), toff.view(np.int32), packed.view(np.int32), counts.view(np.int32),
             units.view(np.int32), scales, zeros)
 
 
 def decode_quant(bmp, packed, tile_off, scales, zeros, b, M, N, is_value, bit=2, dequant_mode=0):
+    """Dense dequantised [M, N] of batch entry b; the group size follows from the shape of scales ([B,T] or [B,T,2])."""
     dense = np.empty((M, N), np.float16)
-    lib().orc_decode_quant(_p(_c(bmp, np.int64)), _p(_c(packed, np.int32)), _p(_c(tile_off, np.int32)),
-                           _p(_c(scales, np.float16)), _p(_c(zeros, np.float16)), ctypes.c_int(b), ctypes.c_int(M),
-                           ctypes.c_int(N), ctypes.c_int(int(is_value)), ctypes.c_int(bit), ctypes.c_int(dequant_mode),
-                           _p(dense))
+    group_size = 32 if np.ndim(scales) == 3 and np.shape(scales)[2] == 2 else 64
+    lib().orc_decode_quant_grouped(_p(_c(bmp, np.int64)), _p(_c(packed, np.int32)), _p(_c(tile_off, np.int32)),
+                                   _p(_c(scales, np.float16)), _p(_c(zeros, np.float16)), ctypes.c_int(b),
+                                   ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(int(is_value)), ctypes.c_int(bit),
+                                   ctypes.c_int(dequant_mode), ctypes.c_int(group_size), _p(dense))
     return dense
 
 

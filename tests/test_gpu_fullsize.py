@@ -4,7 +4,8 @@ which shares no code with the kernels under test.
 
   configs[1]  batch 8 x 8 KV heads (64 heads), 4096 tokens, 70 % and 50 %: formats, three-launch and fused attention
   configs[2]  batch 16 x 8 KV heads (128 heads), 4096 tokens, 50 / 70 / 90 %: formats of both compressors
-  configs[3]  batch 32 x 8 KV heads (256 heads), 4096 tokens, 70 %, 2- and 4-bit codes: producer arrays against the
+  configs[3]  batch 32 x 8 KV heads (256 heads), 4096 tokens, 70 %, 2- and 4-bit codes, one scale / zero pair per
+              64-element tile (the reference) and per group of 32: producer arrays against the
               closed form, three-launch and fused quantised attention against dense attention on the dequantised cache
 
   * format invariants of the compressed cache (padding rule, offsets, popcounts) and checksums of its content
@@ -184,16 +185,18 @@ def test_decode_attention_full_size(BKV, kth):
 
 
 # ------------------------------------------------------------------ configs[3]: quantised cache, 256 heads x 4096 tokens
-def torch_quantise(xp, is_value, bit):
+def torch_quantise(xp, is_value, bit, group_size=64):
     """The producer's closed form (kernel_quant/compression_quant.py:41-57, 143-145) and the consumer's dequantisation
-    (kernel_quant/csrc/SpMM_Kernel_Quant.cuh:238-240) with torch operators on [B, L, D] pruned values: per 64-element
-    tile fp32 scale / zero-point rounded to fp16, codes, and the dequantised dense tensor (mode 0)."""
+    (kernel_quant/csrc/SpMM_Kernel_Quant.cuh:238-240) with torch operators on [B, L, D] pruned values: per group of
+    group_size consecutive elements of a 64-element tile fp32 scale / zero-point rounded to fp16, codes, and the
+    dequantised dense tensor (mode 0).  Returns scales, zeros ([B, T] or [B, T, 2]) and the dense tensor."""
     B, length, _ = xp.shape
     if is_value:
         tiles = xp.view(B, length // 64, 64, 2, 64).permute(0, 1, 3, 2, 4)      # [b, blk, half, tok, ch]
     else:
         tiles = xp.view(B, length // 64, 64, D).permute(0, 1, 3, 2)             # [b, blk, ch, tok]
-    tiles = tiles.reshape(B, -1, 64).float()
+    ngrp = 64 // group_size
+    tiles = tiles.reshape(B, -1, ngrp, group_size).float()
     nz = tiles != 0
     maxq = float((1 << bit) - 1)
     inf = torch.tensor(float("inf"), device=xp.device)
@@ -211,23 +214,26 @@ def torch_quantise(xp, is_value, bit):
         dense = deq.view(B, length // 64, 2, 64, 64).permute(0, 1, 3, 2, 4).reshape(B, length, D)
     else:
         dense = deq.view(B, length // 64, D, 64).permute(0, 1, 3, 2).reshape(B, length, D)
+    if ngrp == 1:
+        s16, z16 = s16[..., 0], z16[..., 0]
     return s16, z16, dense.contiguous()
 
 
-@pytest.mark.parametrize("bit", [2, 4])
-def test_quantised_decode_attention_full_size(bit):
+@pytest.mark.parametrize("bit,group_size", [(2, 64), (4, 64), (2, 32), (4, 32)])
+def test_quantised_decode_attention_full_size(bit, group_size):
     from mustafar_amd import compression_quant as cq
     from mustafar_amd import mustafar_package_quant as mpq
     from mustafar_amd import ops
     bkv = 256
     K, V, q, Kp, Vp = make_data(bkv, KTH)
     Bq, cap = bkv * GROUPS, 32 // bit
-    kq = cq.convert_key_batched_quant(Kp, return_metadata=True, bit=bit)
-    vq = cq.convert_value_batched_quant(Vp, bit=bit)
-    ks, kz, Kd = torch_quantise(Kp, False, bit)
-    vs, vz, Vd = torch_quantise(Vp, True, bit)
+    kq = cq.convert_key_batched_quant(Kp, return_metadata=True, bit=bit, group_size=group_size)
+    vq = cq.convert_value_batched_quant(Vp, bit=bit, group_size=group_size)
+    ks, kz, Kd = torch_quantise(Kp, False, bit, group_size)
+    vs, vz, Vd = torch_quantise(Vp, True, bit, group_size)
     # producer arrays at the full size: scales / zero-points bit for bit, counts = popcounts, offsets = running units
     for got, (s16, z16) in ((kq, (ks, kz)), (vq, (vs, vz))):
+        assert got[5].shape == s16.shape and got[6].shape == z16.shape
         assert torch.equal(got[5].view(torch.int16), s16.view(torch.int16))
         assert torch.equal(got[6].view(torch.int16), z16.view(torch.int16))
         pop = popcount64(got[0])

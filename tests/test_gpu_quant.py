@@ -35,19 +35,25 @@ def pruned(seed, B, M, kth=89):
     return orc.prune_rows(K, kth), orc.prune_rows(V, kth)
 
 
+@pytest.mark.parametrize("group_size", [64, 32])
 @pytest.mark.parametrize("bit", [2, 4])
 @pytest.mark.parametrize("is_value", [0, 1])
-def test_quant_compress_bit_exact(bit, is_value):
+def test_quant_compress_bit_exact(bit, is_value, group_size):
     from mustafar_amd import compression_quant as cq
     Kp, Vp = pruned(31 + bit, 3, 256)
     x = Vp if is_value else Kp
-    ref = orc.compress_quant(x, is_value, bit)
+    if group_size == 32:
+        x[1, 70, 64:96] = 0                       # a value tile whose first group is empty
+        x[2, 64:96, 20] = 0                       # a key tile whose first group is empty
+        x[2, 128:160, 21] = np.float16(-3.5)      # a group of equal survivors
+    ref = orc.compress_quant(x, is_value, bit, group_size)
     if is_value:
-        got = cq.convert_value_batched_quant(to_gpu(x), bit=bit)
+        got = cq.convert_value_batched_quant(to_gpu(x), bit=bit, group_size=group_size)
     else:
-        got = cq.convert_key_batched_quant(to_gpu(x), return_metadata=True, bit=bit)
-        short = cq.convert_key_batched_quant(to_gpu(x), bit=bit)
+        got = cq.convert_key_batched_quant(to_gpu(x), return_metadata=True, bit=bit, group_size=group_size)
+        short = cq.convert_key_batched_quant(to_gpu(x), bit=bit, group_size=group_size)
         assert len(short) == 5
+    assert tuple(got[5].shape) == ((3, 512) if group_size == 64 else (3, 512, 2))
     names = ["bitmaps", "tile_offsets", "packed", "counts", "units", "scales", "zeros"]
     dtypes = [torch.int64, torch.int32, torch.int32, torch.int32, torch.int32, torch.float16, torch.float16]
     for name, g, r, dt in zip(names, got, ref, dtypes):
@@ -105,9 +111,10 @@ def test_quant_formulations_reference_api(bit, dequant_mode):
         mq.mustafar_key_formulation_quant(kb, kp, ko, ks, kz, padded_query, Lc, D, Bq, groups, bit, cap + 1)
 
 
+@pytest.mark.parametrize("group_size", [64, 32])
 @pytest.mark.parametrize("bit", [2, 4])
 @pytest.mark.parametrize("groups,Bkv,Lc", [(4, 2, 1024), (1, 3, 256), (8, 1, 512)])
-def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc):
+def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc, group_size):
     """Quantised compress -> key SpMV -> softmax -> value SpMV against the oracle's dense masked attention run
     on the dequantised cache (the reference semantics of the quantised path), one query token per head."""
     from mustafar_amd import compression_quant as cq, mustafar_package_quant as mq, ops
@@ -116,34 +123,44 @@ def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc
     cap = 32 // bit
     K, V = orc.make_kv(500 + Lc + bit, Bkv, Lc, D)
     Kp, Vp = orc.prune_rows(K, 89), orc.prune_rows(V, 89)
-    rk = orc.compress_quant(Kp, 0, bit)
-    rv = orc.compress_quant(Vp, 1, bit)
+    rk = orc.compress_quant(Kp, 0, bit, group_size)
+    rv = orc.compress_quant(Vp, 1, bit, group_size)
     Kd = np.stack([orc.decode_quant(rk[0], rk[2], rk[1], rk[5], rk[6], b, Lc, D, 0, bit, 0) for b in range(Bkv)])
     Vd = np.stack([orc.decode_quant(rv[0], rv[2], rv[1], rv[5], rv[6], b, Lc, D, 1, bit, 0) for b in range(Bkv)])
     q = np.random.default_rng(Lc).standard_normal((Bq, D)).astype(np.float16)
     sc_ref, pr_ref, out_ref = orc.dense_masked_attention(q, Kd, Vd, groups)
 
-    kb, ko, kp, kc, ku, ks, kz = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
-    vb, vo, vp, vc, vu, vs, vz = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    kb, ko, kp, kc, ku, ks, kz = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit,
+                                                              group_size=group_size)
+    vb, vo, vp, vc, vu, vs, vz = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit, group_size=group_size)
     L = __import__("mustafar_amd._lib", fromlist=["lib"]).lib()
     st = torch.cuda.current_stream().cuda_stream
     s = torch.empty((Bq, 1, Lc), dtype=torch.float16, device=dev())
     qg = to_gpu(q).view(Bq, 1, D)
-    assert L.mstf_key_spmv_quant(st, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), None, None, ks.data_ptr(),
-                                 kz.data_ptr(), qg.data_ptr(), s.data_ptr(), Lc, D, Bq, groups, 1, bit, cap, 0) == 0
+    if group_size == 64:
+        assert L.mstf_key_spmv_quant(st, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), None, None, ks.data_ptr(),
+                                     kz.data_ptr(), qg.data_ptr(), s.data_ptr(), Lc, D, Bq, groups, 1, bit, cap, 0) == 0
+    else:
+        assert L.mstf_key_spmv_quant_grouped(st, kb.data_ptr(), kp.data_ptr(), ko.data_ptr(), ks.data_ptr(), kz.data_ptr(),
+                                             qg.data_ptr(), s.data_ptr(), Lc, D, Bq, groups, 1, bit, cap, 0, 32) == 0
     p = ops.scale_softmax(s, D)
     o = mq.mustafar_value_formulation_quant_decode_n1(vb, vp, vo, vc, vu, vs, vz, p.view(Bq, Lc), None, D, Lc, Bq,
                                                       groups, bit, cap)
     check_chain(QTOL, sc_ref, pr_ref, out_ref, Vd, groups, s=s[:, 0], p=p[:, 0], o=o)
     # the quantisation itself stays within half a step of the fp16 cache
     err = np.abs(Kd.astype(np.float32) - np.where(Kp != 0, Kp, 0).astype(np.float32))
-    step = np.repeat(rk[5].astype(np.float32).reshape(Bkv, Lc // 64, D), 64, axis=1)   # key tile = 64 tokens x 1 channel
+    if group_size == 64:
+        step = np.repeat(rk[5].astype(np.float32).reshape(Bkv, Lc // 64, D), 64, axis=1)   # key tile = 64 tokens x 1 channel
+    else:    # pair g of tile (block, channel) serves tokens 32g .. 32g+31 of the block
+        step = np.repeat(rk[5].astype(np.float32).reshape(Bkv, Lc // 64, D, 2).transpose(0, 1, 3, 2).reshape(Bkv, Lc // 32, D),
+                         32, axis=1)
     assert (err <= 0.5 * step * 1.01 + 2e-3 * np.abs(Kp.astype(np.float32)) + 1e-6).all()
 
 
+@pytest.mark.parametrize("group_size", [64, 32])
 @pytest.mark.parametrize("bit", [2, 4, 8])
 @pytest.mark.parametrize("dequant_mode", [0, 1])
-def test_quant_dequantised_values_bit_exact(bit, dequant_mode):
+def test_quant_dequantised_values_bit_exact(bit, dequant_mode, group_size):
     """One-hot query rows / probability rows turn the SpMVs into a read-out of the dequantised cache: every
     output is a single product value * 1, so it must equal the oracle's decode bit for bit.  Some tiles sit far
     from zero (zero-point beyond +-1024), which takes the kernels' literal per-mode arithmetic."""
@@ -158,7 +175,7 @@ def test_quant_dequantised_values_bit_exact(bit, dequant_mode):
     Vp[1, 7, :64] = (512.0 + (k % steps) * 0.5).astype(np.float16)
     Bq = B * groups
     for is_value, x in ((0, Kp), (1, Vp)):
-        ref = orc.compress_quant(x, is_value, bit)
+        ref = orc.compress_quant(x, is_value, bit, group_size)
         assert np.abs(ref[6].astype(np.float32)).max() > 1024      # the slow path is exercised
         dense = np.stack([orc.decode_quant(ref[0], ref[2], ref[1], ref[5], ref[6], b, M, D, is_value, bit, dequant_mode)
                           for b in range(B)])                      # [B, M, D]
@@ -195,9 +212,10 @@ def test_quant_dequantised_values_bit_exact(bit, dequant_mode):
                             assert np.array_equal(got & ((got != 0x8000) * 0xFFFF), want & ((want != 0x8000) * 0xFFFF))
 
 
+@pytest.mark.parametrize("group_size", [64, 32])
 @pytest.mark.parametrize("bit", [2, 4, 8])
 @pytest.mark.parametrize("groups,Bkv,Lc", [(4, 2, 1024), (8, 1, 576), (1, 3, 64)])
-def test_fused_quant_decode_attention(bit, groups, Bkv, Lc):
+def test_fused_quant_decode_attention(bit, groups, Bkv, Lc, group_size):
     """The one-launch path against dense masked attention on the dequantised cache (1e-2) and against the
     three-launch quantised path (same dequantised values, so only the softmax rounding differs)."""
     from mustafar_amd import compression_quant as cq
@@ -206,8 +224,8 @@ def test_fused_quant_decode_attention(bit, groups, Bkv, Lc):
     D = 128
     Bq = Bkv * groups
     Kp, Vp = pruned(90 + bit + Lc, Bkv, Lc)
-    kq = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit)
-    vq = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit)
+    kq = cq.convert_key_batched_quant(to_gpu(Kp), return_metadata=True, bit=bit, group_size=group_size)
+    vq = cq.convert_value_batched_quant(to_gpu(Vp), bit=bit, group_size=group_size)
     kr = [t.cpu().numpy() for t in kq]
     vr = [t.cpu().numpy() for t in vq]
     Kd = np.stack([orc.decode_quant(kr[0], kr[2], kr[1], kr[5], kr[6], b, Lc, D, 0, bit) for b in range(Bkv)])

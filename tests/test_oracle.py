@@ -333,3 +333,41 @@ def test_quant_spmv_reduces_to_matmul_on_dequantised(bit):
     # half-arithmetic dequant stays within the quantisation step of the fp32 one
     dq1 = orc.decode_quant(bmp, packed, toff, scales, zeros, 0, Lc, D, 0, bit, 1)
     assert np.abs(dq1.astype(np.float32) - dq[0].astype(np.float32)).max() <= 2e-2 * np.abs(dq[0].astype(np.float32)).max()
+
+
+# ------------------------------------------------------------------ group-32 option of the quantiser
+@pytest.mark.parametrize("bit", [2, 4])
+@pytest.mark.parametrize("is_value", [0, 1])
+def test_group32_reduces_to_the_per_tile_quantiser_on_half_tiles(bit, is_value):
+    """Pair g of a tile, and the codes / dequantised values of the elements 32g .. 32g+31, must be what the per-tile
+    quantiser (pinned by the reference-written fixtures) gives for the same tile with its other half emptied."""
+    Kp, Vp = _pruned(29, 2, 128)
+    x = (Vp if is_value else Kp).copy()
+    B, M, N = x.shape
+    g32 = orc.compress_quant(x, is_value, bit, 32)
+    d32 = np.stack([orc.decode_quant(g32[0], g32[2], g32[1], g32[5], g32[6], b, M, N, is_value, bit, 0) for b in range(B)])
+    assert g32[5].shape == (B, M * N // 64, 2)
+    for g in range(2):
+        half = x.copy()
+        if is_value:                       # value tile: 64 channels of one token; element i = channel 64*half + i
+            keep = ((np.arange(N) % 64) // 32 == g)
+            half[:, :, ~keep] = 0
+            pos = np.broadcast_to(keep, x.shape)
+        else:                              # key tile: 64 tokens of one channel; element i = token 64*blk + i
+            keep = ((np.arange(M) % 64) // 32 == g)
+            half[:, ~keep, :] = 0
+            pos = np.broadcast_to(keep[None, :, None], x.shape)
+        g64 = orc.compress_quant(half, is_value, bit, 64)
+        assert np.array_equal(g64[5].view(np.uint16), g32[5][..., g].view(np.uint16))     # scales
+        assert np.array_equal(g64[6].view(np.uint16), g32[6][..., g].view(np.uint16))     # zero-points
+        d64 = np.stack([orc.decode_quant(g64[0], g64[2], g64[1], g64[5], g64[6], b, M, N, is_value, bit, 0) for b in range(B)])
+        assert np.array_equal(d64[pos].view(np.uint16), d32[pos].view(np.uint16))          # same codes, same values
+    # bitmaps, counts, units and offsets do not depend on the grouping
+    g64 = orc.compress_quant(x, is_value, bit, 64)
+    for i in (0, 1, 3, 4):
+        assert np.array_equal(g64[i], g32[i])
+    # finer groups never quantise worse
+    d64 = np.stack([orc.decode_quant(g64[0], g64[2], g64[1], g64[5], g64[6], b, M, N, is_value, bit, 0) for b in range(B)])
+    e32 = np.abs(d32.astype(np.float32) - x.astype(np.float32))
+    e64 = np.abs(d64.astype(np.float32) - x.astype(np.float32))
+    assert e32.mean() <= e64.mean()
