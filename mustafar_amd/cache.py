@@ -75,8 +75,8 @@ class CompressedPool:
         self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens = 0
 
-    def append(self, x, kth):
-        """x: [heads, M, head_dim] fp16, M % 64 == 0."""
+    def append(self, x, kth, ws=None):
+        """x: [heads, M, head_dim] fp16, M % 64 == 0.  ws: the caller's ops.Workspace (default: the stream's)."""
         B, M, N = x.shape
         assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
         x = x.contiguous()
@@ -85,7 +85,7 @@ class CompressedPool:
         bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
         idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
         dst = self.nz_off + self.idx[:, -1] // 4          # 16-byte units; idx counts 4-byte units
-        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, M, N))
+        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, M, N), ws)
         fn = L.mstf_append_value_f16 if self.is_value else L.mstf_append_key_f16
         check(fn(torch.cuda.current_stream().cuda_stream, x.data_ptr(), B, M, N, int(kth), bmp_c.data_ptr(),
                  idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(), self.overflow.data_ptr(),
@@ -94,7 +94,7 @@ class CompressedPool:
         self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
         self.tokens += M
 
-    def append_proj(self, x, kth, M, cos=None, sin=None, rot=None):
+    def append_proj(self, x, kth, M, cos=None, sin=None, rot=None, ws=None):
         """The first M tokens of x [batch, rows, heads per batch entry, head_dim] (a view of the projection output,
         ops.proj_source) without a contiguous copy; with cos / sin all rows are rotated into rot (default: in place)
         before the first M are compressed."""
@@ -107,7 +107,7 @@ class CompressedPool:
         bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
         idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
         dst = self.nz_off + self.idx[:, -1] // 4
-        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, max(M, 64), N))
+        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, max(M, 64), N), ws)
         check(L.mstf_append_proj_f16(torch.cuda.current_stream().cuda_stream, ctypes.byref(src), int(self.is_value), M, N,
                                      int(kth), bmp_c.data_ptr(), idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(),
                                      self.nz.data_ptr(), self.overflow.data_ptr(), ws.data_ptr(), ws.numel()),
@@ -151,6 +151,12 @@ class SparseKVCache:
         self.k_win = self.v_win = None      # [bs, n_kv, Lw, D] dense
         self.compressed_length = 0
         self.kv_len = 0
+        self.ws = None                      # ops.Workspace of this cache: never shared with another cache or stream
+
+    def _workspace(self, device):
+        if self.ws is None:
+            self.ws = ops.Workspace(device)
+        return self.ws
 
     def _grow(self, K, V):
         """Adds the tokens K, V [bs, n_kv, M, D] to the compressed part."""
@@ -159,8 +165,9 @@ class SparseKVCache:
             if self.k_pool is None:
                 self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, K.device)
                 self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, K.device)
-            self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k)
-            self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v)
+            ws = self._workspace(K.device)
+            self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
+            self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
             self.k, self.v = self.k_pool.view(), self.v_pool.view()
             return
         ck, cv = self._compress(K, V)
@@ -169,8 +176,9 @@ class SparseKVCache:
 
     def _compress(self, K, V):
         bs, n_kv, L, D = K.shape
-        ck = ops.compress(K.reshape(bs * n_kv, L, D), False, kth=self.kth_k)
-        cv = ops.compress(V.reshape(bs * n_kv, L, D), True, kth=self.kth_v)
+        ws = self._workspace(K.device)
+        ck = ops.compress(K.reshape(bs * n_kv, L, D), False, kth=self.kth_k, ws=ws)
+        cv = ops.compress(V.reshape(bs * n_kv, L, D), True, kth=self.kth_v, ws=ws)
         return ck, cv
 
     def prefill_proj(self, kx, vx, cos, sin):
@@ -185,14 +193,16 @@ class SparseKVCache:
             if self.k_pool is None:
                 self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, kx.device)
                 self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, kx.device)
-            self.k_pool.append_proj(kx, self.kth_k, Lc, cos, sin)
+            ws = self._workspace(kx.device)
+            self.k_pool.append_proj(kx, self.kth_k, Lc, cos, sin, ws=ws)
             if Lc > 0:
-                self.v_pool.append_proj(vx, self.kth_v, Lc)
+                self.v_pool.append_proj(vx, self.kth_v, Lc, ws=ws)
                 self.k, self.v = self.k_pool.view(), self.v_pool.view()
         else:
-            ck, _ = ops.compress_proj(kx, False, self.kth_k, Lc, cos, sin)
+            ws = self._workspace(kx.device)
+            ck, _ = ops.compress_proj(kx, False, self.kth_k, Lc, cos, sin, ws=ws)
             if Lc > 0:
-                cv, _ = ops.compress_proj(vx, True, self.kth_v, Lc)
+                cv, _ = ops.compress_proj(vx, True, self.kth_v, Lc, ws=ws)
                 self.k, self.v = ck, cv
         K, V = kx.transpose(1, 2), vx.transpose(1, 2)
         self._prefill_window(K, V, Lc)
@@ -245,7 +255,7 @@ class SparseKVCache:
     def _attend_device(self, q2):
         """Attention of the query rows q2 [Bq, D] over [compressed | window buffer] (three launches)."""
         return ops.decode_attention_window(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1], self.groups,
-                                           win_len_dev=self._wlen_dev)
+                                           win_len_dev=self._wlen_dev, ws=self._workspace(q2.device))
 
     def advance(self):
         """Host-side bookkeeping after decode_device (or a replay of it): counts the token and, when the window holds
@@ -278,7 +288,8 @@ class SparseKVCache:
         bs, n_q, _, D = q.shape
         g = self.groups
         lse = torch.empty((bs * n_q, 2), dtype=torch.float32, device=q.device)
-        o_c = ops.decode_attention(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), g, lse=lse)
+        o_c = ops.decode_attention(self.k, self.v, q.reshape(bs * n_q, D).contiguous(), g, lse=lse,
+                                   ws=self._workspace(q.device))
         m_c = lse[:, 0].view(bs, n_q, 1, 1)
         l_c = lse[:, 1].view(bs, n_q, 1, 1)
         w = (s_loc / ops.sqrt_head_dim(D)).float()        # fp16 division first, as for the compressed scores
@@ -309,7 +320,8 @@ class SparseKVCache:
             p = ops.scale_softmax(s.contiguous(), D)
             out = torch.matmul(p[..., Lc:], _repeat_kv(self.v_win, g))
             if Lc > 0:
-                o_cmp = ops.value_spmv(self.v, p[..., :Lc].reshape(bs * n_q, 1, Lc).contiguous(), g)
+                o_cmp = ops.value_spmv(self.v, p[..., :Lc].reshape(bs * n_q, 1, Lc).contiguous(), g,
+                                       ws=self._workspace(q.device))
                 out = out + o_cmp.view(bs, n_q, 1, D)
         if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.k_win.shape[2] >= CHUNK:
             self._grow(self.k_win[:, :, :CHUNK].contiguous(), self.v_win[:, :, :CHUNK].contiguous())
@@ -344,13 +356,14 @@ class QuantSparseKVCache(SparseKVCache):
     def _attend_device(self, q2):
         from . import mustafar_package_quant as mpq
         return mpq.decode_attention_window_quant(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1],
-                                                 self.groups, self.bit, self.dequant_mode, win_len_dev=self._wlen_dev)
+                                                 self.groups, self.bit, self.dequant_mode, win_len_dev=self._wlen_dev,
+                                                 ws=self._workspace(q2.device))
 
     def prefill_proj(self, kx, vx, cos, sin):
         """As SparseKVCache.prefill_proj for the rotation - the keys are rotated in place by the compressor's kernel,
         in the projection's own layout - while the quantised producer, which takes contiguous rows like the
         reference's, goes through prefill on the transposed views."""
-        ops.compress_proj(kx, False, self.kth_k, 0, cos, sin)      # M = 0: rotation only
+        ops.compress_proj(kx, False, self.kth_k, 0, cos, sin, ws=self._workspace(kx.device))      # M = 0: rotation only
         K, V = kx.transpose(1, 2), vx.transpose(1, 2)
         self.prefill(K, V)
         return K, V
@@ -360,8 +373,9 @@ class QuantSparseKVCache(SparseKVCache):
         bs, n_kv, M, D = K.shape
         Kp = ops.prune_rows(K.reshape(-1, D).contiguous(), self.kth_k).view(bs * n_kv, M, D)
         Vp = ops.prune_rows(V.reshape(-1, D).contiguous(), self.kth_v).view(bs * n_kv, M, D)
-        return (list(cq.convert_key_batched_quant(Kp, return_metadata=True, bit=self.bit)),
-                list(cq.convert_value_batched_quant(Vp, bit=self.bit)))
+        ws = self._workspace(K.device)
+        return (list(cq.convert_key_batched_quant(Kp, return_metadata=True, bit=self.bit, ws=ws)),
+                list(cq.convert_value_batched_quant(Vp, bit=self.bit, ws=ws)))
 
     @staticmethod
     def _append(old, new):
@@ -391,7 +405,7 @@ class QuantSparseKVCache(SparseKVCache):
         if Lc > 0 and self.fused:
             lse = torch.empty((Bq, 2), dtype=torch.float32, device=q.device)
             o_c = mpq.decode_attention_quant(self.k, self.v, q.reshape(Bq, D).contiguous(), g, self.bit,
-                                             self.dequant_mode, lse=lse)
+                                             self.dequant_mode, lse=lse, ws=self._workspace(q.device))
             m_c, l_c = lse[:, 0].view(bs, n_q, 1, 1), lse[:, 1].view(bs, n_q, 1, 1)
             w = (s_loc / ops.sqrt_head_dim(D)).float()
             M = torch.maximum(m_c, w.amax(-1, keepdim=True))

@@ -11,7 +11,7 @@ from . import ops
 from ._lib import check, lib
 
 
-def _convert(inputs, is_value, bit, kth=0, group_size=64):
+def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
     assert inputs.is_cuda
     assert inputs.dim() == 3
     B, M, N = inputs.shape
@@ -32,7 +32,7 @@ def _convert(inputs, is_value, bit, kth=0, group_size=64):
     scales = torch.empty(meta_shape, dtype=torch.float16, device=dev)
     zeros = torch.empty(meta_shape, dtype=torch.float16, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
-    ws = ops.workspace(dev, L.mstf_compress_quant_workspace_bytes(B, M, N))
+    ws = ops.workspace(dev, L.mstf_compress_quant_workspace_bytes(B, M, N), ws)
     name = "mstf_compress_quant_grouped"
     st = torch.cuda.current_stream().cuda_stream
     # one pass with room for the worst case (every element kept: 64 // capacity words per tile), then the used
@@ -49,12 +49,13 @@ def _convert(inputs, is_value, bit, kth=0, group_size=64):
     return bmp, tile_off, packed, counts, units, scales, zeros
 
 
-def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2, group_size: int = 64):
-    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit, group_size=group_size)
+def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2, group_size: int = 64,
+                              ws=None):
+    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit, group_size=group_size, ws=ws)
     if return_metadata:
         return bmp, tile_off, packed, counts, units, scales, zeros
     return bmp, tile_off, packed, scales, zeros
 
 
-def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2, group_size: int = 64):
-    return _convert(inputs, True, bit, group_size=group_size)
+def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2, group_size: int = 64, ws=None):
+    return _convert(inputs, True, bit, group_size=group_size, ws=ws)

@@ -158,15 +158,16 @@ __device__ __forceinline__ void words_issue_flat(const uint32_t* src, uint32_t n
 {
     static_assert(PIECES == 2 || PIECES == 4 || PIECES == 8, "pieces of 64 words");
     uint32_t t, m0_kept;
+    uint64_t sv;  // exec as found, handed back
 #define MSTF_WPIECE(I)                                                     \
     "s_sub_i32 %[t], %[n], " #I " * 64\n\t"                                \
     "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"                                     \
     "s_mov_b64 exec, vcc\n\t"                                              \
     "global_load_lds_dword %[l4], %[src] offset:" #I " * 256\n\t"
-#define MSTF_WHEAD "s_mov_b32 %[keep], m0\n\ts_mov_b32 m0, %[dst]\n\t"
-#define MSTF_WTAIL "s_mov_b64 exec, -1\n\ts_mov_b32 m0, %[keep]"
+#define MSTF_WHEAD "s_mov_b32 %[keep], m0\n\ts_mov_b64 %[sv], exec\n\ts_mov_b32 m0, %[dst]\n\t"
+#define MSTF_WTAIL "s_mov_b64 exec, %[sv]\n\ts_mov_b32 m0, %[keep]"
 #define MSTF_WOPS                                                                                      \
-    : [t] "=&s"(t), [keep] "=&s"(m0_kept)                                                              \
+    : [t] "=&s"(t), [keep] "=&s"(m0_kept), [sv] "=&s"(sv)                                              \
     : [dst] "s"(dst_lds), [n] "s"(nw), [l] "v"(lane), [l4] "v"(lane4), [src] "s"(src)                  \
     : "vcc", "scc", "memory"
     if constexpr (PIECES == 2)
@@ -249,6 +250,7 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
 #pragma unroll
     for (int m = 1; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(wbase + (uint32_t)WOFF + (uint32_t)m * wgroup);
     uint32_t v0, v1, v2, v3;
+    uint64_t sv;  // exec as found, handed back
 #define MSTF_TILE(I, H, A)                                       \
     "s_brev_b64 exec, %[m" #I "]\n\t"                            \
     "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
@@ -256,12 +258,13 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
     "v_lshl_add_u32 v" #A ", v" #A ", 1, %[img]\n\t"             \
     "ds_read_u16 v" #H ", v" #A " offset:%[i" #I "]\n\t"
 #define MSTF_GATHER                                                                                  \
+    "s_mov_b64 %[sv], exec\n\t"                                                                      \
     "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                   \
     "ds_read_b128 v[112:115], %[z]\n\t"                                                              \
     "ds_read_b128 v[116:119], %[z]\n\t"                                                              \
     MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)      \
     MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)      \
-    "s_mov_b64 exec, -1\n\t"                                                                         \
+    "s_mov_b64 exec, %[sv]\n\t"                                                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                       \
     "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                        \
     "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                        \
@@ -278,12 +281,13 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
         "v126", "v127", "memory"
     if constexpr (PREFETCH) {
         asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t" MSTF_GATHER
-                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [nm] "=&s"(nxt)
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [sv] "=&s"(sv),
+                       [nm] "=&s"(nxt)
                      : MSTF_IN, [nb] "s"(bm), [boff] "i"(BOFF)
                      : MSTF_CLOBBER);
     } else {
         asm volatile(MSTF_GATHER
-                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0])
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [sv] "=&s"(sv)
                      : MSTF_IN
                      : MSTF_CLOBBER);
         nxt = mv;

@@ -68,7 +68,10 @@ struct Batch {
 // top), so the select instruction disappears - per tile one s_brev_b64 into exec, two v_mbcnt on exec, the
 // scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (v112-v127, the top of the
 // budget of a kernel that runs four wavefronts per SIMD, listed as clobbered) because nothing of the compiler's may
-// be scheduled while exec is partial; the wavefront must be in uniform control flow with all 64 lanes active.  The scalar loads of the coming batch (PREFETCH) are part of the
+// be scheduled while exec is partial.  The statement saves the exec mask it is entered with and hands it back, but
+// between the two every tile runs under its own bitmap: callers sit in wave-uniform control flow with all 64 lanes
+// active (every kernel that uses it is launched with a multiple of 64 threads and branches only on wave-uniform values
+// around it).  The scalar loads of the coming batch (PREFETCH) are part of the
 // statement: requested first, completed by its one wait - the compiler, which cannot see that wait, would otherwise
 // put one of its own in front of the statement and expose the round trip of a request it has just made.
 //   nbm + BOFF bytes, nix + IOFF bytes : bitmaps and offsets of the coming batch
@@ -82,6 +85,7 @@ __device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, cons
 #pragma unroll
     for (int m = 1; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(wbase + (uint32_t)WOFF + (uint32_t)m * wgroup);
     uint32_t v0, v1, v2, v3, t;
+    uint64_t sv;  // the exec mask the statement was entered with, handed back at its end
 #define MSTF_TILE(I, H, A)                                       \
     "s_brev_b64 exec, %[m" #I "]\n\t"                            \
     "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
@@ -90,12 +94,13 @@ __device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, cons
     "v_lshl_add_u32 v" #A ", v" #A ", 1, %[t]\n\t"               \
     "ds_read_u16 v" #H ", v" #A "\n\t"
 #define MSTF_GATHER                                                                                                  \
+    "s_mov_b64 %[sv], exec\n\t"                                                                                      \
     "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                                   \
     "ds_read_b128 v[112:115], %[z]\n\t"                                                                              \
     "ds_read_b128 v[116:119], %[z]\n\t"                                                                              \
     MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)                              \
     MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)                              \
-    "s_mov_b64 exec, -1\n\t"                                                                                         \
+    "s_mov_b64 exec, %[sv]\n\t"                                                                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
     "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                                          \
     "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                                          \
@@ -114,12 +119,13 @@ __device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, cons
         asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t"
                      "s_load_dwordx8 %[no], %[ni], %[ioff]\n\t" MSTF_GATHER
                      : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [t] "=&s"(t),
-                       [nm] "=&s"(nxt.mv), [no] "=&s"(nxt.ov)
+                       [sv] "=&s"(sv), [nm] "=&s"(nxt.mv), [no] "=&s"(nxt.ov)
                      : MSTF_GATHER_IN, [nb] "s"(nbm), [ni] "s"(nix), [boff] "i"(BOFF), [ioff] "i"(IOFF)
                      : MSTF_GATHER_CLOBBER);
     } else {
         asm volatile(MSTF_GATHER
-                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [t] "=&s"(t)
+                     : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [t] "=&s"(t),
+                       [sv] "=&s"(sv)
                      : MSTF_GATHER_IN
                      : MSTF_GATHER_CLOBBER);
         nxt = b;
@@ -194,7 +200,9 @@ __device__ __forceinline__ void sub_issue_flat(const char* src, uint32_t bytes, 
 {
     static_assert(kSubBytes == 4096, "four 1 KB pieces");
     uint32_t t, m0_kept;  // m0 is the compiler's to manage: handed back as it was found
+    uint64_t sv;          // so is exec
     asm volatile("s_mov_b32 %[keep], m0\n\t"
+                 "s_mov_b64 %[sv], exec\n\t"
                  "s_mov_b32 m0, %[dst]\n\t"
                  "v_cmp_gt_i32 vcc, %[b], %[l]\n\t"
                  "s_mov_b64 exec, vcc\n\t"
@@ -211,9 +219,9 @@ __device__ __forceinline__ void sub_issue_flat(const char* src, uint32_t bytes, 
                  "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
                  "s_mov_b64 exec, vcc\n\t"
                  "global_load_lds_dwordx4 %[l], %[src] offset:3072\n\t"
-                 "s_mov_b64 exec, -1\n\t"
+                 "s_mov_b64 exec, %[sv]\n\t"
                  "s_mov_b32 m0, %[keep]"
-                 : [t] "=&s"(t), [keep] "=&s"(m0_kept)
+                 : [t] "=&s"(t), [keep] "=&s"(m0_kept), [sv] "=&s"(sv)
                  : [dst] "s"(dst_lds), [b] "s"(bytes), [l] "v"(lane16), [src] "s"(src)
                  : "vcc", "scc", "memory");
 }

@@ -121,7 +121,8 @@ def mustafar_value_formulation_quant_decode_n1(bmp, NZ_quant, tile_offsets, tile
                   "mustafar_value_formulation_quant_decode_n1")
 
 
-def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, dequant_mode=0, out=None, lse=None):
+def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, dequant_mode=0, out=None, lse=None,
+                           ws=None):
     """One launch for key SpMV -> / sqrt(d) -> softmax -> value SpMV over a quantised cache (no counterpart in the
     reference, which runs the three steps separately).
 
@@ -137,7 +138,7 @@ def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, d
     tokens = kb.shape[1] * 64 // D
     L = lib()
     o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
-    ws = ops.workspace(q.device, L.mstf_decode_attention_workspace_bytes(tokens, D, Bq, num_key_value_groups))
+    ws = ops.workspace(q.device, L.mstf_decode_attention_workspace_bytes(tokens, D, Bq, num_key_value_groups), ws)
     group_size = _group_size(kb, ks, kz)
     if _group_size(vb, vs, vz) != group_size:
         raise RuntimeError("key side and value side must use the same group size.")
@@ -151,7 +152,7 @@ def decode_attention_quant(key_side, value_side, q, num_key_value_groups, bit, d
 
 
 def decode_attention_window_quant(key_side, value_side, q, k_win, v_win, win_len, num_key_value_groups, bit,
-                                  dequant_mode=0, out=None, lse=None, win_len_dev=None):
+                                  dequant_mode=0, out=None, lse=None, win_len_dev=None, ws=None):
     """The whole attention of a decode step over [quantised compressed tokens | dense window] in three launches
     (ops.decode_attention_window for the quantised format).  key_side / value_side may be None while nothing is
     compressed yet.  k_win, v_win: [Bkv, stride, 128] fp16, the first win_len tokens valid; win_len_dev: optional
@@ -173,7 +174,7 @@ def decode_attention_window_quant(key_side, value_side, q, k_win, v_win, win_len
     else:
         tokens, ptrs = 0, [None] * 10
     ws = ops.workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(tokens, int(win_len), D, Bq,
-                                                                                int(num_key_value_groups)))
+                                                                                int(num_key_value_groups)), ws)
     check(L.mstf_decode_attention_window_quant(
         torch.cuda.current_stream().cuda_stream, *ptrs, q.contiguous().data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
         int(win_len), win_len_dev.data_ptr() if win_len_dev is not None else None, int(k_win.shape[1]), o.data_ptr(),

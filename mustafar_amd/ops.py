@@ -9,6 +9,37 @@ import torch
 
 from ._lib import check, lib
 
+class Workspace:
+    """Scratch memory for the entry points that need it (split partials, compressor scans), owned by one caller.
+
+    A cache, a decode loop or a benchmark that records its calls into a HIP graph creates one sized for its largest
+    call BEFORE capturing and passes it as `ws=`: the buffer then never moves, and calls on different streams with
+    different workspaces are independent.  `get` hands out the buffer if it is large enough; growing replaces it but
+    keeps the old buffers alive (a captured graph may still point at them), and growing while the current stream is
+    being captured is an error."""
+
+    def __init__(self, device, nbytes=1 << 20):
+        self.device = torch.device(device)
+        self._bufs = [torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)]
+
+    @property
+    def tensor(self):
+        return self._bufs[-1]
+
+    def reserve(self, nbytes):
+        """Makes room for nbytes; to be called outside any graph capture."""
+        if self.tensor.numel() < nbytes:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("workspace of %d bytes is too small for a call that needs %d and cannot grow while "
+                                   "the stream is being captured: reserve() it before the capture"
+                                   % (self.tensor.numel(), nbytes))
+            self._bufs.append(torch.empty(int(nbytes), dtype=torch.uint8, device=self.device))
+        return self.tensor
+
+    def get(self, nbytes):
+        return self.reserve(nbytes)
+
+
 _WS = {}
 
 
@@ -16,14 +47,18 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def workspace(device, nbytes):
-    """A per-device scratch tensor that only grows (256-byte aligned by the caching allocator)."""
-    key = (device.type, device.index)
-    t = _WS.get(key)
-    if t is None or t.numel() < nbytes:
-        t = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-        _WS[key] = t
-    return t
+def workspace(device, nbytes, ws=None):
+    """The scratch tensor for a call that needs nbytes: the caller's Workspace (`ws`) or, for the mirrors of the
+    reference's operators, which have no such argument, a default one per (device, stream) - so two streams never
+    share a buffer unless the caller passes the same Workspace to both."""
+    if ws is not None:
+        return ws.get(nbytes) if isinstance(ws, Workspace) else ws
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), _stream())
+    w = _WS.get(key)
+    if w is None:
+        w = _WS[key] = Workspace(device)
+    return w.get(nbytes)
 
 
 def kth_from_sparsity(sparsity, head_dim):
@@ -65,7 +100,7 @@ def prune_rows(x, kth, out=None):
     return y
 
 
-def compress(x, is_value, kth=0, capacity_halfs=None):
+def compress(x, is_value, kth=0, capacity_halfs=None, ws=None):
     """Prune (kth > 0) and compress x [B, M, N] into the bitmap format.
 
     With capacity_halfs=None the packed size is read back once (like the reference's .item());
@@ -81,7 +116,7 @@ def compress(x, is_value, kth=0, capacity_halfs=None):
     nz_off = torch.empty((B,), dtype=torch.int32, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
     wsb = L.mstf_compress_workspace_bytes(B, M, N)
-    ws = workspace(dev, wsb)
+    ws = workspace(dev, wsb, ws)
     fn = L.mstf_compress_value_f16 if is_value else L.mstf_compress_key_f16
     name = "mstf_compress_value_f16" if is_value else "mstf_compress_key_f16"
     if capacity_halfs is None:
@@ -124,7 +159,7 @@ def proj_source(x, cos=None, sin=None, rot=None):
     return src, rot
 
 
-def compress_proj(x, is_value, kth, M, cos=None, sin=None, rot=None, capacity_halfs=None):
+def compress_proj(x, is_value, kth, M, cos=None, sin=None, rot=None, capacity_halfs=None, ws=None):
     """Prune and compress the first M tokens of x [batch, rows, heads, 128] where the projection left them, the keys
     rotated first when cos / sin are given (all rows are rotated and written to rot).  Heads are numbered
     batch * heads + head.  Returns (CompressedKV, rot)."""
@@ -139,7 +174,7 @@ def compress_proj(x, is_value, kth, M, cos=None, sin=None, rot=None, capacity_ha
     nz_off = torch.empty((B,), dtype=torch.int32, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
     nz = torch.empty((max(cap, 8),), dtype=torch.float16, device=dev)
-    ws = workspace(dev, L.mstf_compress_workspace_bytes(B, max(M, 64), N))
+    ws = workspace(dev, L.mstf_compress_workspace_bytes(B, max(M, 64), N), ws)
     check(L.mstf_compress_proj_f16(_stream(), ctypes.byref(src), int(is_value), M, N, int(kth), bmp.data_ptr(),
                                    idx.data_ptr(), nz_off.data_ptr(), total.data_ptr(), nz.data_ptr(), cap,
                                    ws.data_ptr(), ws.numel()), "mstf_compress_proj_f16")
@@ -162,21 +197,21 @@ def key_spmv(ck, q, groups, n_rows=1, out=None):
     return C
 
 
-def value_spmv(cv, p, groups, n_rows=1, out=None):
+def value_spmv(cv, p, groups, n_rows=1, out=None, ws=None):
     """out[bq, n, d] = sum_t V[bq // groups][t, d] * p[bq, n, t].  p: [Bq, n_rows, Lc]."""
     assert p.dtype == torch.float16 and p.is_contiguous()
     Bq = p.numel() // (n_rows * cv.tokens)
     L = lib()
     C = torch.empty((Bq, n_rows, cv.head_dim), dtype=torch.float16, device=p.device) if out is None else out
     wsb = L.mstf_value_spmv_workspace_bytes(cv.head_dim, cv.tokens, Bq, groups, n_rows)
-    ws = workspace(p.device, wsb)
+    ws = workspace(p.device, wsb, ws)
     check(L.mstf_value_spmv_f16(_stream(), cv.bmp.data_ptr(), cv.nz.data_ptr(), cv.idx.data_ptr(),
                                 cv.nz_off.data_ptr(), p.data_ptr(), C.data_ptr(), cv.head_dim, cv.tokens, Bq, groups,
                                 n_rows, ws.data_ptr(), ws.numel()), "mstf_value_spmv_f16")
     return C
 
 
-def decode_attention(ck, cv, q, groups, out=None, lse=None):
+def decode_attention(ck, cv, q, groups, out=None, lse=None, ws=None):
     """Fused key SpMV -> scale+softmax -> value SpMV over the compressed tokens, one query row per head.
 
     q: [Bq, D] fp16 -> out [Bq, D] fp16.  lse (optional fp32 [Bq, 2]) receives (max, sum) of every row."""
@@ -185,7 +220,7 @@ def decode_attention(ck, cv, q, groups, out=None, lse=None):
     Bq = q.numel() // D
     L = lib()
     o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
-    ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups))
+    ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups), ws)
     check(L.mstf_decode_attention_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
                                       ck.nz_off.data_ptr(), cv.bmp.data_ptr(), cv.nz.data_ptr(), cv.idx.data_ptr(),
                                       cv.nz_off.data_ptr(), q.data_ptr(), o.data_ptr(),
@@ -209,7 +244,7 @@ def decode_attention_static(ck, cv, q, groups, out=None, lse=None):
     return o
 
 
-def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, lse=None, win_len_dev=None):
+def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, lse=None, win_len_dev=None, ws=None):
     """Attention of one decode step over [compressed tokens | dense window] under one softmax, three launches.
 
     ck, cv: CompressedKV or None (nothing compressed yet); q: [Bq, D]; k_win, v_win: [Bkv, win_stride, D] fp16 with
@@ -222,7 +257,7 @@ def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, 
     tokens = ck.tokens if ck is not None else 0
     L = lib()
     o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
-    ws = workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(tokens, int(win_len), D, Bq, groups))
+    ws = workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(tokens, int(win_len), D, Bq, groups), ws)
     cp = [t.data_ptr() for t in (ck.bmp, ck.nz, ck.idx, ck.nz_off, cv.bmp, cv.nz, cv.idx, cv.nz_off)] if tokens else [None] * 8
     check(L.mstf_decode_attention_window_f16(_stream(), *cp, q.data_ptr(), k_win.data_ptr(), v_win.data_ptr(), int(win_len),
                                              win_len_dev.data_ptr() if win_len_dev is not None else None,
@@ -238,8 +273,7 @@ def decode_attention_partial(ck, cv, q, groups, ws=None):
     D = ck.head_dim
     Bq = q.numel() // D
     L = lib()
-    if ws is None:
-        ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups))
+    ws = workspace(q.device, L.mstf_decode_attention_workspace_bytes(ck.tokens, D, Bq, groups), ws)
     check(L.mstf_decode_attention_partial_f16(_stream(), ck.bmp.data_ptr(), ck.nz.data_ptr(), ck.idx.data_ptr(),
                                               ck.nz_off.data_ptr(), cv.bmp.data_ptr(), cv.nz.data_ptr(),
                                               cv.idx.data_ptr(), cv.nz_off.data_ptr(), q.data_ptr(), ck.tokens, D, Bq,

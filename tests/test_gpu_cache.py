@@ -158,3 +158,34 @@ def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
             for t in (0, 17, units.shape[1] // 2 + 3, units.shape[1] - 1):
                 n = int(units[h, t])
                 assert np.array_equal(got_words[got_off[h, t]:got_off[h, t] + n], ref[2][ref[1][h, t]:ref[1][h, t] + n])
+
+
+def test_workspaces_are_owned_and_do_not_move_under_capture():
+    """Every cache has its own scratch buffer; the default one is per (device, stream); a buffer that was handed out
+    stays alive when a larger one replaces it; growing while the stream is being captured is refused."""
+    from mustafar_amd import ops
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    a, b = ops.Workspace(dev, 1024), ops.Workspace(dev, 1024)
+    assert a.tensor.data_ptr() != b.tensor.data_ptr()
+    first = a.get(512)
+    ptr = first.data_ptr()
+    big = a.get(1 << 16)                                   # grows: a new buffer, the old one kept alive
+    assert big.numel() >= 1 << 16 and first.data_ptr() == ptr and a._bufs[0] is first
+    assert a.get(100).data_ptr() == big.data_ptr()          # no shrink, no further move
+    # default workspaces: one per stream
+    s1 = torch.cuda.Stream()
+    d0 = ops.workspace(dev, 256)
+    with torch.cuda.stream(s1):
+        d1 = ops.workspace(dev, 256)
+    assert d0.data_ptr() != d1.data_ptr()
+    # a capture must not make a workspace grow
+    small = ops.Workspace(dev, 256)
+    g = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="reserve"):
+        with torch.cuda.graph(g):
+            small.get(1 << 20)
+    small.reserve(1 << 20)                                  # outside the capture it is fine
+    cache_a = SparseKVCache(4, max_tokens=512, window_kernel=True)
+    cache_b = SparseKVCache(4, max_tokens=512, window_kernel=True)
+    assert cache_a._workspace(dev) is not cache_b._workspace(dev)
