@@ -220,6 +220,21 @@ int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_bmp, const 
                                      int tokens, int head_dim, int Bq, int groups, void* workspace,
                                      size_t workspace_bytes);
 
+/* mstf_decode_attention_window_f16 over a cache that is pre-allocated for more tokens than it holds and grows in
+ * place (mstf_append_*_f16 into per-head slabs): the bitmap rows of two heads lie tile_capacity tiles apart
+ * (tile_capacity >= max_tokens * head_dim / 64), the offset rows tile_capacity + 1, and the number of cached tokens
+ * is read from device memory - min(*tokens_dev, max_tokens), a multiple of 64, may be 0 - while max_tokens sizes the
+ * launch and the workspace (mstf_decode_attention_window_workspace_bytes(max_tokens, ...)).  A call recorded into a
+ * HIP graph therefore stays valid while chunks are appended between replays: no array moves and no argument
+ * changes (the reference re-concatenates every per-tile array per chunk, models/llama_mustafar_kernel.py:461-511). */
+int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                                          const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                                          const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q,
+                                          const mstf_half* k_win, const mstf_half* v_win, int win_len,
+                                          const int32_t* win_len_dev, int win_stride, mstf_half* out, float* lse_out,
+                                          int max_tokens, const int32_t* tokens_dev, int64_t tile_capacity, int head_dim,
+                                          int Bq, int groups, void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),
  * with the bit width a parameter (the reference hard-codes 2).  Same tiles and bitmaps as above;

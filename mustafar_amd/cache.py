@@ -55,25 +55,57 @@ class CompressedPool:
 
     Every head owns a slab of the packed-value pool (nz_off[b] = start of slab b, which the format allows); a chunk
     is compressed straight to the end of each head's values by mstf_append_*_f16, so appending re-copies no packed
-    values, reads nothing back to the host and launches the same three kernels whatever the cache holds.  Only the
-    small per-tile arrays (bitmaps, offsets: 12 bytes per 64 elements) are re-concatenated, on the device.
+    values, reads nothing back to the host and launches the same three kernels whatever the cache holds.  The per-tile
+    arrays are pre-allocated for max_tokens too (bmp_store [heads, tile_capacity], idx_store [heads, tile_capacity + 1])
+    and a chunk's bitmaps and offsets are written behind the ones that are there, so no array of the pool ever moves;
+    the number of tokens held is mirrored in device memory (tokens_dev) for consumers recorded into a HIP graph
+    (ops.decode_attention_window_pool).
 
     slab_fraction: slab size relative to the dense size of max_tokens tokens (1.0 can never overflow; smaller
-    saves memory and is guarded by the sticky `overflow` flag, to be checked by the caller at a point where it
-    synchronises anyway)."""
+    saves memory and is guarded by the sticky `overflow` flag: check_overflow() raises once it is set)."""
 
     def __init__(self, heads, head_dim, max_tokens, is_value, device, slab_fraction=1.0):
         assert max_tokens % 64 == 0
         self.heads, self.head_dim, self.is_value, self.max_tokens = heads, head_dim, is_value, max_tokens
+        self.slab_fraction = slab_fraction
         slab16 = (int(math.ceil(max_tokens * head_dim * 2 * slab_fraction)) + 15) // 16
         self.slab16 = slab16
         self.nz = torch.zeros(heads * slab16 * 8, dtype=torch.float16, device=device)
         self.nz_off = (torch.arange(heads, device=device, dtype=torch.int64) * slab16).to(torch.int32)
         self.limit = (self.nz_off.to(torch.int64) + slab16).to(torch.int32)
-        self.bmp = torch.empty((heads, 0), dtype=torch.int64, device=device)
-        self.idx = torch.zeros((heads, 1), dtype=torch.int32, device=device)
+        self.tile_capacity = max_tokens * head_dim // 64
+        self.bmp_store = torch.zeros((heads, self.tile_capacity), dtype=torch.int64, device=device)
+        self.idx_store = torch.zeros((heads, self.tile_capacity + 1), dtype=torch.int32, device=device)
         self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
+        self.tokens_dev = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens = 0
+
+    @property
+    def tiles(self):
+        return self.tokens * self.head_dim // 64
+
+    @property
+    def bmp(self):
+        """Bitmaps of the tokens held, [heads, tiles] (a view of the pre-allocated array: rows are tile_capacity apart)."""
+        return self.bmp_store[:, :self.tiles]
+
+    @property
+    def idx(self):
+        return self.idx_store[:, :self.tiles + 1]
+
+    def _publish(self, bmp_c, idx_c, M):
+        """Writes a chunk's bitmaps and offsets (counted from the chunk's first value) behind the ones held."""
+        T0, Tc = self.tiles, bmp_c.shape[1]
+        self.bmp_store[:, T0:T0 + Tc] = bmp_c
+        self.idx_store[:, T0 + 1:T0 + Tc + 1] = idx_c[:, 1:] + self.idx_store[:, T0:T0 + 1]
+        self.tokens += M
+        self.tokens_dev += M
+
+    def check_overflow(self):
+        """Raises if a chunk did not fit into a head's slab (possible only with slab_fraction < 1; one host read)."""
+        if self.slab_fraction < 1.0 and int(self.overflow) != 0:
+            raise RuntimeError("compressed pool overflow: a head's packed values outgrew its slab "
+                               "(slab_fraction %.2f); the cache is no longer usable" % self.slab_fraction)
 
     def append(self, x, kth, ws=None):
         """x: [heads, M, head_dim] fp16, M % 64 == 0.  ws: the caller's ops.Workspace (default: the stream's)."""
@@ -84,15 +116,13 @@ class CompressedPool:
         Tc = M * N // 64
         bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
         idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
-        dst = self.nz_off + self.idx[:, -1] // 4          # 16-byte units; idx counts 4-byte units
+        dst = self.nz_off + self.idx_store[:, self.tiles] // 4          # 16-byte units; idx counts 4-byte units
         ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, M, N), ws)
         fn = L.mstf_append_value_f16 if self.is_value else L.mstf_append_key_f16
         check(fn(torch.cuda.current_stream().cuda_stream, x.data_ptr(), B, M, N, int(kth), bmp_c.data_ptr(),
                  idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(), self.overflow.data_ptr(),
                  ws.data_ptr(), ws.numel()), "mstf_append_f16")
-        self.bmp = torch.cat([self.bmp, bmp_c], dim=1)
-        self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
-        self.tokens += M
+        self._publish(bmp_c, idx_c, M)
 
     def append_proj(self, x, kth, M, cos=None, sin=None, rot=None, ws=None):
         """The first M tokens of x [batch, rows, heads per batch entry, head_dim] (a view of the projection output,
@@ -106,22 +136,20 @@ class CompressedPool:
         Tc = M * N // 64
         bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
         idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
-        dst = self.nz_off + self.idx[:, -1] // 4
+        dst = self.nz_off + self.idx_store[:, self.tiles] // 4
         ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, max(M, 64), N), ws)
         check(L.mstf_append_proj_f16(torch.cuda.current_stream().cuda_stream, ctypes.byref(src), int(self.is_value), M, N,
                                      int(kth), bmp_c.data_ptr(), idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(),
                                      self.nz.data_ptr(), self.overflow.data_ptr(), ws.data_ptr(), ws.numel()),
               "mstf_append_proj_f16")
         if M > 0:
-            self.bmp = torch.cat([self.bmp, bmp_c], dim=1)
-            self.idx = torch.cat([self.idx[:, :-1], idx_c + self.idx[:, -1:]], dim=1).contiguous()
-            self.tokens += M
+            self._publish(bmp_c, idx_c, M)
         return rot
 
     def view(self):
         """The cache as the operators take it (ops.key_spmv / value_spmv / decode_attention)."""
-        return ops.CompressedKV(self.bmp, self.idx, self.nz, self.nz_off, self.tokens, self.head_dim, self.is_value,
-                                None)
+        return ops.CompressedKV(self.bmp.contiguous(), self.idx.contiguous(), self.nz, self.nz_off, self.tokens,
+                                self.head_dim, self.is_value, None)
 
     def head_values(self, b):
         """Packed values of head b (a host read: for tests and debugging)."""
@@ -168,11 +196,21 @@ class SparseKVCache:
             ws = self._workspace(K.device)
             self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
             self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
-            self.k, self.v = self.k_pool.view(), self.v_pool.view()
+            self._pool_views()
             return
         ck, cv = self._compress(K, V)
         self.k = ck if self.k is None else append_compressed(self.k, ck)
         self.v = cv if self.v is None else append_compressed(self.v, cv)
+
+    def _pool_views(self):
+        """After an append to the pools.  With window_kernel the attention reads the pools themselves (nothing moved,
+        nothing to rebuild); the operator-by-operator paths take contiguous per-tile arrays, copied here."""
+        self.k_pool.check_overflow()
+        self.v_pool.check_overflow()
+        if self.window_kernel:
+            self.k, self.v = self.k_pool, self.v_pool
+        else:
+            self.k, self.v = self.k_pool.view(), self.v_pool.view()
 
     def _compress(self, K, V):
         bs, n_kv, L, D = K.shape
@@ -197,7 +235,7 @@ class SparseKVCache:
             self.k_pool.append_proj(kx, self.kth_k, Lc, cos, sin, ws=ws)
             if Lc > 0:
                 self.v_pool.append_proj(vx, self.kth_v, Lc, ws=ws)
-                self.k, self.v = self.k_pool.view(), self.v_pool.view()
+                self._pool_views()
         else:
             ws = self._workspace(kx.device)
             ck, _ = ops.compress_proj(kx, False, self.kth_k, Lc, cos, sin, ws=ws)
@@ -221,6 +259,9 @@ class SparseKVCache:
         self.compressed_length, self.kv_len = Lc, L
         if self.window_kernel:
             bs, n_kv, _, D = K.shape
+            if self.max_tokens > 0 and self.k_pool is None:   # nothing compressed yet: the (empty) pools exist from the
+                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, K.device)   # start, so the attention
+                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, K.device)    # call never changes form
             cap = max(self.residual_length + CHUNK, L - Lc)   # the window never holds more before a chunk leaves
             self._kbuf = torch.empty((bs * n_kv, cap, D), dtype=torch.float16, device=K.device)
             self._vbuf = torch.empty_like(self._kbuf)
@@ -254,13 +295,17 @@ class SparseKVCache:
 
     def _attend_device(self, q2):
         """Attention of the query rows q2 [Bq, D] over [compressed | window buffer] (three launches)."""
+        if self.k_pool is not None:
+            return ops.decode_attention_window_pool(self.k_pool, self.v_pool, q2, self._kbuf, self._vbuf,
+                                                    self._kbuf.shape[1], self.groups, self._wlen_dev,
+                                                    ws=self._workspace(q2.device))
         return ops.decode_attention_window(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1], self.groups,
                                            win_len_dev=self._wlen_dev, ws=self._workspace(q2.device))
 
     def advance(self):
         """Host-side bookkeeping after decode_device (or a replay of it): counts the token and, when the window holds
-        residual_length + 256 tokens, compresses its oldest 256.  Returns True when the compressed part grew (its
-        arrays moved: a captured graph must be captured again)."""
+        residual_length + 256 tokens, compresses its oldest 256.  Returns True when arrays of the compressed part moved
+        (a captured graph must then be captured again): never with pools (max_tokens > 0), which grow in place."""
         bs, n_kv, D = self._shape
         self.kv_len += 1
         self._wlen += 1
@@ -274,7 +319,7 @@ class SparseKVCache:
             self._widx.fill_(rest)
             self._wlen_dev.fill_(rest)
             self.compressed_length += CHUNK
-            grew = True
+            grew = self.k_pool is None
         self._window_views()
         return grew
 

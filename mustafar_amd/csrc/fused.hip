@@ -31,10 +31,18 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
-    _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int Lc, int groups, int nblk,
-    int nsplit, int write_final, float sqrt_d, int bpw)
+    _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, size_t tstride, int groups,
+    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev)
 {
+    // tstride: tiles between the bitmap rows of two heads (offsets: one more), which is the tile count of the cached
+    // tokens unless the cache is pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read
+    // from device memory, at most nblk blocks of it; the launch is then sized for the capacity and the wavefronts
+    // beyond the valid blocks leave neutral partials, so a recorded launch stays valid while the cache grows.
     constexpr int D = kFusedD;
+    if (tokens_dev) {
+        const int valid = *tokens_dev / 64;
+        nblk = valid < nblk ? valid : nblk;
+    }
     constexpr int kQLds = NM * 4 * D * 2;          // query rows [4*NM][D] fp16
     constexpr int kPRow = 64 * 2;                  // one row of block weights: 64 tokens fp16
     constexpr int kPLds = NM * 4 * kPRow;
@@ -53,7 +61,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     if (MULTI) nb = nb > bpw ? bpw : nb;
     const bool active = nb > 0;
     const int j = lane & 3;
-    const size_t T = (size_t)Lc * D / 64;
+    const size_t T = tstride;
     char* my = lds[wave];
     char* ql = my + kNzLds;
     char* pl = ql + kQLds;
@@ -516,8 +524,10 @@ static int decode_check(const void* k_bmp, const void* k_nz, const void* k_idx, 
 static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
                          const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
                          const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
-                         int groups, void* workspace, int write_final, int nsplit_total = 0)
+                         int groups, void* workspace, int write_final, int nsplit_total = 0, size_t tile_stride = 0,
+                         const int32_t* tokens_dev = nullptr)
 {
+    const size_t tstride = tile_stride ? tile_stride : (size_t)tokens * head_dim / 64;
     const int Bkv = Bq / groups, nblk = tokens / 64;
     const int bpw = fused_blocks_per_wave(tokens, Bkv), ns = fused_nsplit(tokens, bpw);
     const int nst = nsplit_total > 0 ? nsplit_total : ns;
@@ -531,8 +541,8 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     const float sq = sqrtf((float)head_dim);
 #define MSTF_FD(NMV, MULTIV)                                                                                         \
     hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, \
-                       k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tokens, groups, nblk, nst,     \
-                       write_final, sq, bpw)
+                       k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,    \
+                       write_final, sq, bpw, tokens_dev)
     if (groups <= 4) {
         if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
     } else {
@@ -728,6 +738,39 @@ extern "C" int mstf_decode_attention_window_f16(void* stream, const uint64_t* k_
                            tokens, head_dim, Bq, groups, workspace, 0, nst);
         if (rc != MSTF_OK) return rc;
     }
+    if ((rc = window_launch(as_stream(stream), k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq,
+                            groups, nst, ns)) != MSTF_OK)
+        return rc;
+    return merge_splits(as_stream(stream), workspace, out, lse_out, nst, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz,
+                                                     const uint32_t* k_idx, const uint32_t* k_nz_off,
+                                                     const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
+                                                     const uint32_t* v_nz_off, const mstf_half* q, const mstf_half* k_win,
+                                                     const mstf_half* v_win, int win_len, const int32_t* win_len_dev,
+                                                     int win_stride, mstf_half* out, float* lse_out, int max_tokens,
+                                                     const int32_t* tokens_dev, int64_t tile_capacity, int head_dim,
+                                                     int Bq, int groups, void* workspace, size_t workspace_bytes)
+{
+    if (!q || !k_win || !v_win || !out || !tokens_dev) return MSTF_EINVAL;
+    if (max_tokens <= 0 || win_len <= 0 || win_stride < win_len || Bq <= 0 || groups <= 0 || Bq % groups != 0)
+        return MSTF_EINVAL;
+    if (head_dim != kFusedD || max_tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (tile_capacity < (int64_t)max_tokens * head_dim / 64) return MSTF_EINVAL;
+    if (!aligned_to(q, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)) || !aligned_to(tokens_dev, 4))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    const int ns = splits_of(max_tokens, Bq, groups), nst = ns + window_blocks(win_len);
+    int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, max_tokens, head_dim, Bq, groups,
+                          workspace, workspace_bytes);
+    if (rc != MSTF_OK) return rc;
+    rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, nullptr, max_tokens,
+                       head_dim, Bq, groups, workspace, 0, nst, (size_t)tile_capacity, tokens_dev);
+    if (rc != MSTF_OK) return rc;
     if ((rc = window_launch(as_stream(stream), k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq,
                             groups, nst, ns)) != MSTF_OK)
         return rc;

@@ -222,9 +222,10 @@ class GraphedGreedyLoop:
     """Greedy decoding with the whole step - embedding to argmax - replayed from a HIP graph.
 
     Everything that changes from step to step lives in device memory and is updated inside the graph: the token
-    ids, the position (RoPE), the window length and write index of every layer's cache.  The host only counts
-    (SparseKVCache.advance) and, every 256 tokens, lets the caches compress a chunk; the compressed arrays move
-    then, so the graph is captured again."""
+    ids, the position (RoPE), the window length, write index and compressed-token count of every layer's cache.  The
+    host only counts (SparseKVCache.advance) and, every 256 tokens, lets the caches compress a chunk between two
+    replays.  Pooled caches (max_tokens > 0) grow in place and the graph stays valid; a cache whose arrays move
+    (the quantised one) reports it and the graph is captured again."""
 
     def __init__(self, dec, first_ids, position):
         self.dec = dec

@@ -267,6 +267,31 @@ def decode_attention_window(ck, cv, q, k_win, v_win, win_len, groups, out=None, 
     return o
 
 
+def decode_attention_window_pool(k_pool, v_pool, q, k_win, v_win, win_len, groups, win_len_dev, out=None, lse=None,
+                                 ws=None):
+    """decode_attention_window over two cache.CompressedPool sides that grow in place: the pools' pre-allocated
+    per-tile arrays are read with their row stride and the number of compressed tokens comes from the pool's device
+    counter, so nothing about the call changes when a chunk is appended (a HIP graph holding it stays valid)."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
+    assert k_pool.max_tokens == v_pool.max_tokens
+    D = k_win.shape[-1]
+    Bq = q.numel() // D
+    L = lib()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    ws = workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(k_pool.max_tokens, int(win_len), D, Bq,
+                                                                           groups), ws)
+    cp = [t.data_ptr() for t in (k_pool.bmp_store, k_pool.nz, k_pool.idx_store, k_pool.nz_off, v_pool.bmp_store, v_pool.nz,
+                                 v_pool.idx_store, v_pool.nz_off)]
+    check(L.mstf_decode_attention_window_pool_f16(_stream(), *cp, q.data_ptr(), k_win.data_ptr(), v_win.data_ptr(),
+                                                  int(win_len), win_len_dev.data_ptr() if win_len_dev is not None else None,
+                                                  k_win.shape[1], o.data_ptr(), lse.data_ptr() if lse is not None else None,
+                                                  k_pool.max_tokens, k_pool.tokens_dev.data_ptr(), k_pool.tile_capacity, D,
+                                                  Bq, groups, ws.data_ptr(), ws.numel()),
+          "mstf_decode_attention_window_pool_f16")
+    return o
+
+
 def decode_attention_partial(ck, cv, q, groups, ws=None):
     """First phase of decode_attention: un-normalised outputs and (max, sum) per 512-token split, left in `ws`."""
     assert q.dtype == torch.float16 and q.is_contiguous()

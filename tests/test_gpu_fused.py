@@ -131,3 +131,33 @@ def test_fused_rejects_bad_arguments():
     assert L.mstf_decode_attention_window_workspace_bytes(4096, 512, 128, 256, 4) == 256 * 16 * 130 * 4
     assert L.mstf_decode_attention_merge_f16(None, a, 1 << 13, None, None, 64, 128, 4, 4) == -1
     assert L.mstf_decode_attention_merge_f16(None, a, 16, a, None, 64, 128, 4, 4) == -4
+
+
+@pytest.mark.parametrize("groups,Bkv,held,capacity,Lw", [(4, 2, 512, 1024, 300), (2, 3, 0, 512, 70), (8, 1, 1024, 1024, 1)])
+def test_pooled_entry_point_reads_a_cache_that_is_allocated_for_more(groups, Bkv, held, capacity, Lw):
+    """mstf_decode_attention_window_pool_f16 (row stride of the per-tile arrays = capacity, token count read from device
+    memory) against mstf_decode_attention_window_f16 on contiguous copies of the same cache: identical bit for bit,
+    with the cache partly filled, empty and full."""
+    from mustafar_amd import ops
+    from mustafar_amd.cache import CompressedPool
+    dev = torch.device("cuda:0")
+    D = 128
+    Bq = Bkv * groups
+    K, V = orc.make_kv(400 + held + Lw, Bkv, max(held, 64) + Lw, D)
+    kp, vp = CompressedPool(Bkv, D, capacity, False, dev), CompressedPool(Bkv, D, capacity, True, dev)
+    Kt, Vt = torch.from_numpy(K).to(dev), torch.from_numpy(V).to(dev)
+    for s in range(0, held, 256):                          # grown chunk by chunk, in place
+        kp.append(Kt[:, s:s + 256], 89)
+        vp.append(Vt[:, s:s + 256], 89)
+    assert kp.tokens == held and int(kp.tokens_dev) == held
+    q = torch.from_numpy(np.random.default_rng(Lw).standard_normal((Bq, D)).astype(np.float16)).to(dev)
+    cap = Lw + 5
+    kw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev)
+    vw = torch.full((Bkv, cap, D), float("nan"), dtype=torch.float16, device=dev)
+    kw[:, :Lw] = Kt[:, max(held, 64):max(held, 64) + Lw]
+    vw[:, :Lw] = Vt[:, max(held, 64):max(held, 64) + Lw]
+    wl = torch.tensor([Lw], dtype=torch.int32, device=dev)
+    got = ops.decode_attention_window_pool(kp, vp, q, kw, vw, cap, groups, wl)
+    want = ops.decode_attention_window(kp.view() if held else None, vp.view() if held else None, q, kw, vw, cap, groups,
+                                       win_len_dev=wl)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
