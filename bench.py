@@ -8,7 +8,11 @@ the fused kernel plus its split merge (or, with --unfused, as the three separate
 of the reference's call sequence).  Several distinct caches are rotated between steps so that
 reads come from HBM, not from the 256 MB Infinity Cache.  Prints exactly one JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu] [--unfused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu] [--unfused] [--no-configs]
+
+Beside the headline the line carries `configs`: the other benchmark configurations measured in the same run
+(configs[1] at 50 %, configs[2] compressors at batch 16, configs[3] quantised decode at batch 32, a short configs[4]
+decode loop); every kernel time in the line is the GPU time of launches replayed from HIP graphs on rotating caches.
 """
 import argparse
 import json
@@ -89,6 +93,209 @@ def cpu_baseline(args, bs, nkv, groups, L, D, kth):
     }
 
 
+def ring_time_us(torch, fn, n_slots, reps):
+    """GPU time of one fn(i): fn(0) .. fn(n_slots - 1) are captured back to back into one HIP graph (slot i works on
+    rotating cache i, so its reads are cold), the graph is replayed `reps` times between two HIP events."""
+    for i in range(n_slots):
+        fn(i)   # warm-up outside the capture (module load, workspace growth)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(n_slots):
+            fn(i)
+    g.replay()
+    return event_time_us(torch, g.replay, max(1, reps)) / n_slots
+
+
+def read_calibration(torch):
+    """Plain reads (mstf_probe_read: 16 bytes per lane, nothing else) of cold buffers: per size the average launch time
+    over rotating copies (at least 1 GiB apart in total, so that nothing is served from the last-level cache)."""
+    from mustafar_amd._lib import lib, check
+    L = lib()
+    dev = torch.device("cuda:0")
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+    out = {"what": "plain read of a cold buffer, 16 bytes per lane, 256 threads per workgroup; HIP-graph replays of one "
+                   "launch per rotating copy", "sizes": []}
+    for mb, wgs in ((31, 4096), (62, 4096), (62, 2048), (134, 4096), (249, 4096), (512, 8192), (1024, 8192)):
+        nbytes = mb << 20
+        copies = max(2, min(8, (1536 << 20) // nbytes))
+        bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(copies)]
+
+        def run(i):
+            check(L.mstf_probe_read(torch.cuda.current_stream().cuda_stream, bufs[i].data_ptr(), nbytes, sink.data_ptr(), wgs),
+                  "mstf_probe_read")
+        us = ring_time_us(torch, run, copies, 20)
+        out["sizes"].append({"MiB": mb, "workgroups": wgs, "copies": copies, "us": round(us, 2),
+                             "gbs": round(nbytes / us / 1e3, 1), "frac_of_8TBs": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+        del bufs
+        torch.cuda.empty_cache()
+    return out
+
+
+def compressed_bytes(c):
+    return c.bmp.numel() * 8 + c.idx.numel() * 4 + int(c.total_halfs.item()) * 2
+
+
+def build_caches(torch, ops, dev, gen, Bkv, L, D, kth, n, keep_dense=False):
+    caches, dense = [], []
+    for _ in range(n):
+        K, V = make_kv(torch, dev, Bkv, L, D, gen)
+        caches.append((ops.compress(K, False, kth=kth, capacity_halfs=K.numel()),
+                       ops.compress(V, True, kth=kth, capacity_halfs=V.numel())))
+        if keep_dense:
+            dense.append((K, V))
+        del K, V
+    return caches, dense
+
+
+def fp16_decode_record(torch, ops, dev, gen, bs, L, sparsity, n_caches, reps):
+    """Fused step (kernel + merge), the fused kernel alone and the three-launch stages at batch `bs`."""
+    nq, nkv, D = 32, 8, 128
+    g, Bkv, Bq = nq // nkv, bs * nkv, bs * nq
+    kth = ops.kth_from_sparsity(sparsity, D)
+    caches, _ = build_caches(torch, ops, dev, gen, Bkv, L, D, kth, n_caches)
+    kb, vb = compressed_bytes(caches[0][0]), compressed_bytes(caches[0][1])
+    q = torch.randn((Bq, D), generator=gen, device=dev, dtype=torch.float32).half()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=dev)
+    s = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
+    p = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
+    ws = ops.Workspace(dev)
+    step = ring_time_us(torch, lambda i: ops.decode_attention(caches[i][0], caches[i][1], q, g, out=o, ws=ws), n_caches, reps)
+    kern = ring_time_us(torch, lambda i: ops.decode_attention_partial(caches[i][0], caches[i][1], q, g, ws=ws), n_caches, reps)
+    key = ring_time_us(torch, lambda i: ops.key_spmv(caches[i][0], q.view(Bq, 1, D), g, out=s), n_caches, reps)
+    sm = ring_time_us(torch, lambda i: ops.scale_softmax(s, D, out=p), n_caches, reps)
+    val = ring_time_us(torch, lambda i: ops.value_spmv(caches[i][1], p, g, out=o.view(Bq, 1, D), ws=ws), n_caches, reps)
+    alg = kb + vb + 2 * Bq * D * 2
+    return {"batch": bs, "ctx": L, "sparsity": sparsity, "step_us": round(step, 2), "fused_kernel_us": round(kern, 2),
+            "fused_kernel_gbs": round(alg / kern / 1e3, 1), "fused_kernel_frac_of_peak": round(alg / kern / 1e3 / HBM_PEAK_GBS, 4),
+            "key_spmv_us": round(key, 2), "scale_softmax_us": round(sm, 2), "value_spmv_us": round(val, 2),
+            "algorithmic_bytes": int(alg), "tokens_per_s": round(bs / (step * 1e-6), 1)}
+
+
+def compress_record(torch, ops, dev, gen, bs, L, sparsity, reps):
+    """configs[2]: prune + compress of the whole context, keys and values, three launches each from a replayed graph."""
+    nkv, D = 8, 128
+    Bkv = bs * nkv
+    kth = ops.kth_from_sparsity(sparsity, D)
+    K, V = make_kv(torch, dev, Bkv, L, D, gen)
+    ws = ops.Workspace(dev)
+    out = {"batch": bs, "ctx": L, "sparsity": sparsity}
+    for name, x, is_value in (("key", K, False), ("value", V, True)):
+        keep = []
+
+        def run(i):
+            keep[:] = [ops.compress(x, is_value, kth=kth, capacity_halfs=x.numel(), ws=ws)]
+        us = ring_time_us(torch, run, 1, reps)
+        written = compressed_bytes(keep[0])
+        read = x.numel() * 2
+        out[name] = {"us": round(us, 1), "read_bytes": int(read), "written_bytes": int(written),
+                     "gbs": round((read + written) / us / 1e3, 1),
+                     "frac_of_peak": round((read + written) / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return out
+
+
+def quant_record(torch, ops, dev, gen, bs, L, sparsity, bit, group_size, reps):
+    """configs[3]: decode over the quantised cache - key SpMV, value SpMV (one row per head) and the fused launch."""
+    from mustafar_amd import compression_quant as cq
+    from mustafar_amd import mustafar_package_quant as mpq
+    from mustafar_amd._lib import lib, check
+    nq, nkv, D = 32, 8, 128
+    g, Bkv, Bq = nq // nkv, bs * nkv, bs * nq
+    kth = ops.kth_from_sparsity(sparsity, D)
+    Lh = lib()
+    n_caches = 2
+    sides = []
+    for _ in range(n_caches):
+        K, V = make_kv(torch, dev, Bkv, L, D, gen)
+        Kp = ops.prune_rows(K.view(-1, D), kth).view(Bkv, L, D)
+        Vp = ops.prune_rows(V.view(-1, D), kth).view(Bkv, L, D)
+        sides.append((cq.convert_key_batched_quant(Kp, return_metadata=True, bit=bit, group_size=group_size),
+                      cq.convert_value_batched_quant(Vp, bit=bit, group_size=group_size)))
+        del K, V, Kp, Vp
+    q = torch.randn((Bq, D), generator=gen, device=dev, dtype=torch.float32).half()
+    p1 = torch.softmax(torch.randn((Bq, L), generator=gen, device=dev), -1).half()
+    s1 = torch.empty((Bq, L), dtype=torch.float16, device=dev)
+    o = torch.empty((Bq, D), dtype=torch.float16, device=dev)
+    ws = ops.Workspace(dev)
+    wsv = ws.get(Lh.mstf_value_spmv_quant_workspace_bytes(D, L, Bq, g, 1))
+    def qkey(i):
+        st = torch.cuda.current_stream().cuda_stream   # the capturing stream while a graph is recorded
+        kq = sides[i][0]
+        check(Lh.mstf_key_spmv_quant_grouped(st, kq[0].data_ptr(), kq[2].data_ptr(), kq[1].data_ptr(), kq[5].data_ptr(),
+                                             kq[6].data_ptr(), q.data_ptr(), s1.data_ptr(), L, D, Bq, g, 1, bit, 32 // bit,
+                                             0, group_size), "mstf_key_spmv_quant_grouped")
+
+    def qval(i):
+        st = torch.cuda.current_stream().cuda_stream
+        vq = sides[i][1]
+        check(Lh.mstf_value_spmv_quant_grouped(st, vq[0].data_ptr(), vq[2].data_ptr(), vq[1].data_ptr(), vq[5].data_ptr(),
+                                               vq[6].data_ptr(), p1.data_ptr(), o.data_ptr(), D, L, Bq, g, 1, bit,
+                                               32 // bit, 0, group_size, wsv.data_ptr(), wsv.numel()),
+              "mstf_value_spmv_quant_grouped")
+
+    def side_bytes(t):
+        return sum(x.numel() * x.element_size() for x in (t[0], t[1], t[2], t[5], t[6]))
+    kb, vb = side_bytes(sides[0][0]), side_bytes(sides[0][1])
+    key = ring_time_us(torch, qkey, n_caches, reps)
+    val = ring_time_us(torch, qval, n_caches, reps)
+    fused = ring_time_us(torch, lambda i: mpq.decode_attention_quant(sides[i][0], sides[i][1], q, g, bit, out=o, ws=ws),
+                         n_caches, reps)
+    alg = kb + vb + 2 * Bq * D * 2
+    return {"batch": bs, "ctx": L, "sparsity": sparsity, "bit": bit, "group_size": group_size,
+            "key_spmv_us": round(key, 2), "value_spmv_us": round(val, 2), "fused_step_us": round(fused, 2),
+            "key_spmv_gbs": round((kb + Bq * D * 2 + Bq * L * 2) / key / 1e3, 1),
+            "value_spmv_gbs": round((vb + Bq * D * 2 + Bq * L * 2) / val / 1e3, 1),
+            "fused_step_gbs": round(alg / fused / 1e3, 1), "fused_step_frac_of_peak": round(alg / fused / 1e3 / HBM_PEAK_GBS, 4),
+            "bytes_per_token_per_kv_head": {"key": round(kb / Bkv / L, 2), "value": round(vb / Bkv / L, 2)}}
+
+
+def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens):
+    """configs[4], shortened: random-init Llama-3-8B shape, greedy decoding with the step replayed from a HIP graph
+    (tokens/s) and a few eager steps with events around the cache's attention (its share of the step)."""
+    import time as _time
+    from mustafar_amd.cache import CHUNK
+    from mustafar_amd.harness import Config, Decoder, GraphedGreedyLoop
+    cfg = Config(layers=layers)
+    max_tokens = ((prompt + new_tokens + 16 + CHUNK - 1) // CHUNK) * CHUNK
+    dec = Decoder(cfg, dev, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=max_tokens)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    ids = torch.randint(0, cfg.vocab, (batch, prompt), generator=g, device=dev)
+    dec.prefill(ids)                 # untimed: library start-up and kernel selection
+    dec.reset_caches()
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    logits = dec.prefill(ids)
+    torch.cuda.synchronize()
+    t_prefill = _time.perf_counter() - t0
+    nxt = logits[:, -1].argmax(-1, keepdim=True)
+    eager_steps = 6
+    for t in range(2):
+        nxt = dec.step(nxt, prompt + t)[:, -1].argmax(-1, keepdim=True)
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    for t in range(2, 2 + eager_steps):
+        nxt = dec.step(nxt, prompt + t, timed=True)[:, -1].argmax(-1, keepdim=True)
+    torch.cuda.synchronize()
+    t_eager = (_time.perf_counter() - t0) / eager_steps
+    attn_ms = sum(a.elapsed_time(b) for a, b in dec.attn_events) / eager_steps
+    loop = GraphedGreedyLoop(dec, nxt, prompt + 2 + eager_steps)
+    for _ in range(4):
+        loop.step()
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    for _ in range(new_tokens):
+        loop.step()
+    torch.cuda.synchronize()
+    t_step = (_time.perf_counter() - t0) / new_tokens
+    return {"layers": layers, "batch": batch, "prompt": prompt, "new_tokens_timed": new_tokens, "prefill_s": round(t_prefill, 3),
+            "graphed_decode_ms_per_step": round(1e3 * t_step, 3), "tokens_per_s": round(batch / t_step, 1),
+            "graph_captures": loop.captures, "eager_decode_ms_per_step": round(1e3 * t_eager, 3),
+            "eager_attention_over_cache_ms_per_step": round(attn_ms, 3),
+            "eager_attention_share": round(attn_ms / (1e3 * t_eager), 4),
+            "compressed_tokens_at_end": dec.caches[0].compressed_length}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,8 +309,13 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying HIP graphs")
     ap.add_argument("--unfused", action="store_true", help="step = the three separate operator launches")
-    ap.add_argument("--no-quant", action="store_true", help="skip the stage timings of the quantised format")
+    ap.add_argument("--no-quant", action="store_true", help="skip the quantised format at the headline shape")
     ap.add_argument("--no-dense", action="store_true", help="skip the dense fp16 attention timed beside the sparse path")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other benchmark configurations (configs sub-records)")
+    ap.add_argument("--loop-layers", type=int, default=32, help="layers of the configs[4] decode loop (0 = skip it)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="instead of the benchmark: time plain 16-byte-per-lane reads of buffers of the sizes the "
+                         "kernels stream (one JSON line), the practical floor their times are read against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one GPU "
@@ -117,46 +329,20 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if args.calibrate:
+        print(json.dumps(read_calibration(torch)))
+        return
     bs, nq, nkv, D, L = args.batch, 32, 8, 128, args.ctx
     groups = nq // nkv
     Bkv, Bq = bs * nkv, bs * nq
     kth = ops.kth_from_sparsity(args.sparsity, D)
     gen = torch.Generator(device=dev)
     gen.manual_seed(20260312)
+    reps = max(5, args.steps // args.caches)
 
-    # ---- build the rotating compressed caches (also times the fused prune+compress kernels)
-    caches = []
-    dense = []   # the same tokens uncompressed, for the dense fp16 attention timed beside the sparse path
-    t_ck = t_cv = 0.0
-    for i in range(args.caches):
-        K, V = make_kv(torch, dev, Bkv, L, D, gen)
-        cap = K.numel()
-        if i == 0:
-            ops.compress(K, False, kth=kth, capacity_halfs=cap)  # warm-up (module load)
-        t_ck += event_time_us(torch, lambda: caches.append([ops.compress(K, False, kth=kth, capacity_halfs=cap)]), 1)
-        t_cv += event_time_us(torch, lambda: caches[-1].append(ops.compress(V, True, kth=kth, capacity_halfs=cap)), 1)
-        if i == args.caches - 1:
-            # GPU time of the compressors without the launch gaps of the Python calls: one capture, replayed
-            try:
-                def graphed_us(x, is_value):
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g):
-                        keep = ops.compress(x, is_value, kth=kth, capacity_halfs=cap)
-                    g.replay()
-                    t = event_time_us(torch, g.replay, 5)
-                    del keep
-                    return t
-                tg_ck, tg_cv = graphed_us(K, False), graphed_us(V, True)
-            except Exception as e:  # pragma: no cover - reported as null in the JSON line
-                print("compress graph capture failed (%s)" % e, file=sys.stderr)
-                tg_ck = tg_cv = None
-        if not args.no_dense:
-            dense.append((K.view(bs, nkv, L, D), V.view(bs, nkv, L, D)))
-        del K, V
-    t_ck /= args.caches
-    t_cv /= args.caches
-    kbytes = caches[0][0].bmp.numel() * 8 + caches[0][0].idx.numel() * 4 + int(caches[0][0].total_halfs.item()) * 2
-    vbytes = caches[0][1].bmp.numel() * 8 + caches[0][1].idx.numel() * 4 + int(caches[0][1].total_halfs.item()) * 2
+    # ---- the rotating compressed caches of the headline workload
+    caches, dense = build_caches(torch, ops, dev, gen, Bkv, L, D, kth, args.caches, keep_dense=not args.no_dense)
+    kbytes, vbytes = compressed_bytes(caches[0][0]), compressed_bytes(caches[0][1])
 
     q = torch.randn((Bq, 1, D), generator=gen, device=dev, dtype=torch.float32).half()
     q2 = q.view(Bq, D)
@@ -164,6 +350,7 @@ def main():
     p = torch.empty((Bq, 1, L), dtype=torch.float16, device=dev)
     o = torch.empty((Bq, 1, D), dtype=torch.float16, device=dev)
     o2 = o.view(Bq, D)
+    ws = ops.Workspace(dev)
     it = [0]
 
     def launch(i):
@@ -171,9 +358,9 @@ def main():
         if args.unfused:
             ops.key_spmv(ck, q, groups, out=s)
             ops.scale_softmax(s, D, out=p)
-            ops.value_spmv(cv, p, groups, out=o)
+            ops.value_spmv(cv, p, groups, out=o, ws=ws)
         else:
-            ops.decode_attention(ck, cv, q2, groups, out=o2)
+            ops.decode_attention(ck, cv, q2, groups, out=o2, ws=ws)
 
     # The launches are captured once and replayed, so that the timed region measures the GPU work of a step
     # rather than the Python call overhead of its launches: one graph holds one step on each of the rotating
@@ -226,41 +413,32 @@ def main():
 
     # the same step on ONE cache over and over: its compressed bytes stay in the last-level cache between steps.
     # Reported beside `value` (which rotates the caches so that every step reads from HBM), never instead of it.
-    warm_us = None
-    if graphs is not None:
-        warm_ring = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(warm_ring):
-            for _ in range(args.caches):
-                launch(0)
-        reps = max(1, args.steps // args.caches)
-        for _ in range(3):
-            warm_ring.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            warm_ring.replay()
-        torch.cuda.synchronize()
-        warm_us = (time.perf_counter() - t0) * 1e6 / (reps * args.caches)
+    warm_us = ring_time_us(torch, lambda i: launch(0), args.caches, reps)
 
-    # ---- per-kernel averages over back-to-back launches on rotating caches (HIP events on the launch stream)
-    def rot(j):
-        c = caches[it[0] % args.caches][j]
-        it[0] += 1
-        return c
+    # ---- per-kernel GPU times, every one from launches replayed out of a HIP graph on the rotating caches
+    fused_us = ring_time_us(torch, lambda i: ops.decode_attention_partial(caches[i][0], caches[i][1], q2, groups, ws=ws),
+                            args.caches, reps)
+    wsm = ops.decode_attention_partial(caches[0][0], caches[0][1], q2, groups, ws=ws)
+    merge_us = ring_time_us(torch, lambda i: ops.decode_attention_merge(wsm, L, D, Bq, groups, out=o2), args.caches, reps)
+    key_us = ring_time_us(torch, lambda i: ops.key_spmv(caches[i][0], q, groups, out=s), args.caches, reps)
+    val_us = ring_time_us(torch, lambda i: ops.value_spmv(caches[i][1], p, groups, out=o, ws=ws), args.caches, reps)
+    sm_us = ring_time_us(torch, lambda i: ops.scale_softmax(s, D, out=p), args.caches, reps)
 
-    def fused_only():
-        i = it[0] % args.caches
-        it[0] += 1
-        ops.decode_attention_partial(caches[i][0], caches[i][1], q2, groups)
+    # the compressors at the headline shape: prune + compress of the whole context, three launches per side
+    comp = {}
+    Kc, Vc = make_kv(torch, dev, Bkv, L, D, gen)
+    for name, is_value in (("key", False), ("value", True)):
+        x = Vc if is_value else Kc
+        held = []
 
-    n = max(args.steps, 50)
-    launch(0)
-    fused_us = event_time_us(torch, fused_only, n)
-    ws = ops.decode_attention_partial(caches[0][0], caches[0][1], q2, groups)
-    merge_us = event_time_us(torch, lambda: ops.decode_attention_merge(ws, L, D, Bq, groups, out=o2), n)
-    key_us = event_time_us(torch, lambda: ops.key_spmv(rot(0), q, groups, out=s), n)
-    val_us = event_time_us(torch, lambda: ops.value_spmv(rot(1), p, groups, out=o), n)
-    sm_us = event_time_us(torch, lambda: ops.scale_softmax(s, D, out=p), n)
+        def run_c(i):
+            held[:] = [ops.compress(x, is_value, kth=kth, capacity_halfs=x.numel(), ws=ws)]
+        us = ring_time_us(torch, run_c, 1, 5)
+        wr = compressed_bytes(held[0])
+        comp[name] = {"us": round(us, 1), "read_bytes": int(x.numel() * 2), "written_bytes": int(wr),
+                      "gbs": round((x.numel() * 2 + wr) / us / 1e3, 1)}
+        del held
+    del Kc, Vc
 
     # dense fp16 decode attention over the same (unpruned) tokens with library operators, cold caches rotated alike:
     # what the sparse path has to beat.  "matmul" batches the query heads of a KV head into one product, so K and V
@@ -273,71 +451,44 @@ def main():
 
         def dense_matmul(i):
             Kd, Vd = dense[i]
-            w = torch.matmul(q5, Kd.transpose(2, 3)) / math.sqrt(D)
-            return torch.matmul(torch.softmax(w, -1, dtype=torch.float32).half(), Vd)
+            w = torch.matmul(q5, Kd.view(bs, nkv, L, D).transpose(2, 3)) / math.sqrt(D)
+            return torch.matmul(torch.softmax(w, -1, dtype=torch.float32).half(), Vd.view(bs, nkv, L, D))
 
         def dense_sdpa(i):
             Kd, Vd = dense[i]
-            return F.scaled_dot_product_attention(q4, Kd, Vd, enable_gqa=True)
+            return F.scaled_dot_product_attention(q4, Kd.view(bs, nkv, L, D), Vd.view(bs, nkv, L, D), enable_gqa=True)
 
-        def ring_time_us(fn):
-            """One step on each rotating cache captured into one HIP graph (as the sparse step is), replayed."""
-            for i in range(args.caches):
-                fn(i)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for i in range(args.caches):
-                    fn(i)
-            g.replay()
-            reps = max(n // args.caches, 5)
-            return event_time_us(torch, g.replay, reps) / args.caches
+        dense_us = {"matmul_softmax_matmul": round(ring_time_us(torch, dense_matmul, args.caches, reps), 2),
+                    "sdpa": round(ring_time_us(torch, dense_sdpa, args.caches, reps), 2), "bytes": int(2 * Bkv * L * D * 2)}
+    del dense
 
-        dense_us = {"matmul_softmax_matmul": round(ring_time_us(dense_matmul), 2),
-                    "sdpa": round(ring_time_us(dense_sdpa), 2), "bytes": int(2 * Bkv * L * D * 2)}
-
-    # quantised format (2- and 4-bit codes) on the same shape: producer once, then the key / value SpMVs with one
-    # row per query head through the C ABI
-    quant_us = {}
+    quant_here = {}
     if not args.no_quant:
-        from mustafar_amd import compression_quant as cq
-        from mustafar_amd._lib import lib, check
-        Lh = lib()
-        Kd, Vd = make_kv(torch, dev, Bkv, L, D, gen)
-        Kd, Vd = ops.prune_rows(Kd.view(-1, D), kth).view(Bkv, L, D), ops.prune_rows(Vd.view(-1, D), kth).view(Bkv, L, D)
-        p1 = torch.softmax(torch.randn((Bq, L), generator=gen, device=dev), -1).half()
-        s1 = torch.empty((Bq, L), dtype=torch.float16, device=dev)
         for bit in (2, 4):
-            kq = cq.convert_key_batched_quant(Kd, return_metadata=True, bit=bit)
-            vq = cq.convert_value_batched_quant(Vd, bit=bit)
-            st = torch.cuda.current_stream().cuda_stream
-            wsq = ops.workspace(dev, Lh.mstf_value_spmv_quant_workspace_bytes(D, L, Bq, groups, 1))
+            r = quant_record(torch, ops, dev, gen, bs, L, args.sparsity, bit, 64, 10)
+            quant_here["%dbit" % bit] = {k: r[k] for k in ("key_spmv_us", "value_spmv_us", "fused_step_us",
+                                                           "fused_step_gbs", "bytes_per_token_per_kv_head")}
 
-            def qkey():
-                check(Lh.mstf_key_spmv_quant(st, kq[0].data_ptr(), kq[2].data_ptr(), kq[1].data_ptr(), None, None,
-                                             kq[5].data_ptr(), kq[6].data_ptr(), q2.data_ptr(), s1.data_ptr(), L, D, Bq,
-                                             groups, 1, bit, 32 // bit, 0), "mstf_key_spmv_quant")
-
-            def qval():
-                check(Lh.mstf_value_spmv_quant(st, vq[0].data_ptr(), vq[2].data_ptr(), vq[1].data_ptr(), None, None,
-                                               vq[5].data_ptr(), vq[6].data_ptr(), p1.data_ptr(), o2.data_ptr(), D, L, Bq,
-                                               groups, 1, bit, 32 // bit, 0, wsq.data_ptr(), wsq.numel()),
-                      "mstf_value_spmv_quant")
-
-            from mustafar_amd import mustafar_package_quant as mpq
-
-            def qfused():
-                mpq.decode_attention_quant(kq, vq, q2, groups, bit, out=o2)
-
-            qkey(), qval(), qfused()
-            nbytes = lambda t: sum(x.numel() * x.element_size() for x in (t[0], t[1], t[2], t[5], t[6]))
-            quant_us["%dbit" % bit] = {"key_spmv": round(event_time_us(torch, qkey, 30), 2),
-                                       "value_spmv": round(event_time_us(torch, qval, 30), 2),
-                                       "fused_decode_attention_incl_merge": round(event_time_us(torch, qfused, 30), 2),
-                                       "bytes_per_token_per_kv_head": {"key": round(nbytes(kq) / Bkv / L, 2),
-                                                                       "value": round(nbytes(vq) / Bkv / L, 2)}}
-            del kq, vq
-        del Kd, Vd
+    # ---- the other benchmark configurations, in the same run (skipped for a non-default workload)
+    configs = None
+    default_workload = (args.batch, args.ctx, args.sparsity, args.unfused) == (8, 4096, 0.7, False)
+    if not args.no_configs and default_workload:
+        del caches
+        torch.cuda.empty_cache()
+        configs = {"configs1_bs8_sparsity50": fp16_decode_record(torch, ops, dev, gen, 8, 4096, 0.5, 6, 20)}
+        configs["configs2_compress_bs16"] = [compress_record(torch, ops, dev, gen, 16, 4096, sp, 5) for sp in (0.5, 0.7, 0.9)]
+        torch.cuda.empty_cache()
+        configs["configs3_fp16_bs32_for_comparison"] = fp16_decode_record(torch, ops, dev, gen, 32, 4096, 0.7, 3, 20)
+        torch.cuda.empty_cache()
+        configs["configs3_quant_bs32"] = [quant_record(torch, ops, dev, gen, 32, 4096, 0.7, bit, gs, 10)
+                                          for bit, gs in ((2, 64), (4, 64), (2, 32), (4, 32))]
+        torch.cuda.empty_cache()
+        if args.loop_layers > 0:
+            try:
+                configs["configs4_decode_loop"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 32)
+            except Exception as e:  # pragma: no cover - e.g. out of memory on a shared box; reported, not fatal
+                configs["configs4_decode_loop"] = {"error": str(e)[:200]}
+        torch.cuda.empty_cache()
 
     # a copy of known size, so that a counter run of this same command can be calibrated (outside every timed region)
     cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
@@ -385,20 +536,13 @@ def main():
                                                        "value": round(vbytes / Bkv / L, 2)},
         },
         "tokens_per_s": round(bs / (wall_us * 1e-6), 1),
-        "warm_cache_us_per_layer": None if warm_us is None else round(warm_us, 2),
+        "warm_cache_us_per_layer": round(warm_us, 2),
+        # GPU time of each kernel, replayed from HIP graphs on the rotating caches (no Python launch gaps inside)
         "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
-                      "prune_compress_key_ctx": round(t_ck, 1), "prune_compress_value_ctx": round(t_cv, 1)},
-        # the compressors alone (configs[2] reports them): GPU time from a replayed capture, bytes read (dense fp16
-        # context) and written (bitmaps + offsets + packed values), and the resulting rate
-        "compress": {
-            "key": {"us": None if tg_ck is None else round(tg_ck, 1), "read_bytes": int(Bkv * L * D * 2),
-                    "written_bytes": int(kbytes),
-                    "gbs": None if tg_ck is None else round((Bkv * L * D * 2 + kbytes) / tg_ck / 1e3, 1)},
-            "value": {"us": None if tg_cv is None else round(tg_cv, 1), "read_bytes": int(Bkv * L * D * 2),
-                      "written_bytes": int(vbytes),
-                      "gbs": None if tg_cv is None else round((Bkv * L * D * 2 + vbytes) / tg_cv / 1e3, 1)}},
-        "quant_stages_us": quant_us,
+                      "prune_compress_key_ctx": comp["key"]["us"], "prune_compress_value_ctx": comp["value"]["us"]},
+        "compress": comp,
+        "quant_stages_us": quant_here,
         "dense_fp16_attention_us": dense_us,
         "hbm_gbs_on_compressed_bytes": {"fused_decode_attention": round(fused_alg / fused_us / 1e3, 1),
                                         "key_spmv": round(key_alg / key_us / 1e3, 1),
@@ -406,7 +550,10 @@ def main():
                                         "whole_step": round(fused_alg / wall_us / 1e3, 1)},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args),
+                     "traffic_source": "profiles/decode_attention_bs8_ctx4096_s70_traffic.txt (rocprofv3 --pmc runs of this "
+                                       "command, calibrated on the copy this run ends with)",
                      "algorithmic_bytes": int(dom_bytes), "avg_launch_us": round(dom_us, 2)},
+        "configs": configs,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args, bs, nkv, groups, L, D, kth)

@@ -48,6 +48,11 @@ const char* mstf_strerror(int code);
 int mstf_last_hip_error(void);
 /* library version: major*10000 + minor*100 + patch */
 int mstf_version(void);
+/* Measurement aid (no counterpart in the reference): reads `bytes` of device memory with 16-byte loads per lane from
+ * `workgroups` workgroups of 256 threads and does nothing else; sink: at least `workgroups` uint32 (written only in the
+ * practically impossible case that the xor of all data read by a workgroup hits a fixed constant).  Timing it gives the
+ * plain-read time of a buffer of that size on the box at hand. */
+int mstf_probe_read(void* stream, const void* src, size_t bytes, uint32_t* sink, int workgroups);
 
 /* ------------------------------------------------------------------ pruning (A1)
  * Replaces dh_prune_key / dh_prune_value (models/llama_mustafar_kernel.py:194-274):
