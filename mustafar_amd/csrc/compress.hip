@@ -308,6 +308,264 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
     }
 }
 
+// ------------------------------------------------------------------------------- one pass
+// Pruning + compression with a single read of the input, for the calls that produce the packed values: a wavefront
+// owns the unit of its workgroup index, selects, builds bitmaps and padded counts, publishes the unit's total,
+// compacts the first half of the unit into an LDS image while the units in front of it publish theirs, learns where
+// its values start from a decoupled look-back, and streams the two halves out of the rows it still holds in registers.
+//
+// A workgroup of W wavefronts owns W consecutive units (W divides the units of a head), adds up their totals in LDS
+// and publishes one 64-bit word state[g] = bit 63 | total of workgroup g (4-byte units) with an agent-scope store.
+// Its first wavefront then polls the words of the workgroups in front of it - all of them in the packed layout, where
+// a head's values start behind those of all earlier heads; those of its own head in the pooled layout - 64 per round
+// trip, until every word is set, and adds them up; the others wait at the barrier.
+// A workgroup publishes its total before it waits for anything and waits only for workgroups of a lower index, which
+// the dispatcher has started before it: every wait ends.  The waits are bounded all the same (kSpinLimit polls); a
+// workgroup that gives up sets the flag word behind the workgroup words, writes no values, and *total_halfs reads as
+// all ones.  onepass_init_kernel clears the words before the launch.
+constexpr uint32_t kSpinLimit = 1u << 20;
+
+__global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n)
+{
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < n; i += (int)(gridDim.x * 256)) state[i] = 0ull;
+}
+
+__device__ __forceinline__ uint64_t agent_load(const uint64_t* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void agent_store(uint64_t* p, uint64_t v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+constexpr uint64_t kWordReady = 1ull << 63;
+
+// This wavefront's share of the wait for state[first .. g): the windows of 64 words number `wave`, wave + W, ...,
+// four of them in flight at a time.  Returns its part of the sums over [first, split) and [split, g)
+// (first <= split <= g); false when a wait ran out.
+template <int W>
+__device__ __forceinline__ bool wait_for_words(const uint64_t* state, int first, int split, int g, int wave, int lane,
+                                               uint64_t& sum_lo, uint64_t& sum_hi)
+{
+    constexpr int K = 4;
+    uint64_t lo = 0, hi = 0;
+    uint32_t polls = 0;
+    bool ok = true;
+    for (int w0 = first + wave * 64; w0 < g && ok; w0 += 64 * W * K) {
+        uint64_t v[K];
+        bool got[K];
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            v[k] = 0ull;
+            got[k] = w0 + k * 64 * W + lane >= g;
+        }
+        for (;;) {
+            bool all = true;
+#pragma unroll
+            for (int k = 0; k < K; k++)
+                if (!got[k]) v[k] = agent_load(state + w0 + k * 64 * W + lane);
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                got[k] = got[k] || (v[k] >> 63) != 0ull;
+                all = all && got[k];
+            }
+            if (__ballot(!all) == 0ull) break;
+            if (++polls > kSpinLimit) {
+                ok = false;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i = w0 + k * 64 * W + lane;
+            const uint64_t t = v[k] & ~kWordReady;
+            lo += i < split ? t : 0ull;
+            hi += i >= split && i < g ? t : 0ull;
+        }
+    }
+    sum_lo = wave_sum_u64(lo);
+    sum_hi = wave_sum_u64(hi);
+    return ok;
+}
+
+// Compacts half h of a unit into the LDS image at img (tile offsets relative to the half's first tile).
+//   r     : this lane's token, raw fp16 pairs;  kept: its keep words (see select_kth_planes)
+//   key   : tile c = channel 64h + c over the 64 tokens - the lanes that keep the channel write at the tile's running
+//           offset plus their rank among the keepers; the keepers of a channel are the carry of doubling the
+//           bit-reversed keep word (one instruction pops the next channel of all 64 tokens)
+//   value : tile = this lane's token - the lane appends its kept channels at its own tile's offset own4 (4-byte units)
+template <bool IS_VALUE>
+__device__ __forceinline__ void compact_half(const uint32_t (&r)[64], const uint32_t (&kept)[4], int h, uint32_t own4,
+                                             uint32_t bytes, uint32_t img, int lane)
+{
+    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+        *(MSTF_LDS u32x4_t*)(uintptr_t)(img + o) = u32x4_t{0u, 0u, 0u, 0u};  // the padding stays +0.0
+    uint32_t we = __builtin_bitreverse32(kept[2 * h]), wo = __builtin_bitreverse32(kept[2 * h + 1]);
+    const uint64_t all = __builtin_amdgcn_read_exec();  // every statement hands exec back as it found it
+    if (!IS_VALUE) {
+        uint32_t off = img;  // wave-uniform
+        uint32_t t, n;
+        // doubling pops the channel's keep bit of every token into vcc; the keepers then write at the tile's offset
+        // plus twice their rank among the keepers, and the offset moves on by the padded count
+#define MSTF_KEY_CHANNEL(W, STORE)                                                                                   \
+    asm volatile("v_add_co_u32 %[w], vcc, %[w], %[w]\n\t"                                                            \
+                 "s_mov_b64 exec, vcc\n\t"                                                                           \
+                 "v_mbcnt_lo_u32_b32 %[t], exec_lo, 0\n\t"                                                           \
+                 "v_mbcnt_hi_u32_b32 %[t], exec_hi, %[t]\n\t"                                                        \
+                 "v_lshl_add_u32 %[t], %[t], 1, %[off]\n\t" STORE " %[t], %[v]\n\t"                                  \
+                 "s_bcnt1_i32_b64 %[n], exec\n\t"                                                                    \
+                 "s_add_i32 %[n], %[n], 7\n\t"                                                                       \
+                 "s_andn2_b32 %[n], %[n], 7\n\t"                                                                     \
+                 "s_lshl1_add_u32 %[off], %[n], %[off]\n\t"                                                          \
+                 "s_mov_b64 exec, %[all]"                                                                            \
+                 : [w] "+v"(W), [off] "+s"(off), [t] "=&v"(t), [n] "=&s"(n)                                          \
+                 : [v] "v"(r[32 * h + (c >> 1)]), [all] "s"(all)                                                     \
+                 : "vcc", "scc", "memory")
+#pragma unroll
+        for (int c = 0; c < 64; c += 2) {
+            MSTF_KEY_CHANNEL(we, "ds_write_b16");
+            MSTF_KEY_CHANNEL(wo, "ds_write_b16_d16_hi");
+        }
+#undef MSTF_KEY_CHANNEL
+    } else {
+        uint32_t a = img + own4 * 4u;
+#define MSTF_VALUE_CHANNEL(W, STORE)                                                             \
+    asm volatile("v_add_co_u32 %[w], vcc, %[w], %[w]\n\t"                                        \
+                 "s_mov_b64 exec, vcc\n\t" STORE " %[a], %[v]\n\t"                               \
+                 "v_add_u32 %[a], 2, %[a]\n\t"                                                   \
+                 "s_mov_b64 exec, %[all]"                                                        \
+                 : [w] "+v"(W), [a] "+v"(a)                                                      \
+                 : [v] "v"(r[32 * h + (c >> 1)]), [all] "s"(all)                                 \
+                 : "vcc", "memory")
+#pragma unroll
+        for (int c = 0; c < 64; c += 2) {
+            MSTF_VALUE_CHANNEL(we, "ds_write_b16");
+            MSTF_VALUE_CHANNEL(wo, "ds_write_b16_d16_hi");
+        }
+#undef MSTF_VALUE_CHANNEL
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ void stream_image(uint32_t img, uint32_t bytes, char* dst, int lane)
+{
+    for (uint32_t o = (uint32_t)lane * 16u; o < bytes; o += 1024u)
+        *reinterpret_cast<u32x4_t*>(dst + o) = *(MSTF_LDS const u32x4_t*)(uintptr_t)(img + o);
+    __builtin_amdgcn_wave_barrier();
+}
+
+// grid = ceil(units / W) workgroups of W wavefronts, units = B * M/64, W divides M/64.
+//   packed layout  (dst_off == nullptr): heads back to back, nz_off[b] and *total_halfs are written here;
+//   pooled layout  (dst_off given): head b's values start at nz + 16 * dst_off[b] and may not pass
+//                  nz + 16 * dst_limit[b] (else *overflow is set and the unit's values are not written).
+template <bool IS_VALUE, int W>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void compress_onepass_kernel(
+    const _Float16* __restrict__ x, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
+    uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
+    const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
+    uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total)
+{
+    // per wavefront: staging buffer of a half-slab, then image of half a unit's output (at most 64 tiles x 128 bytes)
+    __shared__ __attribute__((aligned(16))) uint32_t bufs[W][kHalfSlabDw];
+    __shared__ uint32_t wave_total[W];
+    __shared__ uint64_t bases[W][3];  // per wavefront: its part of the sum over the earlier heads, of the sum over
+                                      // the head's earlier workgroups, and whether its waits ended
+    static_assert(kHalfSlabDw * 4 >= 64 * 128, "the image fits the staging buffer");
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int nblk = M / 64;
+    const size_t T = (size_t)M * kD / 64;
+    uint64_t* gave_up = state + groups_total;
+    const int g = (int)blockIdx.x;
+    const int u = g * W + wave;  // all W units are of one head and exist: W divides nblk
+    const int b = u / nblk, tb = u - b * nblk;
+    uint32_t* buf = bufs[wave];
+    uint32_t r[64];  // this lane's token, raw fp16 pairs; they stay in registers until they are compacted
+    unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, buf, lane, r);
+    uint32_t kept[4];
+    if (kth > 0)
+        select_kth_planes<true>(r, kth, kept);  // the sign bits become planes the search never looks at
+    else
+        kept_nonzero(r, kept);
+    uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
+    if (IS_VALUE) {
+        bmA = spread_bitmap(kept[0], kept[1]);
+        bmB = spread_bitmap(kept[2], kept[3]);
+    } else {
+        key_bitmaps_from_kept(kept, lane, bmA, bmB);
+    }
+    uint32_t totA, totB;
+    const uint32_t eA = wave_excl_scan(padded_units(bmA), lane, totA);
+    const uint32_t eB = wave_excl_scan(padded_units(bmB), lane, totB);
+    const uint32_t total = totA + totB;
+    if (lane == 0) wave_total[wave] = total;
+    __syncthreads();
+    uint32_t in_group = 0, group_total = 0;  // units of the workgroup in front of this one / all of them
+#pragma unroll
+    for (int w = 0; w < W; w++) {
+        const uint32_t t = wave_total[w];
+        in_group += w < wave ? t : 0u;
+        group_total += t;
+    }
+    if (threadIdx.x == 0) agent_store(state + g, kWordReady | group_total);
+
+    const uint32_t img = lds_addr(buf);
+    compact_half<IS_VALUE>(r, kept, 0, eA, totA * 4u, img, lane);  // while the workgroups in front publish
+
+    // offset of the unit inside its head and, packed layout, of the head
+    const int head_first = (b * nblk) / W;  // first workgroup of this head
+    {
+        uint64_t lo = 0, hi = 0;
+        const bool ok0 = wait_for_words<W>(state, dst_off ? head_first : 0, head_first, g, wave, lane, lo, hi);
+        if (lane == 0) {
+            bases[wave][0] = lo;
+            bases[wave][1] = hi;
+            bases[wave][2] = ok0 ? 1ull : 0ull;
+        }
+    }
+    __syncthreads();
+    uint64_t H = 0, in_head = 0;
+    bool ok = true;
+#pragma unroll
+    for (int w = 0; w < W; w++) {
+        H += bases[w][0];
+        in_head += bases[w][1];
+        ok = ok && bases[w][2] != 0ull;
+    }
+    if (!ok && threadIdx.x == 0) agent_store(gave_up, 1ull);
+    const uint32_t base = (uint32_t)in_head + in_group;
+    const uint32_t end = base + total;
+
+    uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
+    uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
+    bo[lane] = bmA;
+    bo[64 + lane] = bmB;
+    io[lane] = base + eA;
+    io[64 + lane] = base + totA + eB;
+    if (lane == 0) {
+        if (tb == nblk - 1) io[kD] = end;
+        if (tb == 0 && nz_off) nz_off[b] = (uint32_t)(H >> 2);
+        if (u == units - 1 && total_halfs) *total_halfs = ok ? 2ull * (H + end) : ~0ull;
+    }
+    if (!ok) return;
+    const uint64_t head_half0 = dst_off ? 8ull * dst_off[b] : 2ull * H;
+    if (head_half0 + 2ull * end > nz_capacity_halfs) return;  // would not fit: leave untouched (wave-uniform)
+    if (dst_limit && head_half0 + 2ull * end > 8ull * dst_limit[b]) {
+        if (lane == 0) atomicOr(overflow, 1u);
+        return;
+    }
+    char* dst = nz + (head_half0 + 2ull * base) * 2ull;
+    stream_image(img, totA * 4u, dst, lane);
+    compact_half<IS_VALUE>(r, kept, 1, eB, totB * 4u, img, lane);
+    stream_image(img, totB * 4u, dst + (size_t)totA * 4u, lane);
+}
+
 // ------------------------------------------------------------------------------- dense prune
 // y = x * (|x| >= kth-th smallest |x| of the row); 64 rows per wavefront.
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void prune_rows_kernel(const _Float16* __restrict__ x, _Float16* y, int64_t rows,
@@ -346,10 +604,43 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void pr
 }
 
 // ------------------------------------------------------------------------------- host
-// workspace: unit totals, unit bases (both [B][M/64]) and a spare row of B words
+// workspace: unit totals and unit bases (both [B][M/64], 4 bytes) of the two-pass form, or the status words of the
+// one-pass kernel (8 bytes per unit, 8 per head, the flag word) - the same bytes
 static size_t compress_ws_bytes(int B, int M)
 {
-    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
+    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 8 + 64, 256);
+}
+
+// The one-pass kernel behind its init kernel.
+template <bool IS_VALUE>
+static int launch_onepass(hipStream_t st, const _Float16* xh, int B, int M, int kth, uint64_t* bmp, uint32_t* idx,
+                          uint32_t* nz_off, uint64_t* total_halfs, const uint32_t* dst_off, const uint32_t* dst_limit,
+                          uint32_t* overflow, mstf_half* nz, uint64_t cap, void* ws)
+{
+    const int nblk = M / 64, units = B * nblk;
+#ifndef MSTF_ONEPASS_W
+#define MSTF_ONEPASS_W 4
+#endif
+    const int W = nblk % MSTF_ONEPASS_W == 0 ? MSTF_ONEPASS_W : (nblk % 2 == 0 ? 2 : 1);
+    const int groups = units / W;
+    uint64_t* state = reinterpret_cast<uint64_t*>(ws);
+    const int words = groups + 1;
+    hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
+                       dim3(256), 0, st, state, words);
+    int rc = check_launch();
+    if (rc != MSTF_OK) return rc;
+#define MSTF_OP(WV)                                                                                                   \
+    hipLaunchKernelGGL((compress_onepass_kernel<IS_VALUE, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \
+                       bmp, idx, nz_off, total_halfs, dst_off, dst_limit, overflow, reinterpret_cast<char*>(nz), cap,  \
+                       state, units, groups)
+    if (W == MSTF_ONEPASS_W)
+        MSTF_OP(MSTF_ONEPASS_W);
+    else if (W == 2)
+        MSTF_OP(2);
+    else
+        MSTF_OP(1);
+#undef MSTF_OP
+    return check_launch();
 }
 
 static int check_compress_args(const void* x, int B, int M, int N, int kth)
@@ -404,6 +695,12 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     hipStream_t st = as_stream(stream);
     const int nblk = M / 64;
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
+    if (nz) {
+        if (!aligned_to(nz, 16)) return MSTF_EALIGN;
+        return launch_onepass<IS_VALUE>(st, xh, B, M, kth, bmp, idx, nz_off, total_halfs, nullptr, nullptr, nullptr, nz,
+                                        cap, ws);
+    }
+    // sizing only: counts, scan, final offsets
     const size_t ub = round_up((size_t)B * nblk * 4, 256);
     uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
     uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
@@ -412,15 +709,8 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
                        nz_off, total_halfs, nblk, kD);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    if (nz) {
-        if (!aligned_to(nz, 16)) return MSTF_EALIGN;
-        hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh,
-                           RowsView{}, M, bmp, idx, unit_base, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
-                           (uint32_t*)nullptr);
-    } else {
-        hipLaunchKernelGGL(finalize_idx_kernel, dim3((unsigned)(((size_t)nblk * kD + 255) / 256), (unsigned)B), dim3(256),
-                           0, st, idx, unit_base, nblk, kD);
-    }
+    hipLaunchKernelGGL(finalize_idx_kernel, dim3((unsigned)(((size_t)nblk * kD + 255) / 256), (unsigned)B), dim3(256), 0,
+                       st, idx, unit_base, nblk, kD);
     return check_launch();
 }
 
@@ -438,20 +728,8 @@ static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, in
         return MSTF_EALIGN;
     if (!ws || ws_bytes < compress_ws_bytes(B, M)) return MSTF_EWORKSPACE;
     if (!aligned_to(ws, 256)) return MSTF_EALIGN;
-    hipStream_t st = as_stream(stream);
-    const int nblk = M / 64;
-    const size_t ub = round_up((size_t)B * nblk * 4, 256);
-    uint32_t* unit_tot = reinterpret_cast<uint32_t*>(ws);
-    uint32_t* unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + ub);
-    const _Float16* xh = reinterpret_cast<const _Float16*>(x);
-    launch_count<IS_VALUE>(st, xh, B, M, kth, bmp, idx, unit_tot);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
-                       (uint32_t*)nullptr, (uint64_t*)nullptr, nblk, kD);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, RowsView{},
-                       M, bmp, idx, unit_base, dst_off, reinterpret_cast<char*>(nz), ~0ull, dst_limit, overflow);
-    return check_launch();
+    return launch_onepass<IS_VALUE>(as_stream(stream), reinterpret_cast<const _Float16*>(x), B, M, kth, bmp, idx, nullptr,
+                                    nullptr, dst_off, dst_limit, overflow, nz, ~0ull, ws);
 }
 
 // Rows in the layout of a projection output, optionally rotated first.  dst_off == nullptr: the compress contract

@@ -242,6 +242,69 @@ __device__ __forceinline__ uint64_t spread_bitmap(uint32_t e, uint32_t o)
     return u64_of(lo, hi);
 }
 
+// One stage of the 64x64 bit-matrix transpose across the wavefront (lane = row, the 64 bits of (lo, hi) = columns):
+// lanes l and l ^ D exchange the DxD blocks off the diagonal of every 2Dx2D block.  The partner's word comes through
+// a swizzle (no vector-ALU slot), is rotated so that the wanted bits land on their new positions and merged in.
+template <int D>
+__device__ __forceinline__ void wave_bit_transpose_stage(uint32_t& lo, uint32_t& hi, int lane)
+{
+    constexpr uint32_t M0 = D == 16 ? 0x0000FFFFu : D == 8 ? 0x00FF00FFu : D == 4 ? 0x0F0F0F0Fu : D == 2 ? 0x33333333u : 0x55555555u;
+    const bool up = (lane & D) != 0;
+    const uint32_t keep = up ? ~M0 : M0;                       // the positions this lane keeps
+    const uint32_t amt = up ? (uint32_t)D : (uint32_t)(32 - D);  // rotate right: down by D, or up by D
+    const uint32_t pl = (uint32_t)__builtin_amdgcn_ds_swizzle((int)lo, 0x1F | (D << 10));
+    const uint32_t ph = (uint32_t)__builtin_amdgcn_ds_swizzle((int)hi, 0x1F | (D << 10));
+    const uint32_t rl = __builtin_amdgcn_alignbit(pl, pl, amt), rh = __builtin_amdgcn_alignbit(ph, ph, amt);
+    lo = (lo & keep) | (rl & ~keep);
+    hi = (hi & keep) | (rh & ~keep);
+}
+// Afterwards bit t of lane k's (lo, hi) is what bit k of lane t's was: 21 vector instructions, 10 swizzles and a
+// handful of per-lane constants, against two instructions and two lane writes per column for ballots.
+__device__ __forceinline__ void wave_bit_transpose64(uint32_t& lo, uint32_t& hi, int lane)
+{
+    typedef unsigned u2v_t __attribute__((ext_vector_type(2)));
+    const u2v_t r = __builtin_amdgcn_permlane32_swap(lo, hi, false, false);  // lo of lanes 32.. <-> hi of lanes ..31
+    lo = r[0];
+    hi = r[1];
+    wave_bit_transpose_stage<16>(lo, hi, lane);
+    wave_bit_transpose_stage<8>(lo, hi, lane);
+    wave_bit_transpose_stage<4>(lo, hi, lane);
+    wave_bit_transpose_stage<2>(lo, hi, lane);
+    wave_bit_transpose_stage<1>(lo, hi, lane);
+}
+
+// Key tile bitmaps (MSB-first, lane l: tiles l and 64 + l of the unit) from the keep words of the lanes' rows
+// (kept[2h + p] bit j of lane t = channel 64h + 2j + p of token t is kept).
+__device__ __forceinline__ void key_bitmaps_from_kept(const uint32_t (&kept)[4], int lane, uint64_t& bmA, uint64_t& bmB)
+{
+    // after the transpose lane k < 32 holds channel 2k of the half, lane 32 + k channel 2k + 1
+    const int from = ((lane >> 1) + 32 * (lane & 1)) * 4;
+    uint64_t bm[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint32_t lo = kept[2 * h], hi = kept[2 * h + 1];
+        wave_bit_transpose64(lo, hi, lane);
+        lo = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)lo);
+        hi = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)hi);
+        bm[h] = u64_of(__builtin_bitreverse32(hi), __builtin_bitreverse32(lo));  // token t -> bit 63 - t
+    }
+    bmA = bm[0];
+    bmB = bm[1];
+}
+
+// Keep words of an already pruned row: every non-zero magnitude (layout of select_kth_planes' keep words).
+__device__ __forceinline__ void kept_nonzero(const uint32_t (&r)[64], uint32_t (&kept)[4])
+{
+#pragma unroll
+    for (int w = 0; w < 4; w++) kept[w] = 0u;
+#pragma unroll
+    for (int j = 0; j < 64; j++) {
+        const uint32_t e = (r[j] & 0x7FFFu) != 0u ? 1u : 0u, o = (r[j] & 0x7FFF0000u) != 0u ? 1u : 0u;
+        kept[2 * (j >> 5)] |= e << (j & 31);
+        kept[2 * (j >> 5) + 1] |= o << (j & 31);
+    }
+}
+
 __device__ __forceinline__ uint32_t wave_excl_scan(uint32_t v, int lane, uint32_t& total)
 {
     uint32_t inc = v;
