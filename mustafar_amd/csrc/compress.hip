@@ -487,7 +487,11 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     const int b = u / nblk, tb = u - b * nblk;
     uint32_t* buf = bufs[wave];
     uint32_t r[64];  // this lane's token, raw fp16 pairs; they stay in registers until they are compacted
-    unit_rows(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, buf, lane, r);
+    {
+        UnitRaw raw;  // all 16 KB requested at once; M % 64 == 0: every row exists
+        unit_fetch(x + (size_t)b * M * kD, (int64_t)tb * 64, lane, raw);
+        unit_rows_from(raw, buf, lane, r);
+    }
     uint32_t kept[4];
     if (kth > 0)
         select_kth_planes<true>(r, kth, kept);  // the sign bits become planes the search never looks at

@@ -23,17 +23,27 @@ __device__ __forceinline__ void half_slab_load(const _Float16* x, int64_t row0, 
                                                int lane, int64_t stride = kD)
 {
     const _Float16* src = x + row0 * stride + h * 64;
+    // all eight pieces are requested before the first one is staged: the loads are unconditional (a row past the
+    // end reads the last valid row instead, row0 < rows_valid) and the zeros are put in afterwards
+    uint4 v[8];
+    const int64_t last = rows_valid - 1 - row0;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const int e = j * 64 + lane;  // 16-byte piece index inside the half-slab: 8 pieces per row
         const int row = e >> 3, c16 = e & 7;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + row < rows_valid) v = *reinterpret_cast<const uint4*>(src + row * stride + c16 * 8);
+        const int64_t rr = row <= last ? row : last;
+        v[j] = *reinterpret_cast<const uint4*>(src + rr * stride + c16 * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int e = j * 64 + lane;
+        const int row = e >> 3, c16 = e & 7;
+        if (row > last) v[j] = make_uint4(0u, 0u, 0u, 0u);
         uint32_t* d = slab + row * kHalfRowDw + c16 * 4;
-        d[0] = v.x;
-        d[1] = v.y;
-        d[2] = v.z;
-        d[3] = v.w;
+        d[0] = v[j].x;
+        d[1] = v[j].y;
+        d[2] = v[j].z;
+        d[3] = v[j].w;
     }
 }
 // The 32 dwords (64 channels) of this lane's token out of the staged half-slab, into r[first .. first+32).
