@@ -68,8 +68,11 @@ int mstf_prune_rows_f16(void* stream, const mstf_half* x, mstf_half* y, int64_t 
  *   kth == 0: x is already pruned, zeros are the holes (exactly what the reference converts).
  * Phase 1 ("count") writes bmp [B,T], idx [B,T+1], nz_off [B] and *total_halfs (device uint64:
  * number of fp16 values the flat nz buffer must hold).  Phase 2 ("scatter") fills nz.
- * mstf_compress_*_f16 runs both; with nz == NULL it runs phase 1 only.  Tiles whose values
- * would not fit in nz_capacity_halfs are not written (compare *total_halfs afterwards). */
+ * mstf_compress_*_f16 produces everything with one read of x (status words in the workspace order
+ * the workgroups; they are cleared by the call itself); with nz == NULL it runs phase 1 only.  Tiles
+ * whose values would not fit in nz_capacity_halfs are not written (compare *total_halfs afterwards).
+ * A workgroup waits for the totals of the workgroups launched before it; should such a wait ever run
+ * out of its (bounded) polls, no values are written for it and *total_halfs reads as all ones. */
 size_t mstf_compress_workspace_bytes(int B, int M, int N);
 int mstf_compress_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
                           uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz,

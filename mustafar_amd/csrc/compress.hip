@@ -6,8 +6,13 @@
 // (padded row stride, so that a lane reads its own row without bank conflicts) into registers: a lane
 // holds the 128 values of its token in 64 registers and the wavefront needs 8.25 KB of LDS.
 //
-//   count kernel   : row threshold by a 15-step radix select on the fp16 magnitudes, bitmaps by ballot
-//                    (key) or in-lane packing (value), padded counts and their prefix inside the unit.
+//   one-pass kernel: everything with one read of the slab (the calls that produce the packed values): row threshold
+//                    by a 15-step radix select on bit planes, bitmaps, padded counts, compaction into an LDS
+//                    image, and the unit's place in the output from the totals that the workgroups in front of it
+//                    publish in the workspace.
+// The two-pass form remains for the sizing-only call, for phase 2 on its own and for the projection layout:
+//   count kernel   : threshold, bitmaps by ballot (key) or in-lane packing (value), padded counts and their prefix
+//                    inside the unit.
 //   scan kernel    : unit totals -> unit bases per head and, summed over the earlier heads, nz_off.
 //   scatter kernel : re-reads the slab and compacts the survivors, half a unit (64 tiles) at a time,
 //                    into an LDS image of the output that reuses the staging buffer - key: one
@@ -15,6 +20,8 @@
 //                    walks the 64 channels of its own tile - and streams the image out with 16-byte stores.
 //                    In the fused call it also turns the unit-local tile offsets in idx into final ones.
 #include "compress_common.hpp"
+
+#include <cstdlib>
 
 namespace mstf {
 
@@ -323,7 +330,7 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 // the dispatcher has started before it: every wait ends.  The waits are bounded all the same (kSpinLimit polls); a
 // workgroup that gives up sets the flag word behind the workgroup words, writes no values, and *total_halfs reads as
 // all ones.  onepass_init_kernel clears the words before the launch.
-constexpr uint32_t kSpinLimit = 1u << 20;
+constexpr uint32_t kSpinLimit = 1u << 20;  // default; the host passes the limit in (MSTF_COMPRESS_SPIN_LIMIT overrides it for tests)
 
 __global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n)
 {
@@ -351,7 +358,7 @@ constexpr uint64_t kWordReady = 1ull << 63;
 // (first <= split <= g); false when a wait ran out.
 template <int W>
 __device__ __forceinline__ bool wait_for_words(const uint64_t* state, int first, int split, int g, int wave, int lane,
-                                               uint64_t& sum_lo, uint64_t& sum_hi)
+                                               uint32_t spin_limit, uint64_t& sum_lo, uint64_t& sum_hi)
 {
     constexpr int K = 4;
     uint64_t lo = 0, hi = 0;
@@ -376,7 +383,7 @@ __device__ __forceinline__ bool wait_for_words(const uint64_t* state, int first,
                 all = all && got[k];
             }
             if (__ballot(!all) == 0ull) break;
-            if (++polls > kSpinLimit) {
+            if (++polls > spin_limit) {
                 ok = false;
                 break;
             }
@@ -469,7 +476,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     const _Float16* __restrict__ x, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
     uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
     const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
-    uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total)
+    uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total, uint32_t spin_limit)
 {
     // per wavefront: staging buffer of a half-slab, then image of half a unit's output (at most 64 tiles x 128 bytes)
     __shared__ __attribute__((aligned(16))) uint32_t bufs[W][kHalfSlabDw];
@@ -526,7 +533,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     const int head_first = (b * nblk) / W;  // first workgroup of this head
     {
         uint64_t lo = 0, hi = 0;
-        const bool ok0 = wait_for_words<W>(state, dst_off ? head_first : 0, head_first, g, wave, lane, lo, hi);
+        const bool ok0 = wait_for_words<W>(state, dst_off ? head_first : 0, head_first, g, wave, lane, spin_limit, lo, hi);
         if (lane == 0) {
             bases[wave][0] = lo;
             bases[wave][1] = hi;
@@ -629,6 +636,8 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, int B, int M, int 
     const int groups = units / W;
     uint64_t* state = reinterpret_cast<uint64_t*>(ws);
     const int words = groups + 1;
+    const char* limit_env = getenv("MSTF_COMPRESS_SPIN_LIMIT");  // read per call: a test lowers it to force the give-up path
+    const uint32_t spin_limit = limit_env ? (uint32_t)strtoul(limit_env, nullptr, 10) : kSpinLimit;
     hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
                        dim3(256), 0, st, state, words);
     int rc = check_launch();
@@ -636,7 +645,7 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, int B, int M, int 
 #define MSTF_OP(WV)                                                                                                   \
     hipLaunchKernelGGL((compress_onepass_kernel<IS_VALUE, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \
                        bmp, idx, nz_off, total_halfs, dst_off, dst_limit, overflow, reinterpret_cast<char*>(nz), cap,  \
-                       state, units, groups)
+                       state, units, groups, spin_limit)
     if (W == MSTF_ONEPASS_W)
         MSTF_OP(MSTF_ONEPASS_W);
     else if (W == 2)

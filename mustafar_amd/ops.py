@@ -80,13 +80,21 @@ class CompressedKV:
     def heads(self):
         return self.bmp.shape[0]
 
+    def used_halfs(self):
+        """Number of fp16 values in use (reads the device-side total once).  The one-pass compressor reports a wait that
+        ran out - which the dispatch order rules out - as a total of all ones: that raises here."""
+        n = int(self.total_halfs)
+        if n < 0 or n > (1 << 62):
+            raise RuntimeError("the compressor gave up waiting for an earlier workgroup; the packed values are incomplete")
+        return n
+
     def packed(self):
         """The used part of the flat value buffer (needs the host-side size)."""
-        return self.nz[:int(self.total_halfs)]
+        return self.nz[:self.used_halfs()]
 
     def nbytes(self):
         """Algorithmic size: bitmaps + offsets + packed values actually used."""
-        used = self.nz.numel() if self.total_halfs is None else int(self.total_halfs)
+        used = self.nz.numel() if self.total_halfs is None else self.used_halfs()
         return self.bmp.numel() * 8 + self.idx.numel() * 4 + used * 2
 
 

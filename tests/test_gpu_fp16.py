@@ -268,3 +268,32 @@ def test_config0_shape_against_oracle():
     o = ops.value_spmv(cv, p, groups)
     check_chain(RTOL, s_ref, p_ref, o_ref, Vp, groups, s=s[:, 0], p=p[:, 0], o=o[:, 0],
                 fused=ops.decode_attention(ck, cv, qg, groups))
+
+
+def test_one_pass_compressor_flags_a_wait_that_ran_out(monkeypatch):
+    """The one-pass compressor orders its workgroups through status words and bounds every wait.  With the bound forced
+    to zero polls from the host, a workgroup whose predecessors have not published yet gives up: then the total must
+    read as all ones (and the host layer must raise), otherwise everything must be exactly right - never a silently
+    wrong result.  Every kernel still runs to its end."""
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    K, _ = orc.make_kv(31, 16, 1024, 128)
+    Kt = torch.from_numpy(K).to(dev)
+    rb, ri, rnz, roff = orc.compress(orc.prune_rows(K, 89), 0)
+    monkeypatch.setenv("MSTF_COMPRESS_SPIN_LIMIT", "0")
+    gave_up = 0
+    for _ in range(4):
+        ck = ops.compress(Kt, False, kth=89, capacity_halfs=Kt.numel())
+        torch.cuda.synchronize()
+        if int(ck.total_halfs) == -1:
+            gave_up += 1
+            with pytest.raises(RuntimeError, match="gave up"):
+                ck.packed()
+        else:
+            assert int(ck.total_halfs) == rnz.size
+            assert np.array_equal(ck.bmp.cpu().numpy(), rb) and np.array_equal(ck.idx.cpu().numpy(), ri)
+            assert np.array_equal(ck.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+    monkeypatch.delenv("MSTF_COMPRESS_SPIN_LIMIT")
+    ck = ops.compress(Kt, False, kth=89, capacity_halfs=Kt.numel())
+    assert int(ck.total_halfs) == rnz.size
+    assert np.array_equal(ck.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
