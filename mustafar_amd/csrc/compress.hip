@@ -68,11 +68,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void co
     }
 }
 
-// The same for rows in the layout of a projection output (RowsView), optionally with the rotary embedding applied
-// first.  With ROPE the units cover all `rows` tokens of a head (ceil(rows / 64) per head): every unit rotates its
-// rows on the way in - in the layout of the loads, where a lane holds 8 channels of a row and their partners 64
-// channels on, so that x, cos, sin and the rotated rows all move as 128-byte runs - writes them to rot (same kind of
-// layout; rot.x may be the input itself) and only the units below M / 64 go on to prune and count.
+// Rows in the layout of a projection output (RowsView), optionally with the rotary embedding applied first: a unit
+// rotates its rows on the way in - in the layout of the loads, where a lane holds 8 channels of a row and their
+// partners 64 channels on, so that x, cos, sin and the rotated rows all move as 128-byte runs - and writes them to
+// rot (same kind of layout; rot.x may be the input itself).  The units below M / 64 do so inside the one-pass
+// kernel, the tokens behind them in rope_tail_kernel.
 // cos / sin: [batch entry][token][128] fp16 with strides rb, rt.
 struct RopeTables {
     const _Float16* cos;
@@ -87,81 +87,55 @@ __device__ __forceinline__ void unit_fetch_rotated(const RowsView& src, const Ro
     _Float16* rb = const_cast<_Float16*>(rot.head(b));
     const _Float16* cb = rope.cos + bt * rope.rb;
     const _Float16* sb = rope.sin + bt * rope.rb;
+    // four pieces at a time: all 24 loads of a batch are requested before the first one is used (loads behind a
+    // per-piece branch would each wait for the one before); a row past the end reads the last row instead and is
+    // neither rotated into the output nor stored
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const int e = j * 64 + lane;
-        const int64_t t = (int64_t)tb * 64 + (e >> 3);
-        const int c = (e & 7) * 8;
-        const uint4 z = make_uint4(0u, 0u, 0u, 0u);
-        uint4 x0 = z, x1 = z, c0 = z, c1 = z, s0 = z, s1 = z;
-        if (t < rows) {
+    for (int j0 = 0; j0 < 8; j0 += 4) {
+        uint4 x0[4], x1[4], c0[4], c1[4], s0[4], s1[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int e = (j0 + k) * 64 + lane;
+            int64_t t = (int64_t)tb * 64 + (e >> 3);
+            t = t < rows ? t : rows - 1;
+            const int c = (e & 7) * 8;
             const _Float16* xp = xb + t * src.st + c;
             const _Float16* cp = cb + t * rope.rt + c;
             const _Float16* sp = sb + t * rope.rt + c;
-            x0 = *reinterpret_cast<const uint4*>(xp);
-            x1 = *reinterpret_cast<const uint4*>(xp + 64);
-            c0 = *reinterpret_cast<const uint4*>(cp);
-            c1 = *reinterpret_cast<const uint4*>(cp + 64);
-            s0 = *reinterpret_cast<const uint4*>(sp);
-            s1 = *reinterpret_cast<const uint4*>(sp + 64);
+            x0[k] = *reinterpret_cast<const uint4*>(xp);
+            x1[k] = *reinterpret_cast<const uint4*>(xp + 64);
+            c0[k] = *reinterpret_cast<const uint4*>(cp);
+            c1[k] = *reinterpret_cast<const uint4*>(cp + 64);
+            s0[k] = *reinterpret_cast<const uint4*>(sp);
+            s1[k] = *reinterpret_cast<const uint4*>(sp + 64);
         }
-        rope_piece(x0, x1, c0, c1, s0, s1, raw.v[0][j], raw.v[1][j]);
-        if (t < rows) {
-            _Float16* rp = rb + t * rot.st + c;
-            *reinterpret_cast<uint4*>(rp) = raw.v[0][j];
-            *reinterpret_cast<uint4*>(rp + 64) = raw.v[1][j];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int j = j0 + k;
+            const int e = j * 64 + lane;
+            const int64_t t = (int64_t)tb * 64 + (e >> 3);
+            const int c = (e & 7) * 8;
+            rope_piece(x0[k], x1[k], c0[k], c1[k], s0[k], s1[k], raw.v[0][j], raw.v[1][j]);
+            if (t < rows) {
+                _Float16* rp = rb + t * rot.st + c;
+                *reinterpret_cast<uint4*>(rp) = raw.v[0][j];
+                *reinterpret_cast<uint4*>(rp + 64) = raw.v[1][j];
+            } else {
+                raw.v[0][j] = make_uint4(0u, 0u, 0u, 0u);
+                raw.v[1][j] = make_uint4(0u, 0u, 0u, 0u);
+            }
         }
     }
 }
-// grid = ceil(units / upw), 64 threads; units = B * (ROPE ? ceil(rows / 64) : M / 64); upw = 1 with ROPE.
-template <bool IS_VALUE, bool ROPE>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void proj_count_kernel(
-    RowsView src, RopeTables rope, RowsView rot, int rows, int M, int kth, uint64_t* __restrict__ bmp,
-    uint32_t* __restrict__ idx, uint32_t* __restrict__ unit_tot, int units, int upw)
+// grid = B * tail units (64 tokens each), 64 threads: rotation only, for the tokens behind the compressed ones
+// (first_block = M / 64 onwards) of every head.
+__global__ __launch_bounds__(64) void rope_tail_kernel(RowsView src, RopeTables rope, RowsView rot, int rows,
+                                                       int first_block, int tail_blocks)
 {
-    __shared__ uint32_t slab[kHalfSlabDw];
-    const int lane = lane_id();
-    const int nblk = M / 64;
-    const int nblk_all = ROPE ? (rows + 63) / 64 : nblk;
-    const size_t T = (size_t)M * kD / 64;
-    const int unit0 = (int)blockIdx.x * upw;
-    int n = units - unit0;
-    n = n > upw ? upw : n;
+    const int b = (int)blockIdx.x / tail_blocks;
+    const int tb = first_block + (int)blockIdx.x % tail_blocks;
     UnitRaw raw;
-    if (!ROPE) {
-        const int b0 = unit0 / nblk_all;
-        unit_fetch(src.head(b0), (int64_t)(unit0 - b0 * nblk_all) * 64, lane, raw, src.st);
-    }
-#pragma unroll 1
-    for (int u = 0; u < n; u++) {
-        const int unit = unit0 + u;
-        const int b = unit / nblk_all, tb = unit - b * nblk_all;
-        if (ROPE) {
-            unit_fetch_rotated(src, rope, rot, b, tb, rows, lane, raw);
-            if (tb >= nblk) continue;  // uniform: a unit of the dense tail
-        }
-        uint32_t mag[64];
-        unit_rows_from(raw, slab, lane, mag);
-        if (!ROPE && u + 1 < n) {
-            const int bn = (unit + 1) / nblk_all;
-            unit_fetch(src.head(bn), (int64_t)(unit + 1 - bn * nblk_all) * 64, lane, raw, src.st);
-        }
-#pragma unroll
-        for (int j = 0; j < 64; j++) mag[j] &= 0x7FFF7FFFu;
-        uint64_t bmA, bmB;
-        unit_keep<IS_VALUE>(mag, kth, lane, bmA, bmB);
-        uint64_t* bo = bmp + (size_t)b * T + (size_t)tb * kD;
-        bo[lane] = bmA;
-        bo[64 + lane] = bmB;
-        const uint32_t cA = padded_units(bmA), cB = padded_units(bmB);
-        uint32_t totA, totB;
-        const uint32_t eA = wave_excl_scan(cA, lane, totA);
-        const uint32_t eB = wave_excl_scan(cB, lane, totB);
-        uint32_t* io = idx + (size_t)b * (T + 1) + (size_t)tb * kD;
-        io[lane] = eA;
-        io[64 + lane] = totA + eB;
-        if (lane == 0) unit_tot[(size_t)b * nblk + tb] = totA + totB;
-    }
+    unit_fetch_rotated(src, rope, rot, b, tb, rows, lane_id(), raw);
 }
 
 // ------------------------------------------------------------------------------- scans
@@ -247,9 +221,8 @@ __device__ __forceinline__ void scatter_half(const uint32_t (&v)[32], uint64_t b
 // the unit-local offsets of the count kernel, which are completed here with unit_base (ADD_BASE true).
 // head_limit (nullable): end of head b's slab in 16-byte units from nz; a unit whose values would pass it is
 // skipped and *overflow is set.
-// PROJ: the rows come through `view` (x is ignored) instead of the contiguous [B, M, 128] matrix x.
-template <bool IS_VALUE, bool ADD_BASE, bool PROJ = false>
-__global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, RowsView view, int M,
+template <bool IS_VALUE, bool ADD_BASE>
+__global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __restrict__ x, int M,
                                                               const uint64_t* __restrict__ bmp, uint32_t* idx,
                                                               const uint32_t* __restrict__ unit_base,
                                                               const uint32_t* __restrict__ nz_off,
@@ -302,10 +275,7 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
         uint32_t bytes = ((h == 0 ? mid : end) - s_h) * 4u;
         if (bytes > 64u * 128u) bytes = 64u * 128u;  // never true for offsets that follow from the bitmaps
         uint32_t v[32];
-        if (PROJ)
-            half_slab_load(view.head(b), (int64_t)tb * 64, (int64_t)M, h, buf, lane, view.st);
-        else
-            half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, buf, lane);
+        half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, buf, lane);
         __builtin_amdgcn_wave_barrier();
         row_of_lane(buf, lane, v, 0);
         __builtin_amdgcn_wave_barrier();
@@ -471,9 +441,18 @@ __device__ __forceinline__ void stream_image(uint32_t img, uint32_t bytes, char*
 //   packed layout  (dst_off == nullptr): heads back to back, nz_off[b] and *total_halfs are written here;
 //   pooled layout  (dst_off given): head b's values start at nz + 16 * dst_off[b] and may not pass
 //                  nz + 16 * dst_limit[b] (else *overflow is set and the unit's values are not written).
-template <bool IS_VALUE, int W>
+// SRC: where the rows come from - kSrcMatrix: the contiguous [B, M, 128] matrix x; kSrcView: through `view` (the
+// layout of a projection output); kSrcRope: through `view`, rotated on the way in and written to `rot`.
+enum { kSrcMatrix = 0, kSrcView = 1, kSrcRope = 2 };
+struct ProjArgs {
+    RowsView view;
+    RopeTables rope;
+    RowsView rot;
+    int rows;
+};
+template <bool IS_VALUE, int W, int SRC>
 __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void compress_onepass_kernel(
-    const _Float16* __restrict__ x, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
+    const _Float16* __restrict__ x, ProjArgs proj, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
     uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
     const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
     uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total, uint32_t spin_limit)
@@ -496,7 +475,12 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     uint32_t r[64];  // this lane's token, raw fp16 pairs; they stay in registers until they are compacted
     {
         UnitRaw raw;  // all 16 KB requested at once; M % 64 == 0: every row exists
-        unit_fetch(x + (size_t)b * M * kD, (int64_t)tb * 64, lane, raw);
+        if (SRC == kSrcMatrix)
+            unit_fetch(x + (size_t)b * M * kD, (int64_t)tb * 64, lane, raw);
+        else if (SRC == kSrcView)
+            unit_fetch(proj.view.head(b), (int64_t)tb * 64, lane, raw, proj.view.st);
+        else
+            unit_fetch_rotated(proj.view, proj.rope, proj.rot, b, tb, proj.rows, lane, raw);
         unit_rows_from(raw, buf, lane, r);
     }
     uint32_t kept[4];
@@ -623,8 +607,8 @@ static size_t compress_ws_bytes(int B, int M)
 }
 
 // The one-pass kernel behind its init kernel.
-template <bool IS_VALUE>
-static int launch_onepass(hipStream_t st, const _Float16* xh, int B, int M, int kth, uint64_t* bmp, uint32_t* idx,
+template <bool IS_VALUE, int SRC = kSrcMatrix>
+static int launch_onepass(hipStream_t st, const _Float16* xh, const ProjArgs& proj, int B, int M, int kth, uint64_t* bmp, uint32_t* idx,
                           uint32_t* nz_off, uint64_t* total_halfs, const uint32_t* dst_off, const uint32_t* dst_limit,
                           uint32_t* overflow, mstf_half* nz, uint64_t cap, void* ws)
 {
@@ -643,7 +627,7 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, int B, int M, int 
     int rc = check_launch();
     if (rc != MSTF_OK) return rc;
 #define MSTF_OP(WV)                                                                                                   \
-    hipLaunchKernelGGL((compress_onepass_kernel<IS_VALUE, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \
+    hipLaunchKernelGGL((compress_onepass_kernel<IS_VALUE, WV, SRC>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, proj, M, kth, \
                        bmp, idx, nz_off, total_halfs, dst_off, dst_limit, overflow, reinterpret_cast<char*>(nz), cap,  \
                        state, units, groups, spin_limit)
     if (W == MSTF_ONEPASS_W)
@@ -675,7 +659,7 @@ static int scatter_impl(void* stream, const mstf_half* x, int B, int M, int N, c
     if (!bmp || !idx || !nz_off || !nz) return MSTF_EINVAL;
     if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz_off, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
     hipLaunchKernelGGL((compress_scatter_kernel<IS_VALUE, false>), dim3((unsigned)(B * (M / 64))), dim3(64), 0,
-                       as_stream(stream), reinterpret_cast<const _Float16*>(x), RowsView{}, M, bmp, const_cast<uint32_t*>(idx),
+                       as_stream(stream), reinterpret_cast<const _Float16*>(x), M, bmp, const_cast<uint32_t*>(idx),
                        (const uint32_t*)nullptr, nz_off, reinterpret_cast<char*>(nz), cap, (const uint32_t*)nullptr,
                        (uint32_t*)nullptr);
     return check_launch();
@@ -710,7 +694,7 @@ static int compress_impl(void* stream, const mstf_half* x, int B, int M, int N, 
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     if (nz) {
         if (!aligned_to(nz, 16)) return MSTF_EALIGN;
-        return launch_onepass<IS_VALUE>(st, xh, B, M, kth, bmp, idx, nz_off, total_halfs, nullptr, nullptr, nullptr, nz,
+        return launch_onepass<IS_VALUE>(st, xh, ProjArgs{}, B, M, kth, bmp, idx, nz_off, total_halfs, nullptr, nullptr, nullptr, nz,
                                         cap, ws);
     }
     // sizing only: counts, scan, final offsets
@@ -741,7 +725,7 @@ static int append_impl(void* stream, const mstf_half* x, int B, int M, int N, in
         return MSTF_EALIGN;
     if (!ws || ws_bytes < compress_ws_bytes(B, M)) return MSTF_EWORKSPACE;
     if (!aligned_to(ws, 256)) return MSTF_EALIGN;
-    return launch_onepass<IS_VALUE>(as_stream(stream), reinterpret_cast<const _Float16*>(x), B, M, kth, bmp, idx, nullptr,
+    return launch_onepass<IS_VALUE>(as_stream(stream), reinterpret_cast<const _Float16*>(x), ProjArgs{}, B, M, kth, bmp, idx, nullptr,
                                     nullptr, dst_off, dst_limit, overflow, nz, ~0ull, ws);
 }
 
@@ -775,8 +759,6 @@ static int proj_impl(void* stream, const mstf_proj_source* s, int is_value, int 
                        s->rot_stride_head, s->heads};
     const RopeTables tab{reinterpret_cast<const _Float16*>(s->cos), reinterpret_cast<const _Float16*>(s->sin),
                          s->rope_stride_batch, s->rope_stride_token};
-    uint32_t* unit_tot = nullptr;
-    uint32_t* unit_base = nullptr;
     if (M > 0) {
         if (!bmp || !idx || !nz) return MSTF_EINVAL;
         if (dst_off ? (!dst_limit || !overflow) : (!nz_off || !total_halfs)) return MSTF_EINVAL;
@@ -786,40 +768,28 @@ static int proj_impl(void* stream, const mstf_proj_source* s, int is_value, int 
             return MSTF_EALIGN;
         if (!ws || ws_bytes < compress_ws_bytes(B, M)) return MSTF_EWORKSPACE;
         if (!aligned_to(ws, 256)) return MSTF_EALIGN;
-        unit_tot = reinterpret_cast<uint32_t*>(ws);
-        unit_base = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(ws) + round_up((size_t)B * nblk * 4, 256));
+        const ProjArgs pa{src, tab, rot, s->rows};
+        const uint64_t capacity = dst_off ? ~0ull : cap;
+        int rc;
+        if (rope)
+            rc = launch_onepass<false, kSrcRope>(st, nullptr, pa, B, M, kth, bmp, idx, nz_off, total_halfs, dst_off,
+                                                 dst_limit, overflow, nz, capacity, ws);
+        else if (is_value)
+            rc = launch_onepass<true, kSrcView>(st, nullptr, pa, B, M, kth, bmp, idx, nz_off, total_halfs, dst_off,
+                                                dst_limit, overflow, nz, capacity, ws);
+        else
+            rc = launch_onepass<false, kSrcView>(st, nullptr, pa, B, M, kth, bmp, idx, nz_off, total_halfs, dst_off,
+                                                 dst_limit, overflow, nz, capacity, ws);
+        if (rc != MSTF_OK) return rc;
     }
-    const int units = rope ? (int)units_all : B * nblk;
-    const int upw = !rope && units >= 4096 ? 2 : 1;
-    const unsigned grid = (unsigned)((units + upw - 1) / upw);
-#define MSTF_PC(V, R)                                                                                              \
-    hipLaunchKernelGGL((proj_count_kernel<V, R>), dim3(grid), dim3(64), 0, st, src, tab, rot, s->rows, M, kth, bmp, idx, \
-                       unit_tot, units, upw)
-    if (rope)
-        MSTF_PC(false, true);
-    else if (is_value)
-        MSTF_PC(true, false);
-    else
-        MSTF_PC(false, false);
-#undef MSTF_PC
-    int rc = check_launch();
-    if (rc != MSTF_OK || M == 0) return rc;
-    hipLaunchKernelGGL(scan_units_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base, idx,
-                       dst_off ? (uint32_t*)nullptr : nz_off, dst_off ? (uint64_t*)nullptr : total_halfs, nblk, kD);
-    if ((rc = check_launch()) != MSTF_OK) return rc;
-    const RowsView rd = rope ? rot : src;  // the scatter pass reads the rotated rows
-    const uint32_t* base_of_head = dst_off ? dst_off : nz_off;
-    const uint64_t capacity = dst_off ? ~0ull : cap;
-#define MSTF_PS(V)                                                                                                  \
-    hipLaunchKernelGGL((compress_scatter_kernel<V, true, true>), dim3((unsigned)(B * nblk)), dim3(64), 0, st,       \
-                       (const _Float16*)nullptr, rd, M, bmp, idx, unit_base, base_of_head, reinterpret_cast<char*>(nz), \
-                       capacity, dst_limit, overflow)
-    if (is_value)
-        MSTF_PS(true);
-    else
-        MSTF_PS(false);
-#undef MSTF_PS
-    return check_launch();
+    // the tokens behind the compressed ones are only rotated
+    const int blocks_all = (s->rows + 63) / 64;
+    if (rope && blocks_all > nblk) {
+        hipLaunchKernelGGL(rope_tail_kernel, dim3((unsigned)(B * (blocks_all - nblk))), dim3(64), 0, st, src, tab, rot,
+                           s->rows, nblk, blocks_all - nblk);
+        return check_launch();
+    }
+    return MSTF_OK;
 }
 
 }  // namespace mstf
