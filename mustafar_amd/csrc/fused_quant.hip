@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             const QSide& S = n < kKeySubs ? K : V;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
-                               lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), lane, mode);
+                               lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), end_of(n), lane, mode);
             stage_img_exec<NM>(S.bmp + t, lbase, zaddr, waddr, wgroup, acc);
         };
 

@@ -52,20 +52,36 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t codes, h2_t neg_bias, 
     return as_u32((x + neg_bias) * scale2);
 }
 
-// One stage: every lane owns one packed word (tile = lane / kSlots of the pass, word = lane % kSlots) and
-// writes that word's values to the tile image.  Lanes past a tile's last word decode whatever follows in
-// the staged buffer into image slots no rank ever points to.
-//   meta  : LDS address of the staged metadata; words: LDS address of the staged words, word 0 = `start_word`
+// One stage: every lane owns one packed word and writes that word's values to the tile image.  A tile's words are
+// visited in two halves: first words 0 .. kSlots/2 - 1 of every tile (kSlots/2 lanes per tile: all there is for a tile
+// with at most 32 survivors), then - only if some tile of the stage has more words, a wave-uniform test on the word
+// offsets - words kSlots/2 .. kSlots - 1.  Lanes past a tile's last word decode whatever follows in the staged buffer
+// into image slots no rank ever points to.
+//   meta  : LDS address of the staged metadata; words: LDS address of the staged words, word 0 = `start_word`;
+//   end_word: where the stage's last tile ends
 template <int BIT, bool G32 = false>
-__device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uint32_t img, uint32_t start_word, int lane,
-                                              int mode)
+__device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uint32_t img, uint32_t start_word,
+                                              uint32_t end_word, int lane, int mode)
 {
     using F = QFmt<BIT>;
     typedef short s2_t __attribute__((ext_vector_type(2)));
+    constexpr int kHalfSlots = F::kSlots / 2;
+    constexpr int kTilesPerHalfPass = 64 / kHalfSlots;
+    constexpr int kHalfPasses = kSubTiles / kTilesPerHalfPass;
+    static_assert(kSubTiles == 32, "lanes 0..31 test the 32 tiles of the stage");
+    bool need_high;
+    {
+        const uint32_t t = (uint32_t)(lane < 32 ? lane : 31);
+        const uint32_t o = lds_load_u32(meta + t * 4u);
+        const uint32_t nx = lane < 31 ? lds_load_u32(meta + t * 4u + 4u) : end_word;
+        need_high = __ballot(lane < 32 && nx - o > (uint32_t)kHalfSlots) != 0ull;
+    }
 #pragma unroll
-    for (int p = 0; p < F::kPasses; p++) {
-        const uint32_t tl = (uint32_t)(p * F::kTilesPerPass + lane / F::kSlots);
-        const uint32_t slot = (uint32_t)(lane % F::kSlots);
+    for (int hp = 0; hp < 2 * kHalfPasses; hp++) {
+        const int half = hp / kHalfPasses, p = hp % kHalfPasses;
+        if (half == 1 && !need_high) break;
+        const uint32_t tl = (uint32_t)(p * kTilesPerHalfPass + lane / kHalfSlots);
+        const uint32_t slot = (uint32_t)(half * kHalfSlots + lane % kHalfSlots);
         const uint32_t off = lds_load_u32(meta + tl * 4u);
         // sc / zp: the pair of the tile (low half) or, G32, both pairs (first in the low half)
         const uint32_t sc = G32 ? lds_load_u32(meta + 128u + tl * 4u) : lds_load_u16(meta + 128u + tl * 2u);

@@ -84,15 +84,16 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
         if (n + 1 < nsubs) touch = issue(n + 1, t_nxt, s_nxt, e_nxt);
         const size_t t_now = t_cur;
-        const uint32_t s_now = s_cur;
+        const uint32_t s_now = s_cur, e_now = e_cur;
         t_cur = t_nxt;
         s_cur = s_nxt;
+        e_cur = e_nxt;
         if (n + 2 < nsubs) {
             t_nxt = tile_of(n + 2);
             bounds(t_nxt, s_nxt, e_nxt);
         }
         dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
-                           lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, lane, mode);
+                           lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, uni(e_now), lane, mode);
         const uint64_t* bm = c.bmp + t_now;
         const uint32_t waddr = waddr_of(n);
         stage_img_exec<NM>(bm, lbase, zaddr, waddr, wgroup, acc);

@@ -195,14 +195,20 @@ __global__ __launch_bounds__(256) void scale_softmax_kernel(const _Float16* __re
         typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
         float w[kSoftmaxPieces][8];
         float mx = -INFINITY;
+        // every piece is requested before the first one is used: the loads are unconditional (a piece past the end
+        // reads the row's first one instead and is ignored)
+        h8_t v[kSoftmaxPieces];
 #pragma unroll
         for (int k = 0; k < kSoftmaxPieces; k++) {
             const int i = (k * 256 + tid) * 8;
-            if (i < L) {
-                const h8_t v = *reinterpret_cast<const h8_t*>(sr + i);
+            v[k] = *reinterpret_cast<const h8_t*>(sr + (i < L ? i : 0));
+        }
+#pragma unroll
+        for (int k = 0; k < kSoftmaxPieces; k++) {
+            if ((k * 256 + tid) * 8 < L) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    w[k][e] = (float)(_Float16)((float)v[e] / div);
+                    w[k][e] = (float)(_Float16)((float)v[k][e] / div);
                     mx = fmaxf(mx, w[k][e]);
                 }
             }
