@@ -386,47 +386,51 @@ __device__ __forceinline__ void compact_half(const uint32_t (&r)[64], const uint
         *(MSTF_LDS u32x4_t*)(uintptr_t)(img + o) = u32x4_t{0u, 0u, 0u, 0u};  // the padding stays +0.0
     uint32_t we = __builtin_bitreverse32(kept[2 * h]), wo = __builtin_bitreverse32(kept[2 * h + 1]);
     const uint64_t all = __builtin_amdgcn_read_exec();  // every statement hands exec back as it found it
+    uint64_t m1;
     if (!IS_VALUE) {
-        uint32_t off = img;  // wave-uniform
-        uint32_t t, n;
-        // doubling pops the channel's keep bit of every token into vcc; the keepers then write at the tile's offset
-        // plus twice their rank among the keepers, and the offset moves on by the padded count
-#define MSTF_KEY_CHANNEL(W, STORE)                                                                                   \
-    asm volatile("v_add_co_u32 %[w], vcc, %[w], %[w]\n\t"                                                            \
-                 "s_mov_b64 exec, vcc\n\t"                                                                           \
-                 "v_mbcnt_lo_u32_b32 %[t], exec_lo, 0\n\t"                                                           \
-                 "v_mbcnt_hi_u32_b32 %[t], exec_hi, %[t]\n\t"                                                        \
-                 "v_lshl_add_u32 %[t], %[t], 1, %[off]\n\t" STORE " %[t], %[v]\n\t"                                  \
-                 "s_bcnt1_i32_b64 %[n], exec\n\t"                                                                    \
-                 "s_add_i32 %[n], %[n], 7\n\t"                                                                       \
-                 "s_andn2_b32 %[n], %[n], 7\n\t"                                                                     \
-                 "s_lshl1_add_u32 %[off], %[n], %[off]\n\t"                                                          \
-                 "s_mov_b64 exec, %[all]"                                                                            \
-                 : [w] "+v"(W), [off] "+s"(off), [t] "=&v"(t), [n] "=&s"(n)                                          \
-                 : [v] "v"(r[32 * h + (c >> 1)]), [all] "s"(all)                                                     \
-                 : "vcc", "scc", "memory")
+        const uint32_t voff = img + own4 * 4u;  // lane c: where tile c of the half starts in the image
+        uint32_t t, o0, o1;
+        // two channels per statement: doubling pops the channels' keep bits of every token into vcc and a scalar
+        // pair, the tiles' offsets come out of lanes c and c + 1, then the keepers of each channel write at the
+        // tile's offset plus twice their rank among the keepers
 #pragma unroll
         for (int c = 0; c < 64; c += 2) {
-            MSTF_KEY_CHANNEL(we, "ds_write_b16");
-            MSTF_KEY_CHANNEL(wo, "ds_write_b16_d16_hi");
+            asm volatile("v_add_co_u32 %[we], vcc, %[we], %[we]\n\t"
+                         "v_add_co_u32 %[wo], %[m1], %[wo], %[wo]\n\t"
+                         "v_readlane_b32 %[o0], %[voff], %[c0]\n\t"
+                         "v_readlane_b32 %[o1], %[voff], %[c1]\n\t"
+                         "s_mov_b64 exec, vcc\n\t"
+                         "v_mbcnt_lo_u32_b32 %[t], exec_lo, 0\n\t"
+                         "v_mbcnt_hi_u32_b32 %[t], exec_hi, %[t]\n\t"
+                         "v_lshl_add_u32 %[t], %[t], 1, %[o0]\n\t"
+                         "ds_write_b16 %[t], %[v]\n\t"
+                         "s_mov_b64 exec, %[m1]\n\t"
+                         "v_mbcnt_lo_u32_b32 %[t], exec_lo, 0\n\t"
+                         "v_mbcnt_hi_u32_b32 %[t], exec_hi, %[t]\n\t"
+                         "v_lshl_add_u32 %[t], %[t], 1, %[o1]\n\t"
+                         "ds_write_b16_d16_hi %[t], %[v]\n\t"
+                         "s_mov_b64 exec, %[all]"
+                         : [we] "+v"(we), [wo] "+v"(wo), [t] "=&v"(t), [m1] "=&s"(m1), [o0] "=&s"(o0), [o1] "=&s"(o1)
+                         : [v] "v"(r[32 * h + (c >> 1)]), [voff] "v"(voff), [c0] "n"(c), [c1] "n"(c + 1), [all] "s"(all)
+                         : "vcc", "memory");
         }
-#undef MSTF_KEY_CHANNEL
     } else {
         uint32_t a = img + own4 * 4u;
-#define MSTF_VALUE_CHANNEL(W, STORE)                                                             \
-    asm volatile("v_add_co_u32 %[w], vcc, %[w], %[w]\n\t"                                        \
-                 "s_mov_b64 exec, vcc\n\t" STORE " %[a], %[v]\n\t"                               \
-                 "v_add_u32 %[a], 2, %[a]\n\t"                                                   \
-                 "s_mov_b64 exec, %[all]"                                                        \
-                 : [w] "+v"(W), [a] "+v"(a)                                                      \
-                 : [v] "v"(r[32 * h + (c >> 1)]), [all] "s"(all)                                 \
-                 : "vcc", "memory")
 #pragma unroll
         for (int c = 0; c < 64; c += 2) {
-            MSTF_VALUE_CHANNEL(we, "ds_write_b16");
-            MSTF_VALUE_CHANNEL(wo, "ds_write_b16_d16_hi");
+            asm volatile("v_add_co_u32 %[we], vcc, %[we], %[we]\n\t"
+                         "v_add_co_u32 %[wo], %[m1], %[wo], %[wo]\n\t"
+                         "s_mov_b64 exec, vcc\n\t"
+                         "ds_write_b16 %[a], %[v]\n\t"
+                         "v_add_u32 %[a], 2, %[a]\n\t"
+                         "s_mov_b64 exec, %[m1]\n\t"
+                         "ds_write_b16_d16_hi %[a], %[v]\n\t"
+                         "v_add_u32 %[a], 2, %[a]\n\t"
+                         "s_mov_b64 exec, %[all]"
+                         : [we] "+v"(we), [wo] "+v"(wo), [a] "+v"(a), [m1] "=&s"(m1)
+                         : [v] "v"(r[32 * h + (c >> 1)]), [all] "s"(all)
+                         : "vcc", "memory");
         }
-#undef MSTF_VALUE_CHANNEL
     }
     __builtin_amdgcn_wave_barrier();
 }
