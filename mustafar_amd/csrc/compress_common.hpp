@@ -113,14 +113,15 @@ struct UnitRaw {
 };
 __device__ __forceinline__ void unit_fetch(const _Float16* x, int64_t row0, int lane, UnitRaw& raw, int64_t stride = kD)
 {
+    // one wave-uniform base and a 32-bit byte offset per lane: the sixteen loads differ by constants
+    const char* base = reinterpret_cast<const char*>(x + row0 * stride);
+    const uint32_t row_bytes = (uint32_t)stride * 2u;
+    const uint32_t lane_off = (uint32_t)(lane >> 3) * row_bytes + (uint32_t)(lane & 7) * 16u;
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        const _Float16* src = x + row0 * stride + h * 64;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int e = j * 64 + lane;
-            raw.v[h][j] = *reinterpret_cast<const uint4*>(src + (e >> 3) * stride + (e & 7) * 8);
-        }
+        for (int j = 0; j < 8; j++)
+            raw.v[h][j] = *reinterpret_cast<const uint4*>(base + (lane_off + (uint32_t)j * 8u * row_bytes + (uint32_t)h * 128u));
     }
 }
 __device__ __forceinline__ void unit_rows_from(const UnitRaw& raw, uint32_t* slab, int lane, uint32_t (&r)[64])
