@@ -135,20 +135,21 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
         const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
 
-        auto stage = [&](int n, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
+        auto stage = [&](int n, uint2 bits, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
             const QSide& S = n < kKeySubs ? K : V;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
                                lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), end_of(n), lane, mode);
-            stage_img_exec<NM>(S.bmp + t, lbase, zaddr, waddr, wgroup, acc);
+            stage_img_exec<NM>(S.bmp + t, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc);
         };
 
 #pragma unroll
         for (int n = 0; n < kKeySubs + kValSubs; n++) {
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
+            const uint2 bits = touch;  // lane l < 32: bitmap l of stage n
             if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
             if (n < kKeySubs) {
-                stage(n, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
+                stage(n, bits, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
             } else {
                 if (n == kKeySubs) block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
                 const int vs = n - kKeySubs;  // value stage: half = vs / 2, tokens (vs % 2) * 32..
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
                 f4_t tmp[NM];
 #pragma unroll
                 for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
-                stage(n, prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u, 4u * kPRow, tmp);
+                stage(n, bits, prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u, 4u * kPRow, tmp);
 #pragma unroll
                 for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
             }

@@ -320,16 +320,22 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
     }
 }
 
-// The kSubTiles tiles of one dequantised stage: bitmaps of the first batch requested and waited for here (the
-// dequantisation in front has lane-dependent branches, so nothing scalar is carried across it), the others one
-// batch ahead.  img: LDS address of the stage's image; wbase: LDS address of w[lane & 3][first tile of the stage].
+// The kSubTiles tiles of one dequantised stage.  The bitmaps of the first batch come out of the registers in which
+// lane l < 32 already holds bitmap l of the stage (bm_lo, bm_hi: the coalesced load that pulled the stage's bitmaps
+// into L2 one stage ahead) - the dequantisation in front has lane-dependent branches, so nothing scalar is carried
+// across it, and a scalar load here would be waited for on the spot; the other batches are requested one batch ahead.
+// img: LDS address of the stage's image; wbase: LDS address of w[lane & 3][first tile of the stage].
 template <int NM>
-__device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t img, uint32_t zaddr, uint32_t wbase,
-                                               uint32_t wgroup, f4_t (&acc)[NM])
+__device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t bm_lo, uint32_t bm_hi, uint32_t img,
+                                               uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM])
 {
     constexpr int G = kSubTiles / 8;
     u32x16_t cur;
-    asm volatile("s_load_dwordx16 %0, %1, 0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(cur) : "s"(bm) : "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        cur[2 * i] = (uint32_t)__builtin_amdgcn_readlane((int)bm_lo, i);
+        cur[2 * i + 1] = (uint32_t)__builtin_amdgcn_readlane((int)bm_hi, i);
+    }
     static_for<G>([&](auto gc) {
         constexpr int g = decltype(gc)::value;
         u32x16_t nxt;

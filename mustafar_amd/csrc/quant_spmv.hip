@@ -82,6 +82,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
     bounds(t_nxt, s_nxt, e_nxt);
     for (int n = 0; n < nsubs; n++) {
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
+        const uint2 bits = touch;  // lane l < 32: bitmap l of stage n
         if (n + 1 < nsubs) touch = issue(n + 1, t_nxt, s_nxt, e_nxt);
         const size_t t_now = t_cur;
         const uint32_t s_now = s_cur, e_now = e_cur;
@@ -96,7 +97,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
                            lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, uni(e_now), lane, mode);
         const uint64_t* bm = c.bmp + t_now;
         const uint32_t waddr = waddr_of(n);
-        stage_img_exec<NM>(bm, lbase, zaddr, waddr, wgroup, acc);
+        stage_img_exec<NM>(bm, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc);
         wait_lgkm0();  // every read of the image and of the staged buffers is done before they are rewritten
     }
 }
