@@ -42,6 +42,13 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     if (tokens_dev) {
         const int valid = *tokens_dev / 64;
         nblk = valid < nblk ? valid : nblk;
+        // the launch is sized for one block per wavefront at full capacity; the blocks a wavefront walks follow from
+        // the tokens that are there now, as a launch sized for exactly them would choose (fused_blocks_per_wave), and
+        // the workgroups behind the last block leave neutral partials
+        if (MULTI) {
+            const int r = ((int)gridDim.y * nblk + kFusedResident - 1) / kFusedResident;
+            bpw = r < 1 ? 1 : (r > kFusedMaxBpw ? kFusedMaxBpw : r);
+        }
     }
     constexpr int kQLds = NM * 4 * D * 2;          // query rows [4*NM][D] fp16
     constexpr int kPRow = 64 * 2;                  // one row of block weights: 64 tokens fp16
@@ -529,7 +536,10 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
 {
     const size_t tstride = tile_stride ? tile_stride : (size_t)tokens * head_dim / 64;
     const int Bkv = Bq / groups, nblk = tokens / 64;
-    const int bpw = fused_blocks_per_wave(tokens, Bkv), ns = fused_nsplit(tokens, bpw);
+    // token count in device memory: as many splits as any count up to `tokens` needs, the kernel works out the blocks
+    // per wavefront itself
+    const int bpw = tokens_dev ? 0 : fused_blocks_per_wave(tokens, Bkv);
+    const int ns = tokens_dev ? fused_nsplit_capacity(tokens, Bkv) : fused_nsplit(tokens, bpw);
     const int nst = nsplit_total > 0 ? nsplit_total : ns;
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * nst * head_dim;
@@ -547,7 +557,7 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
         if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
     } else {
         if (bpw == 1) MSTF_FD(2, false); else MSTF_FD(2, true);
-    }
+    }  // (bpw == 0: the kernel decides, MULTI form)
 #undef MSTF_FD
     return check_launch();
 }
@@ -764,7 +774,7 @@ extern "C" int mstf_decode_attention_window_pool_f16(void* stream, const uint64_
     const size_t need = mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, head_dim, Bq, groups);
     if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
     if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
-    const int ns = splits_of(max_tokens, Bq, groups), nst = ns + window_blocks(win_len);
+    const int ns = fused_nsplit_capacity(max_tokens, Bq / groups), nst = ns + window_blocks(win_len);
     int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q, max_tokens, head_dim, Bq, groups,
                           workspace, workspace_bytes);
     if (rc != MSTF_OK) return rc;

@@ -29,6 +29,18 @@ static inline int fused_nsplit(int tokens, int bpw = 1)
     return (tokens / 64 + kFusedWaves * bpw - 1) / (kFusedWaves * bpw);
 }
 
+// Split slots that any token count up to `tokens` can need when the blocks per wavefront follow the count (a launch
+// sized once for a cache that grows): far fewer than one block per wavefront would take once the chip is full.
+static inline int fused_nsplit_capacity(int tokens, int Bkv)
+{
+    int ns = 1;
+    for (int n = 64; n <= tokens; n += 64) {
+        const int s = fused_nsplit(n, fused_blocks_per_wave(n, Bkv));
+        ns = s > ns ? s : ns;
+    }
+    return ns;
+}
+
 // Launches the merge of ns split slots per query row out of a workspace in the layout of the fused kernels
 // (defined beside the merge kernel).
 int merge_splits(hipStream_t st, const void* workspace, mstf_half* out, float* lse_out, int ns, int head_dim, int Bq);
