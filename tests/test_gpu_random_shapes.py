@@ -51,6 +51,16 @@ def test_random_case(seed):
         assert np.array_equal(c.bmp.cpu().numpy(), rb) and np.array_equal(c.idx.cpu().numpy(), ri)
         assert np.array_equal(c.nz_off.cpu().numpy(), roff) and int(c.total_halfs) == rnz.size
         assert np.array_equal(c.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+    # the same through the one-pass form (a value buffer given up front; 1, 2 or 4 units per workgroup by M / 64)
+    for x, xp, is_value, kth in ((K, Kp, 0, kth_k), (V, Vp, 1, kth_v)):
+        c1 = ops.compress(to_gpu(x), bool(is_value), kth=kth, capacity_halfs=x.size)
+        rb, ri, rnz, roff = orc.compress(xp, is_value)
+        assert np.array_equal(c1.bmp.cpu().numpy(), rb) and np.array_equal(c1.idx.cpu().numpy(), ri)
+        assert np.array_equal(c1.nz_off.cpu().numpy(), roff) and int(c1.total_halfs) == rnz.size
+        assert np.array_equal(c1.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+        c0 = ops.compress(to_gpu(xp), bool(is_value), kth=0, capacity_halfs=x.size)     # already pruned input
+        assert np.array_equal(c0.bmp.cpu().numpy(), rb) and np.array_equal(c0.idx.cpu().numpy(), ri)
+        assert np.array_equal(c0.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
     Bq = Bkv * groups
     q = rng.standard_normal((Bq, D)).astype(np.float16)
     s_ref, p_ref, o_ref = orc.dense_masked_attention(q, Kp, Vp, groups)
