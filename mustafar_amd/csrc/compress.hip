@@ -300,78 +300,6 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 // the dispatcher has started before it: every wait ends.  The waits are bounded all the same (kSpinLimit polls); a
 // workgroup that gives up sets the flag word behind the workgroup words, writes no values, and *total_halfs reads as
 // all ones.  onepass_init_kernel clears the words before the launch.
-constexpr uint32_t kSpinLimit = 1u << 20;  // default; the host passes the limit in (MSTF_COMPRESS_SPIN_LIMIT overrides it for tests)
-
-__global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n)
-{
-    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < n; i += (int)(gridDim.x * 256)) state[i] = 0ull;
-}
-
-__device__ __forceinline__ uint64_t agent_load(const uint64_t* p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void agent_store(uint64_t* p, uint64_t v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v)
-{
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-constexpr uint64_t kWordReady = 1ull << 63;
-
-// This wavefront's share of the wait for state[first .. g): the windows of 64 words number `wave`, wave + W, ...,
-// four of them in flight at a time.  Returns its part of the sums over [first, split) and [split, g)
-// (first <= split <= g); false when a wait ran out.
-template <int W>
-__device__ __forceinline__ bool wait_for_words(const uint64_t* state, int first, int split, int g, int wave, int lane,
-                                               uint32_t spin_limit, uint64_t& sum_lo, uint64_t& sum_hi)
-{
-    constexpr int K = 4;
-    uint64_t lo = 0, hi = 0;
-    uint32_t polls = 0;
-    bool ok = true;
-    for (int w0 = first + wave * 64; w0 < g && ok; w0 += 64 * W * K) {
-        uint64_t v[K];
-        bool got[K];
-#pragma unroll
-        for (int k = 0; k < K; k++) {
-            v[k] = 0ull;
-            got[k] = w0 + k * 64 * W + lane >= g;
-        }
-        for (;;) {
-            bool all = true;
-#pragma unroll
-            for (int k = 0; k < K; k++)
-                if (!got[k]) v[k] = agent_load(state + w0 + k * 64 * W + lane);
-#pragma unroll
-            for (int k = 0; k < K; k++) {
-                got[k] = got[k] || (v[k] >> 63) != 0ull;
-                all = all && got[k];
-            }
-            if (__ballot(!all) == 0ull) break;
-            if (++polls > spin_limit) {
-                ok = false;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-#pragma unroll
-        for (int k = 0; k < K; k++) {
-            const int i = w0 + k * 64 * W + lane;
-            const uint64_t t = v[k] & ~kWordReady;
-            lo += i < split ? t : 0ull;
-            hi += i >= split && i < g ? t : 0ull;
-        }
-    }
-    sum_lo = wave_sum_u64(lo);
-    sum_hi = wave_sum_u64(hi);
-    return ok;
-}
-
 // Compacts half h of a unit into the LDS image at img (tile offsets relative to the half's first tile).
 //   r     : this lane's token, raw fp16 pairs;  kept: its keep words (see select_kth_planes)
 //   key   : tile c = channel 64h + c over the 64 tokens - the lanes that keep the channel write at the tile's running

@@ -9,6 +9,8 @@
 #include "compress_common.hpp"
 #include "spmv_common.hpp"
 
+#include <cstdlib>
+
 namespace mstf {
 
 #pragma clang fp contract(off)
@@ -144,8 +146,7 @@ __global__ __launch_bounds__(256) void quant_scan_kernel(const uint32_t* __restr
     }
 }
 
-// tile_off[b][t] += head base + unit base  (global word offsets, as the reference returns them); only when no pack
-// follows, which does it itself.
+// tile_off[b][t] += head base + unit base  (global word offsets, as the reference returns them): the sizing-only call.
 __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restrict__ tile_off,
                                                              const uint32_t* __restrict__ unit_base,
                                                              const uint32_t* __restrict__ head_base, int nblk, size_t T)
@@ -156,59 +157,185 @@ __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restric
     tile_off[(size_t)b * T + t] += head_base[b] + unit_base[(size_t)b * nblk + t / kD];
 }
 
-// ------------------------------------------------------------------------------- producer: pack
-// grid = B * M/64 units, 64 threads; every lane quantises and packs its two tiles.  tile_off still holds the
-// unit-local offsets of the count kernel and is completed here with the unit's and the head's base.
-template <bool IS_VALUE, bool G32>
-__global__ __launch_bounds__(64) void quant_pack_kernel(const _Float16* __restrict__ x, int M, int bit,
-                                                        const uint64_t* __restrict__ bmp,
-                                                        const uint32_t* __restrict__ units, uint32_t* tile_off,
-                                                        const uint32_t* __restrict__ unit_base,
-                                                        const uint32_t* __restrict__ head_base,
-                                                        const _Float16* __restrict__ scales,
-                                                        const _Float16* __restrict__ zeros,
-                                                        uint32_t* __restrict__ packed, uint64_t capacity_words)
+// ------------------------------------------------------------------------------- producer: one pass
+// Everything with one read of the input, for the calls that produce the packed words: the count kernel's work on the
+// rows held in registers, the workgroup's word total published as a status word, the totals of the workgroups in
+// front of it added up (the one-pass ordering of the fp16 compressor, compress.hip), then the pack straight from
+// the registers - a half goes back into the LDS slab, and every lane quantises and packs its two tiles at their
+// final global word offsets.  grid = units / W workgroups of W wavefronts, W divides M / 64.
+// total_words reads as all ones when a wait ran out of its polls.
+template <bool IS_VALUE, bool G32, int W>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void quant_onepass_kernel(
+    const _Float16* __restrict__ x, int M, int kth, int bit, uint64_t* __restrict__ bmp, uint32_t* __restrict__ counts,
+    uint32_t* __restrict__ units, uint32_t* __restrict__ tile_off, _Float16* __restrict__ scales,
+    _Float16* __restrict__ zeros, uint32_t* __restrict__ packed, uint64_t capacity_words,
+    uint64_t* __restrict__ total_words, uint64_t* state, int nunits, int groups_total, uint32_t spin_limit)
 {
-    __shared__ uint32_t slab[kHalfSlabDw];
+    __shared__ uint32_t slabs[W][kHalfSlabDw];
+    __shared__ uint32_t wave_total[W];
+    __shared__ uint64_t bases[W][2];
     const int lane = lane_id();
+    const int wave = wave_id();
     const int nblk = M / 64;
-    const int unit = (int)blockIdx.x;
+    const int g = (int)blockIdx.x;
+    const int unit = g * W + wave;
     const int b = unit / nblk, tb = unit - b * nblk;
     const size_t T = (size_t)M * kD / 64;
+    uint32_t* slab = slabs[wave];
+    uint32_t r[64];  // this lane's token: 128 fp16 values
+    {
+        UnitRaw raw;
+        unit_fetch(x + (size_t)b * M * kD, (int64_t)tb * 64, lane, raw);
+        unit_rows_from(raw, slab, lane, r);
+    }
+    uint64_t bm[2];
+    uint32_t thr = 1u;
+    {
+        uint32_t kept[4];
+        if (kth > 0) {
+            thr = select_kth_planes<true>(r, kth, kept);  // the sign bits become planes the search never looks at
+            if (thr == 0u) thr = 1u;
+        } else {
+            kept_nonzero(r, kept);
+        }
+        if (IS_VALUE) {
+            bm[0] = spread_bitmap(kept[0], kept[1]);
+            bm[1] = spread_bitmap(kept[2], kept[3]);
+        } else {
+            key_bitmaps_from_kept(kept, lane, bm[0], bm[1]);
+        }
+    }
+    // pruned elements become NaN, which the minimum / maximum instructions pass over (see quant_count_kernel)
+    typedef short s2_t __attribute__((ext_vector_type(2)));
+    const us2_t t2 = as_us2(thr | (thr << 16));
+#pragma unroll
+    for (int j = 0; j < 64; j++) {
+        const s2_t d = __builtin_bit_cast(s2_t, (us2_t)(as_us2(r[j] & 0x7FFF7FFFu) - t2));   // < 0 <=> pruned
+        r[j] |= __builtin_bit_cast(uint32_t, (s2_t)(d >> 15)) & 0x7FFF7FFFu;
+    }
     const _Float16* sh = reinterpret_cast<const _Float16*>(slab);
+    const int cap = 32 / bit;
     const float maxq = (float)((1 << bit) - 1);
     const size_t tile0 = (size_t)b * T + (size_t)tb * kD;
-    const uint32_t ubase = head_base[b] + unit_base[(size_t)b * nblk + tb];
+    constexpr int NG = G32 ? 2 : 1;
+    uint32_t u[2];
+    float scg[2][NG], zpg[2][NG];  // the parameters as the consumers will read them: rounded to fp16
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        float mn[NG], mx[NG];
+        if (IS_VALUE) {
+            typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for (int gq = 0; gq < NG; gq++) {
+                h2v_t mn2 = {(_Float16)INFINITY, (_Float16)INFINITY}, mx2 = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+#pragma unroll
+                for (int j = gq * (32 / NG); j < (gq + 1) * (32 / NG); j++) {
+                    const h2v_t v = __builtin_bit_cast(h2v_t, r[32 * h + j]);
+                    mn2 = __builtin_elementwise_min(mn2, v);
+                    mx2 = __builtin_elementwise_max(mx2, v);
+                }
+                mn[gq] = fminf((float)mn2[0], (float)mn2[1]);
+                mx[gq] = fmaxf((float)mx2[0], (float)mx2[1]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int gq = 0; gq < NG; gq++) {
+                float a = INFINITY, z = -INFINITY;
+#pragma unroll 8
+                for (int i = gq * (64 / NG); i < (gq + 1) * (64 / NG); i++) {
+                    const float v = (float)sh[i * (2 * kHalfRowDw) + lane];
+                    a = fminf(a, v);
+                    z = fmaxf(z, v);
+                }
+                mn[gq] = a;
+                mx[gq] = z;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        const uint32_t cnt = (uint32_t)__popcll(bm[h]);
+        const size_t ti = tile0 + (size_t)h * 64 + lane;
+#pragma unroll
+        for (int gq = 0; gq < NG; gq++) {
+            float scale = 1.f, zero = 0.f;
+            if (mn[gq] <= mx[gq]) {
+                scale = (mx[gq] - mn[gq]) / maxq;
+                if (scale == 0.f) scale = 1.f;
+                zero = floorf(-mn[gq] / scale + 0.5f);
+            }
+            const _Float16 s16 = (_Float16)scale, z16 = (_Float16)zero;
+            scales[ti * NG + gq] = s16;
+            zeros[ti * NG + gq] = z16;
+            scg[h][gq] = (float)s16 == 0.f ? 1.f : (float)s16;
+            zpg[h][gq] = (float)z16;
+        }
+        bmp[ti] = bm[h];
+        counts[ti] = cnt;
+        u[h] = (cnt + (uint32_t)cap - 1u) / (uint32_t)cap;
+        units[ti] = u[h];
+    }
+    uint32_t totA, totB;
+    const uint32_t eA = wave_excl_scan(u[0], lane, totA);
+    const uint32_t eB = wave_excl_scan(u[1], lane, totB);
+    if (lane == 0) wave_total[wave] = totA + totB;
+    __syncthreads();
+    uint32_t in_group = 0, group_total = 0;
+#pragma unroll
+    for (int w = 0; w < W; w++) {
+        const uint32_t t = wave_total[w];
+        in_group += w < wave ? t : 0u;
+        group_total += t;
+    }
+    if (threadIdx.x == 0) agent_store(state + g, kWordReady | group_total);
+    {
+        uint64_t lo = 0, hi = 0;
+        const bool ok0 = wait_for_words<W>(state, 0, 0, g, wave, lane, spin_limit, lo, hi);
+        if (lane == 0) {
+            bases[wave][0] = hi;
+            bases[wave][1] = ok0 ? 1ull : 0ull;
+        }
+    }
+    __syncthreads();
+    uint64_t before = in_group;
+    bool ok = true;
+#pragma unroll
+    for (int w = 0; w < W; w++) {
+        before += bases[w][0];
+        ok = ok && bases[w][1] != 0ull;
+    }
+    if (!ok && threadIdx.x == 0) agent_store(state + groups_total, 1ull);
+    if (lane == 0 && unit == nunits - 1) *total_words = ok ? before + totA + totB : ~0ull;
+    const uint64_t off_h[2] = {before + eA, before + totA + eB};
+    tile_off[tile0 + lane] = (uint32_t)off_h[0];
+    tile_off[tile0 + 64 + lane] = (uint32_t)off_h[1];
+    if (!ok) return;
 #pragma unroll 1
     for (int h = 0; h < 2; h++) {
+        // the half back into the slab (the pruned elements are NaN there: the bitmap skips them)
         __builtin_amdgcn_wave_barrier();
-        half_slab_load(x + (size_t)b * M * kD, (int64_t)tb * 64, (int64_t)M, h, slab, lane);
-        __builtin_amdgcn_wave_barrier();
-        const size_t ti = tile0 + (size_t)h * 64 + lane;
-        const uint64_t m = bmp[ti];
-        const uint64_t off = (uint64_t)tile_off[ti] + ubase;
-        tile_off[ti] = (uint32_t)off;
-        if (off + units[ti] > capacity_words) continue;  // would not fit: leave untouched
-        constexpr int NG = G32 ? 2 : 1;
-        float scg[NG], zpg[NG];
+        if (h == 0) {
 #pragma unroll
-        for (int g = 0; g < NG; g++) {
-            scg[g] = (float)scales[ti * NG + g];
-            zpg[g] = (float)zeros[ti * NG + g];
-            if (scg[g] == 0.f) scg[g] = 1.f;
+            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 + j];
         }
+        __builtin_amdgcn_wave_barrier();
+        const uint64_t m = bm[h];
+        const uint64_t off = off_h[h];
+        if (off + u[h] > capacity_words) continue;  // would not fit: leave untouched
         uint32_t cur = 0;
         int pos = 0;
         uint32_t w = 0;
-        // only the kept elements, first to last: the wavefront loops as often as its fullest tile has non-zeros
-        // (about half of 64 at 70 % sparsity), and every round carries a division
         for (uint64_t rem = m; rem != 0ull;) {
             const int i = __builtin_clzll(rem);
             rem &= ~(0x8000000000000000ull >> i);
             const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
             const float v = (float)sh[e];
-            const float sc = (G32 && i >= 32) ? scg[NG - 1] : scg[0];   // the element's position picks the pair
-            const float zp = (G32 && i >= 32) ? zpg[NG - 1] : zpg[0];
+            const float sc = (G32 && i >= 32) ? scg[h][NG - 1] : scg[h][0];   // the element's position picks the pair
+            const float zp = (G32 && i >= 32) ? zpg[h][NG - 1] : zpg[h][0];
             float q = floorf(v / sc + 0.5f) + zp;
             q = fminf(fmaxf(q, 0.f), maxq);
             cur |= (uint32_t)q << pos;
@@ -237,7 +364,7 @@ static int cap_shift_of(int bit)
 // workspace: unit totals, unit bases (both [B][M/64]) and the head bases [B]
 static size_t quant_ws_bytes(int B, int M)
 {
-    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4, 256);
+    return 2 * round_up((size_t)B * (M / 64) * 4, 256) + round_up((size_t)B * 4 + 64, 256);  // also the one-pass status words
 }
 
 template <bool IS_VALUE, bool G32>
@@ -266,6 +393,31 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     uint32_t* head_base = reinterpret_cast<uint32_t*>(w + 2 * ub);
     const _Float16* xh = reinterpret_cast<const _Float16*>(x);
     int rc;
+    if (packed) {
+        const int units_all = B * nblk;
+        const int W = nblk % 4 == 0 ? 4 : (nblk % 2 == 0 ? 2 : 1);
+        const int groups = units_all / W;
+        uint64_t* state = reinterpret_cast<uint64_t*>(ws);
+        const int words = groups + 1;
+        const char* limit_env = getenv("MSTF_COMPRESS_SPIN_LIMIT");
+        const uint32_t spin_limit = limit_env ? (uint32_t)strtoul(limit_env, nullptr, 10) : kSpinLimit;
+        hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
+                           dim3(256), 0, st, state, words);
+        if ((rc = check_launch()) != MSTF_OK) return rc;
+#define MSTF_QOP(WV)                                                                                                  \
+    hipLaunchKernelGGL((quant_onepass_kernel<IS_VALUE, G32, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \
+                       bit, bmp, counts, units, tile_off, reinterpret_cast<_Float16*>(scales),                          \
+                       reinterpret_cast<_Float16*>(zeros), packed, cap_words, total_words, state, units_all, groups,    \
+                       spin_limit)
+        if (W == 4)
+            MSTF_QOP(4);
+        else if (W == 2)
+            MSTF_QOP(2);
+        else
+            MSTF_QOP(1);
+#undef MSTF_QOP
+        return check_launch();
+    }
     hipLaunchKernelGGL((quant_count_kernel<IS_VALUE, G32>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, kth, bit, bmp,
                        counts, units, tile_off, reinterpret_cast<_Float16*>(scales), reinterpret_cast<_Float16*>(zeros),
                        unit_tot);
@@ -273,14 +425,8 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     hipLaunchKernelGGL(quant_scan_kernel, dim3((unsigned)B), dim3(256), (size_t)nblk * 4, st, unit_tot, unit_base,
                        head_base, total_words, nblk);
     if ((rc = check_launch()) != MSTF_OK) return rc;
-    if (packed) {
-        hipLaunchKernelGGL((quant_pack_kernel<IS_VALUE, G32>), dim3((unsigned)(B * nblk)), dim3(64), 0, st, xh, M, bit, bmp,
-                           units, tile_off, unit_base, head_base, reinterpret_cast<const _Float16*>(scales),
-                           reinterpret_cast<const _Float16*>(zeros), packed, cap_words);
-    } else {
-        hipLaunchKernelGGL(quant_finalize_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)B), dim3(256), 0, st,
-                           tile_off, unit_base, head_base, nblk, T);
-    }
+    hipLaunchKernelGGL(quant_finalize_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)B), dim3(256), 0, st, tile_off,
+                       unit_base, head_base, nblk, T);
     if ((rc = check_launch()) != MSTF_OK) return rc;
     return MSTF_OK;
 }
