@@ -251,7 +251,8 @@ int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, c
  *   scales/zeros[B,T] fp16: scale = (max - min) / (2^bit - 1) (1 when 0 or empty),
  *   zero = floor(-min / scale + 0.5); code = clamp(floor(v / scale + 0.5) + zero, 0, 2^bit - 1);
  *   code j of a tile sits at bits bit*(j % capacity) of word j / capacity.
- * kth as in mstf_compress_*_f16.  packed == NULL runs the sizing phase only. */
+ * kth as in mstf_compress_*_f16.  packed == NULL runs the sizing phase only; with packed the input is read once and
+ * the workgroups are ordered as in mstf_compress_*_f16 (*total_words reads as all ones should a bounded wait run out). */
 size_t mstf_compress_quant_workspace_bytes(int B, int M, int N);
 int mstf_compress_key_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit, uint64_t* bmp,
                             uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,

@@ -45,6 +45,8 @@ def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
                                         scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,
                                         ws.data_ptr(), ws.numel()), name)
     n = int(total.item())
+    if n < 0:   # all ones: a workgroup of the one-pass producer gave up waiting (ruled out by the dispatch order)
+        raise RuntimeError("the quantised producer gave up waiting for an earlier workgroup; the packed words are incomplete")
     packed = room[:n].clone()
     return bmp, tile_off, packed, counts, units, scales, zeros
 
