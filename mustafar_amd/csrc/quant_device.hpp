@@ -3,6 +3,10 @@
 #pragma once
 #include "spmv_device.hpp"
 
+#ifndef MSTF_IMG_STRIDE
+#define MSTF_IMG_STRIDE 144
+#endif
+
 namespace mstf {
 
 #pragma clang fp contract(off)
@@ -17,7 +21,11 @@ struct QFmt {
     static constexpr int kWordsMax = kSubTiles * kSlots;        // words of a stage, every tile full
     static constexpr int kWordBuf = kWordsMax * 4 + 64;         // + room for the lanes past a tile's last word
 };
-constexpr int kImgBytes = kSubTiles * 128;   // fp16 image of a stage: 64 slots per tile
+// fp16 image of a stage: 64 two-byte slots per tile, the tiles kImgStride bytes apart.  128 would do; with 144 the
+// sixteen-byte writes of the lanes that dequantise different tiles at the same time (tiles 128 bytes apart start in
+// one of two banks) and the gathers spread over all LDS banks.
+constexpr int kImgStride = MSTF_IMG_STRIDE;
+constexpr int kImgBytes = kSubTiles * kImgStride;
 // Staged metadata of a stage.  One (scale, zero) pair per tile: 32 word offsets, 32 scales, 32 zero-points (256 bytes,
 // one LDS-direct load).  Two pairs per tile (G32: pair g for the elements 32g .. 32g+31): 32 word offsets, 32 x 2
 // scales, 32 x 2 zero-points and the upper halves of the 32 bitmaps (their popcount is the number of codes that
@@ -95,7 +103,7 @@ __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uin
             kb = kb < 0 ? 0 : (kb > F::kCap ? F::kCap : kb);
         }
         const uint32_t w = lds_load_u32(words + (off - start_word + slot) * 4u);
-        const uint32_t dst = img + tl * 128u + slot * (uint32_t)(F::kCap * 2);
+        const uint32_t dst = img + tl * (uint32_t)kImgStride + slot * (uint32_t)(F::kCap * 2);
         const bool small_zero = G32 ? ((zp & 0x7fffu) <= 0x6400u && ((zp >> 16) & 0x7fffu) <= 0x6400u)
                                     : ((zp & 0x7fffu) <= 0x6400u);
         if (small_zero) {
@@ -255,7 +263,7 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
 
 // Expands 8 tiles of the image and accumulates them, the gather under the tile's exec mask (see batch_step_exec in
 // spmv_device.hpp for the statement and the MFMA layout): one statement per batch of 8 tiles on fixed registers
-// v112-v127; the image slots of tile i sit at img + IMG + 128 * i, so the tile's
+// v112-v127; the image slots of tile i sit at img + IMG + kImgStride * i, so the tile's
 // base is an immediate offset of the LDS read.  PREFETCH: the bitmaps of the coming batch (bm + BOFF bytes) are
 // requested first and completed by the statement's wait.
 template <int NM, bool PREFETCH, int BOFF, int IMG, int WOFF>
@@ -290,8 +298,9 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
     [m0] "s"(u64_of(mv[0], mv[1])), [m1] "s"(u64_of(mv[2], mv[3])), [m2] "s"(u64_of(mv[4], mv[5])),                  \
         [m3] "s"(u64_of(mv[6], mv[7])), [m4] "s"(u64_of(mv[8], mv[9])), [m5] "s"(u64_of(mv[10], mv[11])),            \
         [m6] "s"(u64_of(mv[12], mv[13])), [m7] "s"(u64_of(mv[14], mv[15])), [img] "s"(img), [wa] "v"(wbase),         \
-        [woff] "i"(WOFF), [z] "v"(zaddr), [i0] "i"(IMG), [i1] "i"(IMG + 128), [i2] "i"(IMG + 256), [i3] "i"(IMG + 384), \
-        [i4] "i"(IMG + 512), [i5] "i"(IMG + 640), [i6] "i"(IMG + 768), [i7] "i"(IMG + 896)
+        [woff] "i"(WOFF), [z] "v"(zaddr), [i0] "i"(IMG), [i1] "i"(IMG + kImgStride), [i2] "i"(IMG + 2 * kImgStride),        \
+        [i3] "i"(IMG + 3 * kImgStride), [i4] "i"(IMG + 4 * kImgStride), [i5] "i"(IMG + 5 * kImgStride),                 \
+        [i6] "i"(IMG + 6 * kImgStride), [i7] "i"(IMG + 7 * kImgStride)
 #define MSTF_CLOBBER                                                                                                 \
     "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",  \
         "v126", "v127", "memory"
@@ -339,7 +348,7 @@ __device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t bm_l
     static_for<G>([&](auto gc) {
         constexpr int g = decltype(gc)::value;
         u32x16_t nxt;
-        batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 1024, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup, acc);
+        batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 8 * kImgStride, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup, acc);
         cur = nxt;
     });
 }
