@@ -68,13 +68,12 @@ __device__ __forceinline__ float wave_sum_same_column(float v)
 
 // Softmax statistics of one 64-token block from its scores; lane 4b+j holds tokens 4b..4b+3 of head 4m+j in acc_k[m].
 // Scores are rounded to fp16 and divided by sqrt(d) in fp16 (as the reference's glue does); the un-normalised
-// weights exp(w - max) go to LDS as fp16 rows of 64 tokens (the B operand of the value phase) and the block's
+// weights exp(w - max) go to LDS as fp16 rows of 64 tokens, kPRow bytes apart, (the B operand of the value phase) and the block's
 // (max, sum of the fp16 weights) stay in m_run / l_run.  Tokens >= nt (nt < 64 only in a partial block) get weight 0.
-template <int NM>
+template <int NM, int kPRow = 64 * 2>
 __device__ __forceinline__ void block_softmax(const f4_t (&acc_k)[NM], float sqrt_d, int nt, char* pl, int lane,
                                               float (&m_run)[NM], float (&l_run)[NM])
 {
-    constexpr int kPRow = 64 * 2;
     const int j = lane & 3;
 #pragma unroll
     for (int m = 0; m < NM; m++) {

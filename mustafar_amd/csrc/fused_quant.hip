@@ -6,6 +6,10 @@
 // tiles.  A stage's packed words and metadata arrive by LDS-direct loads one stage ahead (double buffers); the
 // stage is dequantised into the wavefront's fp16 tile image and expanded from there.
 #include "fused_common.hpp"
+
+#ifndef MSTF_QPAD
+#define MSTF_QPAD 16
+#endif
 #include "quant_device.hpp"
 
 namespace mstf {
@@ -34,8 +38,11 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
 {
     using F = QFmt<BIT>;
     constexpr int D = kFusedD;
-    constexpr int kQLds = NM * 4 * D * 2;
-    constexpr int kPRow = 64 * 2;
+    // query and weight rows sit 16 bytes further apart than their length: the four rows that the lanes of a group read
+    // together then start in different LDS banks
+    constexpr int kQRow = D * 2 + MSTF_QPAD;
+    constexpr int kQLds = NM * 4 * kQRow;
+    constexpr int kPRow = 64 * 2 + MSTF_QPAD;
     constexpr int kPLds = NM * 4 * kPRow;
     constexpr int kMetaBytes = meta_bytes<G32>();
     constexpr int kStage = q_lds_bytes<BIT, G32>();  // image, zero slot, two word buffers, two metadata buffers
@@ -120,11 +127,14 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         // the query rows of this KV head: groups x D fp16, contiguous
         {
             const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
-            const uint32_t qbytes = (uint32_t)groups * D * 2u;
+            // a row per load: sixteen lanes fetch the 256 bytes of query row `row`, four rows per pass
+            const int row_in_pass = lane >> 4;
 #pragma unroll
-            for (int i = 0; i < (kQLds + 1023) / 1024; i++) {
-                const uint32_t o = (uint32_t)(i * 64 + lane) * 16u;
-                if (o < qbytes) dma16(qsrc + o, ql + i * 1024);
+            for (int i = 0; i < NM; i++) {
+                const int row = i * 4 + row_in_pass;
+                const uint4 v = row < groups ? *reinterpret_cast<const uint4*>(qsrc + row * (D * 2) + (lane & 15) * 16)
+                                             : make_uint4(0u, 0u, 0u, 0u);
+                *reinterpret_cast<uint4*>(ql + row * kQRow + (lane & 15) * 16) = v;
             }
         }
         uint2 touch = issue(0);
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         f4_t acc_k[NM];
 #pragma unroll
         for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
-        const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
+        const uint32_t qrow = lds_addr(ql) + (uint32_t)j * kQRow;
         const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
 
         auto stage = [&](int n, uint2 bits, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
@@ -149,9 +159,9 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             const uint2 bits = touch;  // lane l < 32: bitmap l of stage n
             if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);
             if (n < kKeySubs) {
-                stage(n, bits, qrow + (uint32_t)n * kSubTiles * 2u, (uint32_t)D * 8u, acc_k);
+                stage(n, bits, qrow + (uint32_t)n * kSubTiles * 2u, 4u * kQRow, acc_k);
             } else {
-                if (n == kKeySubs) block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
+                if (n == kKeySubs) block_softmax<NM, kPRow>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
                 const int vs = n - kKeySubs;  // value stage: half = vs / 2, tokens (vs % 2) * 32..
                 constexpr int kSubsPerHalf = 64 / kSubTiles;
                 const int half = vs / kSubsPerHalf;
