@@ -239,6 +239,28 @@ def quant_record(torch, ops, dev, gen, bs, L, sparsity, bit, group_size, reps):
     def side_bytes(t):
         return sum(x.numel() * x.element_size() for x in (t[0], t[1], t[2], t[5], t[6]))
     kb, vb = side_bytes(sides[0][0]), side_bytes(sides[0][1])
+
+    # the producer on the pruned rows (what convert_*_batched_quant runs: kth = 0), outputs pre-allocated for the worst case
+    T = L * D // 64
+    Kp = ops.prune_rows(make_kv(torch, dev, Bkv, L, D, gen)[0].view(-1, D), kth).view(Bkv, L, D)
+    pshape = (Bkv, T) if group_size == 64 else (Bkv, T, 2)
+    pb = dict(bmp=torch.empty((Bkv, T), dtype=torch.int64, device=dev), off=torch.empty((Bkv, T), dtype=torch.int32, device=dev),
+              cnt=torch.empty((Bkv, T), dtype=torch.int32, device=dev), units=torch.empty((Bkv, T), dtype=torch.int32, device=dev),
+              sc=torch.empty(pshape, dtype=torch.float16, device=dev), zp=torch.empty(pshape, dtype=torch.float16, device=dev),
+              tot=torch.empty((1,), dtype=torch.int64, device=dev),
+              room=torch.empty((Bkv * T * (64 * bit // 32),), dtype=torch.int32, device=dev))
+    wsp = ws.get(Lh.mstf_compress_quant_workspace_bytes(Bkv, L, D))
+
+    def produce(is_value):
+        def run(i):
+            check(Lh.mstf_compress_quant_grouped(torch.cuda.current_stream().cuda_stream, Kp.data_ptr(), is_value, Bkv, L, D, 0,
+                                                 bit, group_size, pb["bmp"].data_ptr(), pb["off"].data_ptr(),
+                                                 pb["cnt"].data_ptr(), pb["units"].data_ptr(), pb["sc"].data_ptr(),
+                                                 pb["zp"].data_ptr(), pb["tot"].data_ptr(), pb["room"].data_ptr(),
+                                                 pb["room"].numel(), wsp.data_ptr(), wsp.numel()), "mstf_compress_quant_grouped")
+        return ring_time_us(torch, run, 2, reps)
+    prod_k, prod_v = produce(0), produce(1)
+    del Kp, pb
     key = ring_time_us(torch, qkey, n_caches, reps)
     val = ring_time_us(torch, qval, n_caches, reps)
     fused = ring_time_us(torch, lambda i: mpq.decode_attention_quant(sides[i][0], sides[i][1], q, g, bit, out=o, ws=ws),
@@ -246,6 +268,7 @@ def quant_record(torch, ops, dev, gen, bs, L, sparsity, bit, group_size, reps):
     alg = kb + vb + 2 * Bq * D * 2
     return {"batch": bs, "ctx": L, "sparsity": sparsity, "bit": bit, "group_size": group_size,
             "key_spmv_us": round(key, 2), "value_spmv_us": round(val, 2), "fused_step_us": round(fused, 2),
+            "producer_key_us": round(prod_k, 1), "producer_value_us": round(prod_v, 1),
             "key_spmv_gbs": round((kb + Bq * D * 2 + Bq * L * 2) / key / 1e3, 1),
             "value_spmv_gbs": round((vb + Bq * D * 2 + Bq * L * 2) / val / 1e3, 1),
             "fused_step_gbs": round(alg / fused / 1e3, 1), "fused_step_frac_of_peak": round(alg / fused / 1e3 / HBM_PEAK_GBS, 4),

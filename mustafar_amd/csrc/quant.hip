@@ -311,17 +311,12 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     tile_off[tile0 + lane] = (uint32_t)off_h[0];
     tile_off[tile0 + 64 + lane] = (uint32_t)off_h[1];
     if (!ok) return;
-#pragma unroll 1
-    for (int h = 0; h < 2; h++) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {  // unrolled: everything indexed by h stays in registers
         // the half back into the slab (the pruned elements are NaN there: the bitmap skips them)
         __builtin_amdgcn_wave_barrier();
-        if (h == 0) {
 #pragma unroll
-            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[j];
-        } else {
-#pragma unroll
-            for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 + j];
-        }
+        for (int j = 0; j < 32; j++) slab[lane * kHalfRowDw + j] = r[32 * h + j];
         __builtin_amdgcn_wave_barrier();
         const uint64_t m = bm[h];
         const uint64_t off = off_h[h];
@@ -329,11 +324,15 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
         uint32_t cur = 0;
         int pos = 0;
         uint32_t w = 0;
-        for (uint64_t rem = m; rem != 0ull;) {
-            const int i = __builtin_clzll(rem);
+        // the kept elements first to last; the coming element is read from LDS while the current one is quantised
+        auto at = [&](int i) { return (float)sh[IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane)]; };
+        uint64_t rem = m;
+        int i = rem != 0ull ? __builtin_clzll(rem) : 0;
+        float v = at(i);
+        while (rem != 0ull) {
             rem &= ~(0x8000000000000000ull >> i);
-            const int e = IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane);
-            const float v = (float)sh[e];
+            const int i_next = rem != 0ull ? __builtin_clzll(rem) : i;
+            const float v_next = at(i_next);
             const float sc = (G32 && i >= 32) ? scg[h][NG - 1] : scg[h][0];   // the element's position picks the pair
             const float zp = (G32 && i >= 32) ? zpg[h][NG - 1] : zpg[h][0];
             float q = floorf(v / sc + 0.5f) + zp;
@@ -345,6 +344,8 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
                 cur = 0;
                 pos = 0;
             }
+            v = v_next;
+            i = i_next;
         }
         if (pos > 0) packed[off + w] = cur;
     }
