@@ -324,7 +324,9 @@ __global__ __launch_bounds__(64) void window_attention_kernel(const _Float16* __
     // one array on purpose (LDS-direct loads into several LDS objects make the compiler serialise them)
     __shared__ __attribute__((aligned(16))) char lds[kKSlab + kVBlk + kZero + kQLds + kPLds];
     const int lane = lane_id();
-    const int blk = (int)blockIdx.x, kv = (int)blockIdx.y;
+    // heads vary fastest: the blocks beyond the valid length (a launch sized for the buffer) are dispatched last and do
+    // not stand in the queue in front of working ones
+    const int blk = (int)blockIdx.y, kv = (int)blockIdx.x;
     const int j = lane & 3;
     // the valid length may live in device memory (a captured graph replays with a growing window); the launch is
     // then sized for the buffer and a block beyond the window leaves a neutral triple
@@ -583,7 +585,7 @@ int mstf::window_launch(hipStream_t st, const mstf_half* k_win, const mstf_half*
     const _Float16* vw = reinterpret_cast<const _Float16*>(v_win);
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
     const float sq = sqrtf((float)head_dim);
-    const dim3 grid((unsigned)window_blocks(win_len), (unsigned)(Bq / groups));
+    const dim3 grid((unsigned)(Bq / groups), (unsigned)window_blocks(win_len));
     if (groups <= 4)
         hipLaunchKernelGGL(window_attention_kernel<1>, grid, dim3(64), 0, st, kw, vw, qh, part_o, part_ml, win_len,
                            win_len_dev, win_stride, groups, nst, split0, sq);
