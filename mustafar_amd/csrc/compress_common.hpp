@@ -403,7 +403,7 @@ __device__ __forceinline__ uint32_t threshold_of(const uint32_t (&mag)[64], int 
 
 // Threshold and tile bitmaps of one unit in one go (see unit_bitmaps for the meaning of bmA / bmB).  With pruning
 // (kth > 0) the bitmaps come from the select's own keep masks, so the magnitudes are dead once the bit planes exist:
-// value tiles spread the masks into channel order, key tiles take one ballot per channel over the lanes' mask bits.
+// value tiles spread the masks into channel order, key tiles transpose the lanes' masks across the wavefront.
 // Returns the row's threshold: an element is kept <=> its magnitude is >= the returned value (>= 1: zeros never are).
 template <bool IS_VALUE>
 __device__ __forceinline__ uint32_t unit_keep(const uint32_t (&mag)[64], int kth, int lane, uint64_t& bmA, uint64_t& bmB)
@@ -415,21 +415,7 @@ __device__ __forceinline__ uint32_t unit_keep(const uint32_t (&mag)[64], int kth
             bmA = spread_bitmap(kept[0], kept[1]);
             bmB = spread_bitmap(kept[2], kept[3]);
         } else {
-            uint32_t aLo = 0u, aHi = 0u, bLo = 0u, bHi = 0u;
-#pragma unroll
-            for (int c = 0; c < 128; c++) {
-                const uint32_t bit = 1u << ((c & 63) >> 1);
-                const uint64_t k = __builtin_bitreverse64(__ballot((kept[2 * (c >> 6) + (c & 1)] & bit) != 0u));
-                if (c < 64) {
-                    aLo = write_lane((uint32_t)k, c, aLo);
-                    aHi = write_lane((uint32_t)(k >> 32), c, aHi);
-                } else {
-                    bLo = write_lane((uint32_t)k, c - 64, bLo);
-                    bHi = write_lane((uint32_t)(k >> 32), c - 64, bHi);
-                }
-            }
-            bmA = u64_of(aLo, aHi);
-            bmB = u64_of(bLo, bHi);
+            key_bitmaps_from_kept(kept, lane, bmA, bmB);
         }
         return thr == 0u ? 1u : thr;
     }
