@@ -243,6 +243,29 @@ int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, c
                                           int max_tokens, const int32_t* tokens_dev, int64_t tile_capacity, int head_dim,
                                           int Bq, int groups, void* workspace, size_t workspace_bytes);
 
+/* The caller's per-token work in front of the attention call, in one launch (models/llama_mustafar_kernel.py:363-374:
+ * the views of the projection outputs and apply_rotary_pos_emb; :391, :430: torch.cat of the new key / value row onto
+ * the local windows):
+ *   q_out[b * n_q + h, :]                    = rope(q_in[b, h, :])        (what the attention entry points take as q)
+ *   k_win[b * n_kv + h, row, :]              = rope(k_in[b, h, :])
+ *   v_win[b * n_kv + h, row, :]              = v_in[b, h, :]
+ * with rope(x) = x * cos + rotate_half(x) * sin in fp16, every product and the sum rounded on its own (the arithmetic
+ * of the half-precision expression), rotate_half(x) = [-x[64:], x[:64]].
+ * q_in [bs][n_q * 128], k_in / v_in [bs][n_kv * 128] fp16: the projection outputs of the new token, *_stride halfs
+ * between two batch entries (three slices of one fused projection are fine); cos, sin [bs][128] fp16 for the token's
+ * position, rope_stride halfs between batch entries (0: one position for all), both NULL: no rotation.  q_in and
+ * q_out both NULL: keys and values only.
+ * k_win, v_win [bs * n_kv][win_stride][128] as for mstf_decode_attention_window_f16.  win_len counts the valid rows of
+ * the window AFTER this call, the new token included - the same number the attention call takes - and row =
+ * win_len - 1; with win_len_dev the count is read from device memory instead (a call recorded into a HIP graph
+ * replays with the counter the caller advances between or inside the replays).  A count outside 1 .. win_stride
+ * writes no key / value row and sets *overflow (nullable, sticky) to 1. */
+int mstf_window_append_f16(void* stream, const mstf_half* q_in, int64_t q_stride, const mstf_half* k_in,
+                           int64_t k_stride, const mstf_half* v_in, int64_t v_stride, int bs, int n_q, int n_kv,
+                           int head_dim, const mstf_half* cos, const mstf_half* sin, int64_t rope_stride,
+                           mstf_half* q_out, mstf_half* k_win, mstf_half* v_win, int win_stride, int win_len,
+                           const int32_t* win_len_dev, uint32_t* overflow);
+
 /* ------------------------------------------------------------------ quantised format (Q1-Q4)
  * Producer: convert_{key,value}_batched_quant (kernel_quant/compression_quant.py:159-264, 425-529),
  * with the bit width a parameter (the reference hard-codes 2).  Same tiles and bitmaps as above;

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmustafar_hip.so")
-SOURCES = ["runtime.hip", "spmv.hip", "compress.hip", "quant.hip", "quant_spmv.hip", "fused.hip", "fused_quant.hip"]
+SOURCES = ["runtime.hip", "spmv.hip", "compress.hip", "quant.hip", "quant_spmv.hip", "fused.hip", "fused_quant.hip", "window_append.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are kept out of the generated code on purpose

@@ -266,8 +266,9 @@ class SparseKVCache:
             self._kbuf = torch.empty((bs * n_kv, cap, D), dtype=torch.float16, device=K.device)
             self._vbuf = torch.empty_like(self._kbuf)
             self._wlen = L - Lc
-            self._widx = torch.full((1,), self._wlen, dtype=torch.int64, device=K.device)       # next free row
             self._wlen_dev = torch.full((1,), self._wlen, dtype=torch.int32, device=K.device)   # valid rows
+            self._owns_clock, self._clock_shared = True, False
+            self._wovf = torch.zeros((1,), dtype=torch.int32, device=K.device)   # set by an append past the buffer
             self._kbuf[:, :self._wlen] = K[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
             self._vbuf[:, :self._wlen] = V[:, :, Lc:].reshape(bs * n_kv, self._wlen, D)
             self._shape = (bs, n_kv, D)
@@ -281,17 +282,38 @@ class SparseKVCache:
         self.k_win = self._kbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
         self.v_win = self._vbuf[:, :self._wlen].view(bs, n_kv, self._wlen, D)
 
+    def share_clock(self, other):
+        """Caches that advance in lockstep (the layers of one model) can read the window length from one device
+        counter: this cache takes `other`'s and no longer advances it - the owner's decode_device does, once per step,
+        before any of the sharers runs."""
+        self._wlen_dev = other._wlen_dev
+        self._owns_clock = False
+        other._clock_shared = True
+
     def decode_device(self, q, k_new, v_new):
         """The device work of a decode step in window_kernel mode: append the token to the window, attend.  Only
         device memory changes (the window length is a device counter), so the call can be captured in a HIP graph and
         replayed; the host-side bookkeeping of the step is advance()."""
         bs, n_q, _, D = q.shape
         n_kv = self._shape[1]
-        self._kbuf.index_copy_(1, self._widx, k_new.reshape(bs * n_kv, 1, D))
-        self._vbuf.index_copy_(1, self._widx, v_new.reshape(bs * n_kv, 1, D))
-        self._widx += 1
-        self._wlen_dev += 1
+        if self._owns_clock:
+            self._wlen_dev += 1
+        ops.window_append(k_new.reshape(bs, n_kv * D), v_new.reshape(bs, n_kv * D), self._kbuf, self._vbuf,
+                          self._wlen + 1, win_len_dev=self._wlen_dev, overflow=self._wovf)
         return self._attend_device(q.reshape(bs * n_q, D).contiguous()).view(bs, n_q, 1, D)
+
+    def decode_device_proj(self, q_in, k_in, v_in, cos, sin):
+        """decode_device straight from the projection outputs of the new token, q_in [bs, n_q * D], k_in / v_in
+        [bs, n_kv * D] (slices of one fused projection are fine), not yet rotated: rotation of query and key heads
+        with cos, sin [D] or [bs, D] (sin itself, for rotate_half), the append to the window and the query layout are
+        one launch (ops.window_append) in front of the attention.  Returns [bs, n_q, 1, D]."""
+        bs, D = q_in.shape[0], self._shape[2]
+        n_q = q_in.shape[1] // D
+        if self._owns_clock:
+            self._wlen_dev += 1
+        q2 = ops.window_append(k_in, v_in, self._kbuf, self._vbuf, self._wlen + 1, q_in=q_in, cos=cos, sin=sin,
+                               win_len_dev=self._wlen_dev, overflow=self._wovf)
+        return self._attend_device(q2).view(bs, n_q, 1, D)
 
     def _attend_device(self, q2):
         """Attention of the query rows q2 [Bq, D] over [compressed | window buffer] (three launches)."""
@@ -315,8 +337,9 @@ class SparseKVCache:
             rest = self._wlen - CHUNK
             self._kbuf[:, :rest] = self._kbuf[:, CHUNK:self._wlen].clone()
             self._vbuf[:, :rest] = self._vbuf[:, CHUNK:self._wlen].clone()
+            if int(self._wovf.item()) != 0:
+                raise RuntimeError("a token was appended past the end of the window buffer")
             self._wlen = rest
-            self._widx.fill_(rest)
             self._wlen_dev.fill_(rest)
             self.compressed_length += CHUNK
             grew = self.k_pool is None
@@ -324,6 +347,9 @@ class SparseKVCache:
         return grew
 
     def _decode_window_kernel(self, q, k_new, v_new):
+        if not self._owns_clock or self._clock_shared:
+            raise RuntimeError("caches that share a window counter advance together: decode_device on every cache, "
+                               "then advance on every cache")
         out = self.decode_device(q, k_new, v_new)
         self.advance()
         return out

@@ -199,17 +199,29 @@ class Decoder:
         pos = torch.tensor([position], device=self.dev)
         return self._layers(ids, pos, timed, lambda cache, q, k, v: cache.decode(q, k, v))
 
-    def _layers(self, ids, pos, timed, attend):
+    def _layers(self, ids, pos, timed, attend, from_proj=False):
+        """from_proj: the cache takes the new token's projection output as it is (decode_device_proj: rotation, window
+        append and query layout in one launch); otherwise q, k, v are rotated here and handed over as tensors."""
         c = self.cfg
         tables = list(_rope_tables(pos, c.head_dim, c.rope_theta, torch.float16))   # once per step, shared by the layers
+        if from_proj:
+            half, nq, nk = c.head_dim // 2, c.n_q * c.head_dim, c.n_kv * c.head_dim
+            cos = tables[0]
+            usin = torch.cat([-tables[1][:, :half], tables[1][:, half:]], -1)   # sin itself, for rotate_half
         x = self.embed[ids]
         for lw, cache in zip(self.layers, self.caches):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            q, k, v = self._qkv(lw, h, tables)
+            if from_proj:
+                qkv = F.linear(h, lw["qkv"]).view(x.shape[0], -1)
+            else:
+                q, k, v = self._qkv(lw, h, tables)
             if timed:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            a = attend(cache, q.contiguous(), k, v)
+            if from_proj:
+                a = cache.decode_device_proj(qkv[:, :nq], qkv[:, nq: nq + nk], qkv[:, nq + nk:], cos, usin)
+            else:
+                a = attend(cache, q.contiguous(), k, v)
             if timed:
                 e1.record()
                 self.attn_events.append((e0, e1))
@@ -233,10 +245,13 @@ class GraphedGreedyLoop:
         self.pos = torch.tensor([position], device=dec.dev)
         self.graph = None
         self.captures = 0
+        # the layers' windows grow in lockstep: one device counter, advanced by the first layer's cache
+        for cache in dec.caches[1:]:
+            cache.share_clock(dec.caches[0])
 
     @torch.no_grad()
     def _device_step(self):
-        logits = self.dec._layers(self.ids, self.pos, False, lambda cache, q, k, v: cache.decode_device(q, k, v))
+        logits = self.dec._layers(self.ids, self.pos, False, None, from_proj=True)
         self.ids.copy_(logits[:, -1].argmax(-1, keepdim=True))
         self.pos += 1
 

@@ -300,6 +300,44 @@ def decode_attention_window_pool(k_pool, v_pool, q, k_win, v_win, win_len, group
     return o
 
 
+def window_append(k_in, v_in, k_win, v_win, win_len, q_in=None, cos=None, sin=None, q_out=None, win_len_dev=None,
+                  overflow=None):
+    """The per-token work in front of the attention call in one launch (models/llama_mustafar_kernel.py:363-374, 391,
+    430): q_in [bs, n_q * D], k_in / v_in [bs, n_kv * D] fp16 are the projection outputs of the new token (views with
+    a batch stride are fine); query and key heads are rotated with cos, sin [D] or [bs, D] (None: no rotation), the
+    query rows returned as [bs * n_q, D], key and value rows written to row win_len - 1 of the window buffers
+    k_win, v_win [bs * n_kv, win_stride, D].  win_len counts the valid rows after the call, the new token included;
+    with win_len_dev (int32 tensor) the count is read on the device.  Returns q_out (None without q_in)."""
+    D = k_win.shape[-1]
+    bs = k_in.shape[0]
+    n_kv = k_in.shape[-1] // D
+    for t in (k_in, v_in) + ((q_in,) if q_in is not None else ()):
+        assert t.dtype == torch.float16 and t.dim() == 2 and t.stride(1) == 1 and t.shape[0] == bs
+    assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
+    assert k_win.shape[0] == bs * n_kv and v_in.shape[-1] == n_kv * D
+    n_q = 0
+    if q_in is not None:
+        n_q = q_in.shape[-1] // D
+        if q_out is None:
+            q_out = torch.empty((bs * n_q, D), dtype=torch.float16, device=q_in.device)
+        assert q_out.dtype == torch.float16 and q_out.is_contiguous() and q_out.numel() == bs * n_q * D
+    rope_stride = 0
+    if cos is not None:
+        assert cos.dtype == torch.float16 and sin.dtype == torch.float16 and cos.shape == sin.shape
+        assert cos.shape[-1] == D and cos.stride(-1) == 1 and sin.stride(-1) == 1
+        if cos.dim() == 2 and cos.shape[0] > 1:
+            assert cos.shape[0] == bs and cos.stride(0) == sin.stride(0)
+            rope_stride = cos.stride(0)
+    check(lib().mstf_window_append_f16(
+        _stream(), q_in.data_ptr() if q_in is not None else None, q_in.stride(0) if q_in is not None else 0,
+        k_in.data_ptr(), k_in.stride(0), v_in.data_ptr(), v_in.stride(0), bs, n_q, n_kv, D,
+        cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, rope_stride,
+        q_out.data_ptr() if q_out is not None else None, k_win.data_ptr(), v_win.data_ptr(), k_win.shape[1], int(win_len),
+        win_len_dev.data_ptr() if win_len_dev is not None else None, overflow.data_ptr() if overflow is not None else None),
+        "mstf_window_append_f16")
+    return q_out
+
+
 def decode_attention_partial(ck, cv, q, groups, ws=None):
     """First phase of decode_attention: un-normalised outputs and (max, sum) per 512-token split, left in `ws`."""
     assert q.dtype == torch.float16 and q.is_contiguous()

@@ -189,3 +189,51 @@ def test_workspaces_are_owned_and_do_not_move_under_capture():
     cache_a = SparseKVCache(4, max_tokens=512, window_kernel=True)
     cache_b = SparseKVCache(4, max_tokens=512, window_kernel=True)
     assert cache_a._workspace(dev) is not cache_b._workspace(dev)
+
+
+@pytest.mark.parametrize("per_entry_positions,counter_on_device", [(False, True), (True, False)])
+def test_window_append_rotates_and_appends_the_new_token(per_entry_positions, counter_on_device):
+    """mstf_window_append_f16 against the oracle's apply_rotary_pos_emb restatement and a plain row write: rotated
+    query rows in the attention's layout, rotated key row and value row at row win_len - 1 of the window buffers,
+    every other row untouched - bit for bit; inputs are the three slices of one fused projection output."""
+    from mustafar_amd import ops
+    dev = torch.device("cuda:0")
+    bs, n_q, n_kv, D, stride, wlen = 3, 8, 2, 128, 40, 17
+    rng = np.random.default_rng(11)
+    H = n_q + 2 * n_kv
+    proj = rng.standard_normal((bs, H * D)).astype(np.float16)
+    pos = rng.integers(0, 9000, size=bs) if per_entry_positions else np.full(bs, 4242)
+    cos, sin = orc.rope_tables(pos)                                   # [bs, D]
+    kwin0 = rng.standard_normal((bs * n_kv, stride, D)).astype(np.float16)
+    vwin0 = rng.standard_normal((bs * n_kv, stride, D)).astype(np.float16)
+    pt = torch.from_numpy(proj).to(dev)
+    kw, vw = torch.from_numpy(kwin0).to(dev), torch.from_numpy(vwin0).to(dev)
+    ct = torch.from_numpy(cos if per_entry_positions else cos[0]).to(dev)
+    st = torch.from_numpy(sin if per_entry_positions else sin[0]).to(dev)
+    counter = torch.full((1,), wlen, dtype=torch.int32, device=dev) if counter_on_device else None
+    ovf = torch.zeros((1,), dtype=torch.int32, device=dev)
+    q2 = ops.window_append(pt[:, n_q * D: (n_q + n_kv) * D], pt[:, (n_q + n_kv) * D:], kw, vw,
+                           stride if counter_on_device else wlen, q_in=pt[:, : n_q * D], cos=ct, sin=st,
+                           win_len_dev=counter, overflow=ovf)
+    x = proj.reshape(bs, H, 1, D)
+    rot = orc.rope_rows(x[:, : n_q + n_kv], cos[:, None, None, :], sin[:, None, None, :])
+    assert np.array_equal(q2.cpu().numpy().view(np.int16), rot[:, :n_q].reshape(bs * n_q, D).view(np.int16))
+    kexp, vexp = kwin0.copy(), vwin0.copy()
+    kexp[:, wlen - 1] = rot[:, n_q:].reshape(bs * n_kv, D)
+    vexp[:, wlen - 1] = x[:, n_q + n_kv:].reshape(bs * n_kv, D)
+    assert np.array_equal(kw.cpu().numpy().view(np.int16), kexp.view(np.int16))
+    assert np.array_equal(vw.cpu().numpy().view(np.int16), vexp.view(np.int16))
+    assert int(ovf.item()) == 0
+    # keys and values only, no rotation; then a count past the buffer: nothing written, flag set
+    ops.window_append(pt[:, :n_kv * D], pt[:, n_kv * D: 2 * n_kv * D], kw, vw, wlen + 1)
+    kexp[:, wlen] = proj[:, :n_kv * D].reshape(bs * n_kv, D)
+    vexp[:, wlen] = proj[:, n_kv * D: 2 * n_kv * D].reshape(bs * n_kv, D)
+    assert np.array_equal(kw.cpu().numpy().view(np.int16), kexp.view(np.int16))
+    assert np.array_equal(vw.cpu().numpy().view(np.int16), vexp.view(np.int16))
+    big = torch.full((1,), stride + 1, dtype=torch.int32, device=dev)
+    ops.window_append(pt[:, :n_kv * D], pt[:, n_kv * D: 2 * n_kv * D], kw, vw, stride, win_len_dev=big, overflow=ovf)
+    assert int(ovf.item()) == 1
+    assert np.array_equal(kw.cpu().numpy().view(np.int16), kexp.view(np.int16))
+    assert np.array_equal(vw.cpu().numpy().view(np.int16), vexp.view(np.int16))
+    with pytest.raises(RuntimeError):
+        ops.window_append(pt[:, :n_kv * D], pt[:, n_kv * D: 2 * n_kv * D], kw, vw, stride + 1)   # host count past the buffer
