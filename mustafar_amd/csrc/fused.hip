@@ -27,7 +27,7 @@ namespace mstf {
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
 template <int NM, bool MULTI>
-__global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(4))) void decode_attention_kernel(
+__global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(MSTF_FUSED_OCCUPANCY))) void decode_attention_kernel(
     const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,

@@ -11,7 +11,12 @@ constexpr int kFusedWaves = 8;    // token blocks (= wavefronts) per workgroup: 
 constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
 constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
 
-constexpr int kFusedResident = 4096;  // wavefronts of the fused kernel the 256 CUs hold at once (16 per CU)
+// Wavefronts per SIMD the fused fp16 kernel is built for: its LDS footprint (two stage buffers of kSubTiles tiles) and
+// its register budget (MSTF_GATHER_TOP) have to allow it.
+#ifndef MSTF_FUSED_OCCUPANCY
+#define MSTF_FUSED_OCCUPANCY 4
+#endif
+constexpr int kFusedResident = 1024 * MSTF_FUSED_OCCUPANCY;  // wavefronts of the fused kernel the 256 CUs hold at once
 constexpr int kFusedMaxBpw = 8;
 
 // Token blocks one wavefront of the fp16 kernel walks: 1 while every block can have a resident wavefront of its

@@ -263,7 +263,7 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
 
 // Expands 8 tiles of the image and accumulates them, the gather under the tile's exec mask (see batch_step_exec in
 // spmv_device.hpp for the statement and the MFMA layout): one statement per batch of 8 tiles on fixed registers
-// v112-v127; the image slots of tile i sit at img + IMG + kImgStride * i, so the tile's
+// (MSTF_GV0 .. 15 of spmv_device.hpp); the image slots of tile i sit at img + IMG + kImgStride * i, so the tile's
 // base is an immediate offset of the LDS read.  PREFETCH: the bitmaps of the coming batch (bm + BOFF bytes) are
 // requested first and completed by the statement's wait.
 template <int NM, bool PREFETCH, int BOFF, int IMG, int WOFF>
@@ -277,23 +277,23 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
     uint64_t sv;  // exec as found, handed back
 #define MSTF_TILE(I, H, A)                                       \
     "s_brev_b64 exec, %[m" #I "]\n\t"                            \
-    "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
-    "v_mbcnt_hi_u32_b32 v" #A ", exec_hi, v" #A "\n\t"           \
-    "v_lshl_add_u32 v" #A ", v" #A ", 1, %[img]\n\t"             \
-    "ds_read_u16 v" #H ", v" #A " offset:%[i" #I "]\n\t"
+    "v_mbcnt_lo_u32_b32 " A ", exec_lo, 0\n\t"                   \
+    "v_mbcnt_hi_u32_b32 " A ", exec_hi, " A "\n\t"               \
+    "v_lshl_add_u32 " A ", " A ", 1, %[img]\n\t"                 \
+    "ds_read_u16 " H ", " A " offset:%[i" #I "]\n\t"
 #define MSTF_GATHER                                                                                  \
     "s_mov_b64 %[sv], exec\n\t"                                                                      \
     "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                   \
-    "ds_read_b128 v[112:115], %[z]\n\t"                                                              \
-    "ds_read_b128 v[116:119], %[z]\n\t"                                                              \
-    MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)      \
-    MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)      \
+    "ds_read_b128 " MSTF_GV0_3 ", %[z]\n\t"                                                                  \
+    "ds_read_b128 " MSTF_GV4_7 ", %[z]\n\t"                                                                  \
+    MSTF_TILE(0, MSTF_GV0, MSTF_GV8) MSTF_TILE(1, MSTF_GV1, MSTF_GV9) MSTF_TILE(2, MSTF_GV2, MSTF_GV10) MSTF_TILE(3, MSTF_GV3, MSTF_GV11)      \
+    MSTF_TILE(4, MSTF_GV4, MSTF_GV12) MSTF_TILE(5, MSTF_GV5, MSTF_GV13) MSTF_TILE(6, MSTF_GV6, MSTF_GV14) MSTF_TILE(7, MSTF_GV7, MSTF_GV15)      \
     "s_mov_b64 exec, %[sv]\n\t"                                                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                       \
-    "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                        \
-    "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                        \
-    "v_lshl_or_b32 %[v2], v117, 16, v116\n\t"                                                        \
-    "v_lshl_or_b32 %[v3], v119, 16, v118"
+    "v_lshl_or_b32 %[v0], " MSTF_GV1 ", 16, " MSTF_GV0 "\n\t"                                                        \
+    "v_lshl_or_b32 %[v1], " MSTF_GV3 ", 16, " MSTF_GV2 "\n\t"                                                        \
+    "v_lshl_or_b32 %[v2], " MSTF_GV5 ", 16, " MSTF_GV4 "\n\t"                                                        \
+    "v_lshl_or_b32 %[v3], " MSTF_GV7 ", 16, " MSTF_GV6
 #define MSTF_IN                                                                                                      \
     [m0] "s"(u64_of(mv[0], mv[1])), [m1] "s"(u64_of(mv[2], mv[3])), [m2] "s"(u64_of(mv[4], mv[5])),                  \
         [m3] "s"(u64_of(mv[6], mv[7])), [m4] "s"(u64_of(mv[8], mv[9])), [m5] "s"(u64_of(mv[10], mv[11])),            \
@@ -302,8 +302,7 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
         [i3] "i"(IMG + 3 * kImgStride), [i4] "i"(IMG + 4 * kImgStride), [i5] "i"(IMG + 5 * kImgStride),                 \
         [i6] "i"(IMG + 6 * kImgStride), [i7] "i"(IMG + 7 * kImgStride)
 #define MSTF_CLOBBER                                                                                                 \
-    "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",  \
-        "v126", "v127", "memory"
+    MSTF_GV_CLOBBER, "memory"
     if constexpr (PREFETCH) {
         asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t" MSTF_GATHER
                      : [v0] "=&v"(v0), [v1] "=&v"(v1), [v2] "=&v"(v2), [v3] "=&v"(v3), [qm] "=&v"(qm[0]), [sv] "=&s"(sv),

@@ -15,6 +15,57 @@ constexpr int kNzLds = 2 * kSubBytes + 16;     // value double buffer + zero slo
 
 #define MSTF_GLOBAL __attribute__((address_space(1)))
 
+// The sixteen fixed vector registers of the gather statements (batch_step_exec and its quantised counterpart): the top
+// of the register budget the kernels are built for - 128 registers with four wavefronts per SIMD, 80 with six.
+// MSTF_GV(k): register k as a string, MSTF_GV0_3 / MSTF_GV4_7: the two aligned quads the zero reads fill.
+#ifndef MSTF_GATHER_TOP
+#define MSTF_GATHER_TOP 128
+#endif
+#if MSTF_GATHER_TOP == 128
+#define MSTF_GV0 "v112"
+#define MSTF_GV1 "v113"
+#define MSTF_GV2 "v114"
+#define MSTF_GV3 "v115"
+#define MSTF_GV4 "v116"
+#define MSTF_GV5 "v117"
+#define MSTF_GV6 "v118"
+#define MSTF_GV7 "v119"
+#define MSTF_GV8 "v120"
+#define MSTF_GV9 "v121"
+#define MSTF_GV10 "v122"
+#define MSTF_GV11 "v123"
+#define MSTF_GV12 "v124"
+#define MSTF_GV13 "v125"
+#define MSTF_GV14 "v126"
+#define MSTF_GV15 "v127"
+#define MSTF_GV0_3 "v[112:115]"
+#define MSTF_GV4_7 "v[116:119]"
+#elif MSTF_GATHER_TOP == 80
+#define MSTF_GV0 "v64"
+#define MSTF_GV1 "v65"
+#define MSTF_GV2 "v66"
+#define MSTF_GV3 "v67"
+#define MSTF_GV4 "v68"
+#define MSTF_GV5 "v69"
+#define MSTF_GV6 "v70"
+#define MSTF_GV7 "v71"
+#define MSTF_GV8 "v72"
+#define MSTF_GV9 "v73"
+#define MSTF_GV10 "v74"
+#define MSTF_GV11 "v75"
+#define MSTF_GV12 "v76"
+#define MSTF_GV13 "v77"
+#define MSTF_GV14 "v78"
+#define MSTF_GV15 "v79"
+#define MSTF_GV0_3 "v[64:67]"
+#define MSTF_GV4_7 "v[68:71]"
+#else
+#error "MSTF_GATHER_TOP: 128 or 80"
+#endif
+#define MSTF_GV_CLOBBER                                                                                            \
+    MSTF_GV0, MSTF_GV1, MSTF_GV2, MSTF_GV3, MSTF_GV4, MSTF_GV5, MSTF_GV6, MSTF_GV7, MSTF_GV8, MSTF_GV9, MSTF_GV10, \
+        MSTF_GV11, MSTF_GV12, MSTF_GV13, MSTF_GV14, MSTF_GV15
+
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ h4_t as_h4(uint32_t lo, uint32_t hi)
@@ -66,7 +117,7 @@ struct Batch {
 // present compute a rank and read LDS, the others keep the zero their destination was cleared to (four destinations
 // per 16-byte LDS read of the zero slot at zaddr; LDS reads of a wavefront return in order, so the gathers land on
 // top), so the select instruction disappears - per tile one s_brev_b64 into exec, two v_mbcnt on exec, the
-// scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (v112-v127, the top of the
+// scalar base, one v_lshl_add and the LDS read.  It is one statement on fixed registers (MSTF_GV0 .. 15: v112-v127, the top of the
 // budget of a kernel that runs four wavefronts per SIMD, listed as clobbered) because nothing of the compiler's may
 // be scheduled while exec is partial.  The statement saves the exec mask it is entered with and hands it back, but
 // between the two every tile runs under its own bitmap: callers sit in wave-uniform control flow with all 64 lanes
@@ -88,24 +139,24 @@ __device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, cons
     uint64_t sv;  // the exec mask the statement was entered with, handed back at its end
 #define MSTF_TILE(I, H, A)                                       \
     "s_brev_b64 exec, %[m" #I "]\n\t"                            \
-    "v_mbcnt_lo_u32_b32 v" #A ", exec_lo, 0\n\t"                 \
-    "v_mbcnt_hi_u32_b32 v" #A ", exec_hi, v" #A "\n\t"           \
+    "v_mbcnt_lo_u32_b32 " A ", exec_lo, 0\n\t"                   \
+    "v_mbcnt_hi_u32_b32 " A ", exec_hi, " A "\n\t"               \
     "s_lshl2_add_u32 %[t], %[o" #I "], %[rel]\n\t"               \
-    "v_lshl_add_u32 v" #A ", v" #A ", 1, %[t]\n\t"               \
-    "ds_read_u16 v" #H ", v" #A "\n\t"
+    "v_lshl_add_u32 " A ", " A ", 1, %[t]\n\t"                   \
+    "ds_read_u16 " H ", " A "\n\t"
 #define MSTF_GATHER                                                                                                  \
     "s_mov_b64 %[sv], exec\n\t"                                                                                      \
     "ds_read_b128 %[qm], %[wa] offset:%[woff]\n\t"                                                                   \
-    "ds_read_b128 v[112:115], %[z]\n\t"                                                                              \
-    "ds_read_b128 v[116:119], %[z]\n\t"                                                                              \
-    MSTF_TILE(0, 112, 120) MSTF_TILE(1, 113, 121) MSTF_TILE(2, 114, 122) MSTF_TILE(3, 115, 123)                              \
-    MSTF_TILE(4, 116, 124) MSTF_TILE(5, 117, 125) MSTF_TILE(6, 118, 126) MSTF_TILE(7, 119, 127)                              \
+    "ds_read_b128 " MSTF_GV0_3 ", %[z]\n\t"                                                                                  \
+    "ds_read_b128 " MSTF_GV4_7 ", %[z]\n\t"                                                                                  \
+    MSTF_TILE(0, MSTF_GV0, MSTF_GV8) MSTF_TILE(1, MSTF_GV1, MSTF_GV9) MSTF_TILE(2, MSTF_GV2, MSTF_GV10) MSTF_TILE(3, MSTF_GV3, MSTF_GV11)                              \
+    MSTF_TILE(4, MSTF_GV4, MSTF_GV12) MSTF_TILE(5, MSTF_GV5, MSTF_GV13) MSTF_TILE(6, MSTF_GV6, MSTF_GV14) MSTF_TILE(7, MSTF_GV7, MSTF_GV15)                              \
     "s_mov_b64 exec, %[sv]\n\t"                                                                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
-    "v_lshl_or_b32 %[v0], v113, 16, v112\n\t"                                                                          \
-    "v_lshl_or_b32 %[v1], v115, 16, v114\n\t"                                                                          \
-    "v_lshl_or_b32 %[v2], v117, 16, v116\n\t"                                                                          \
-    "v_lshl_or_b32 %[v3], v119, 16, v118"
+    "v_lshl_or_b32 %[v0], " MSTF_GV1 ", 16, " MSTF_GV0 "\n\t"                                                                          \
+    "v_lshl_or_b32 %[v1], " MSTF_GV3 ", 16, " MSTF_GV2 "\n\t"                                                                          \
+    "v_lshl_or_b32 %[v2], " MSTF_GV5 ", 16, " MSTF_GV4 "\n\t"                                                                          \
+    "v_lshl_or_b32 %[v3], " MSTF_GV7 ", 16, " MSTF_GV6
 #define MSTF_GATHER_IN                                                                                               \
     [m0] "s"(u64_of(b.mv[0], b.mv[1])), [m1] "s"(u64_of(b.mv[2], b.mv[3])), [m2] "s"(u64_of(b.mv[4], b.mv[5])),      \
         [m3] "s"(u64_of(b.mv[6], b.mv[7])), [m4] "s"(u64_of(b.mv[8], b.mv[9])), [m5] "s"(u64_of(b.mv[10], b.mv[11])), \
@@ -113,8 +164,7 @@ __device__ __forceinline__ void batch_step_exec(const Batch& b, Batch& nxt, cons
         [o1] "s"(b.ov[1]), [o2] "s"(b.ov[2]), [o3] "s"(b.ov[3]), [o4] "s"(b.ov[4]), [o5] "s"(b.ov[5]),               \
         [o6] "s"(b.ov[6]), [o7] "s"(b.ov[7]), [rel] "s"(rel), [wa] "v"(wbase), [woff] "i"(WOFF), [z] "v"(zaddr)
 #define MSTF_GATHER_CLOBBER                                                                                          \
-    "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127",  \
-        "scc", "memory"
+    MSTF_GV_CLOBBER, "scc", "memory"
     if constexpr (PREFETCH) {
         asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t"
                      "s_load_dwordx8 %[no], %[ni], %[ioff]\n\t" MSTF_GATHER
@@ -192,38 +242,41 @@ __device__ __forceinline__ void wait_vm0_keep(Touch& t)
 
 // sub_issue and touch_sub without control flow, for a caller that keeps scalar state (the coming batch) in
 // registers across them: a lane predicate written as a branch splits the block there, and values that live
-// across such a split may end up in vector registers.  The four pieces are issued with exec set by hand
+// across such a split may end up in vector registers.  The four (two for 16-tile stages) pieces are issued with exec set by hand
 // (piece i: the lanes with lane*16 + i*1024 < bytes; an empty exec issues nothing) - one compare, one exec write
 // and the load per piece, where the branches cost ten instructions; the wavefront must have all 64 lanes active.
 //   dst_lds : LDS byte address of the buffer (wave-uniform);  lane16 = lane * 16
 __device__ __forceinline__ void sub_issue_flat(const char* src, uint32_t bytes, uint32_t dst_lds, uint32_t lane16)
 {
-    static_assert(kSubBytes == 4096, "four 1 KB pieces");
+    static_assert(kSubBytes == 4096 || kSubBytes == 2048, "four or two 1 KB pieces");
     uint32_t t, m0_kept;  // m0 is the compiler's to manage: handed back as it was found
     uint64_t sv;          // so is exec
-    asm volatile("s_mov_b32 %[keep], m0\n\t"
-                 "s_mov_b64 %[sv], exec\n\t"
-                 "s_mov_b32 m0, %[dst]\n\t"
-                 "v_cmp_gt_i32 vcc, %[b], %[l]\n\t"
-                 "s_mov_b64 exec, vcc\n\t"
-                 "global_load_lds_dwordx4 %[l], %[src]\n\t"
-                 "s_sub_i32 %[t], %[b], 0x400\n\t"
-                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
-                 "s_mov_b64 exec, vcc\n\t"
-                 "global_load_lds_dwordx4 %[l], %[src] offset:1024\n\t"
-                 "s_sub_i32 %[t], %[b], 0x800\n\t"
-                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
-                 "s_mov_b64 exec, vcc\n\t"
-                 "global_load_lds_dwordx4 %[l], %[src] offset:2048\n\t"
-                 "s_sub_i32 %[t], %[b], 0xc00\n\t"
-                 "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"
-                 "s_mov_b64 exec, vcc\n\t"
-                 "global_load_lds_dwordx4 %[l], %[src] offset:3072\n\t"
-                 "s_mov_b64 exec, %[sv]\n\t"
-                 "s_mov_b32 m0, %[keep]"
-                 : [t] "=&s"(t), [keep] "=&s"(m0_kept), [sv] "=&s"(sv)
-                 : [dst] "s"(dst_lds), [b] "s"(bytes), [l] "v"(lane16), [src] "s"(src)
-                 : "vcc", "scc", "memory");
+#define MSTF_SHEAD                   \
+    "s_mov_b32 %[keep], m0\n\t"      \
+    "s_mov_b64 %[sv], exec\n\t"      \
+    "s_mov_b32 m0, %[dst]\n\t"       \
+    "v_cmp_gt_i32 vcc, %[b], %[l]\n\t" \
+    "s_mov_b64 exec, vcc\n\t"        \
+    "global_load_lds_dwordx4 %[l], %[src]\n\t"
+#define MSTF_SPIECE(HEX, OFF)                \
+    "s_sub_i32 %[t], %[b], " HEX "\n\t"      \
+    "v_cmp_gt_i32 vcc, %[t], %[l]\n\t"       \
+    "s_mov_b64 exec, vcc\n\t"                \
+    "global_load_lds_dwordx4 %[l], %[src] offset:" OFF "\n\t"
+#define MSTF_STAIL "s_mov_b64 exec, %[sv]\n\ts_mov_b32 m0, %[keep]"
+#define MSTF_SOPS                                                           \
+    : [t] "=&s"(t), [keep] "=&s"(m0_kept), [sv] "=&s"(sv)                   \
+    : [dst] "s"(dst_lds), [b] "s"(bytes), [l] "v"(lane16), [src] "s"(src)   \
+    : "vcc", "scc", "memory"
+    if constexpr (kSubBytes == 4096)
+        asm volatile(MSTF_SHEAD MSTF_SPIECE("0x400", "1024") MSTF_SPIECE("0x800", "2048") MSTF_SPIECE("0xc00", "3072")
+                         MSTF_STAIL MSTF_SOPS);
+    else
+        asm volatile(MSTF_SHEAD MSTF_SPIECE("0x400", "1024") MSTF_STAIL MSTF_SOPS);
+#undef MSTF_SHEAD
+#undef MSTF_SPIECE
+#undef MSTF_STAIL
+#undef MSTF_SOPS
 }
 // Every lane touches one bitmap and one offset of the sub-chunk; the lanes beyond it repeat the last one.
 //   off8 = min(lane, kSubTiles - 1) * 8, off4 = min(lane, kSubTiles) * 4
