@@ -7,7 +7,10 @@
 namespace mstf {
 
 constexpr int kFusedD = 128;
-constexpr int kFusedWaves = 8;    // token blocks (= wavefronts) per workgroup: 512 tokens per split
+#ifndef MSTF_FUSED_WAVES
+#define MSTF_FUSED_WAVES 8
+#endif
+constexpr int kFusedWaves = MSTF_FUSED_WAVES;    // token blocks (= wavefronts) per workgroup: 512 tokens per split
 constexpr int kKeySubs = kFusedD / kSubTiles;       // sub-chunks of the key phase
 constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value phase (both halves)
 
