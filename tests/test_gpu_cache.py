@@ -237,3 +237,51 @@ def test_window_append_rotates_and_appends_the_new_token(per_entry_positions, co
     assert np.array_equal(vw.cpu().numpy().view(np.int16), vexp.view(np.int16))
     with pytest.raises(RuntimeError):
         ops.window_append(pt[:, :n_kv * D], pt[:, n_kv * D: 2 * n_kv * D], kw, vw, stride + 1)   # host count past the buffer
+
+
+def test_caches_sharing_a_window_counter_advance_together():
+    """Two layers' caches on one device counter (share_clock): decode_device_proj on both, then advance on both, gives
+    what two independent caches give from decode() on rotated inputs; decode() on a sharing cache is refused."""
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D, res = 2, 2, 4, 128, 256
+    L0, steps = 600, 180                                   # a chunk leaves the window at kv_len 768
+    rng = np.random.default_rng(3)
+    n_q = n_kv * g
+    H = n_q + 2 * n_kv
+
+    def make(seed):
+        K, V = orc.make_kv(seed, bs * n_kv, L0, D)
+        Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, L0, D)
+        Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, L0, D)
+        a = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, max_tokens=1024, window_kernel=True)
+        b = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, max_tokens=1024, window_kernel=True)
+        a.prefill(Kt, Vt)
+        b.prefill(Kt, Vt)
+        return a, b
+
+    lone = [make(5)[0], make(6)[0]]
+    shared = [make(5)[1], make(6)[1]]
+    shared[1].share_clock(shared[0])
+    with pytest.raises(RuntimeError):
+        shared[1].decode(torch.zeros((bs, n_q, 1, D), dtype=torch.float16, device=dev),
+                         torch.zeros((bs, n_kv, 1, D), dtype=torch.float16, device=dev),
+                         torch.zeros((bs, n_kv, 1, D), dtype=torch.float16, device=dev))
+    for t in range(steps):
+        cos, sin = orc.rope_tables(np.array([L0 + t]))
+        ct, st = torch.from_numpy(cos[0]).to(dev), torch.from_numpy(sin[0]).to(dev)
+        outs = []
+        for layer in range(2):
+            proj = rng.standard_normal((bs, H * D)).astype(np.float16)
+            pt = torch.from_numpy(proj).to(dev)
+            outs.append(shared[layer].decode_device_proj(pt[:, : n_q * D], pt[:, n_q * D: (n_q + n_kv) * D],
+                                                         pt[:, (n_q + n_kv) * D:], ct, st))
+            x = proj.reshape(bs, H, 1, D)
+            rot = orc.rope_rows(x[:, : n_q + n_kv], cos[:, None, None, :], sin[:, None, None, :])
+            want = lone[layer].decode(torch.from_numpy(np.ascontiguousarray(rot[:, :n_q])).to(dev),
+                                      torch.from_numpy(np.ascontiguousarray(rot[:, n_q:])).to(dev),
+                                      torch.from_numpy(np.ascontiguousarray(x[:, n_q + n_kv:])).to(dev))
+            assert torch.equal(outs[layer].view(torch.int16), want.view(torch.int16)), (t, layer)
+        for c in shared:
+            c.advance()
+    assert shared[0].compressed_length == lone[0].compressed_length == 512
