@@ -235,8 +235,7 @@ class GraphedGreedyLoop:
 
     Everything that changes from step to step lives in device memory and is updated inside the graph: the token
     ids, the position (RoPE), the window length (one counter for all layers) and the compressed-token count of every
-    layer's cache.  The
-    host only counts (SparseKVCache.advance) and, every 256 tokens, lets the caches compress a chunk between two
+    layer's cache.  The host only counts (SparseKVCache.advance) and, every 256 tokens, lets the caches compress a chunk between two
     replays.  Pooled caches (max_tokens > 0) grow in place and the graph stays valid; a cache whose arrays move
     (the quantised one) reports it and the graph is captured again."""
 
