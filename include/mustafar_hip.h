@@ -328,6 +328,25 @@ int mstf_decode_attention_window_quant(void* stream, const uint64_t* k_bmp, cons
                                        int tokens, int head_dim, int Bq, int groups, int bit, int capacity,
                                        int dequant_mode, void* workspace, size_t workspace_bytes);
 
+/* mstf_decode_attention_window_quant over a quantised cache whose per-tile arrays are pre-allocated for max_tokens
+ * tokens and filled in place: bitmaps, word offsets, scales and zero-points of two heads lie tile_capacity entries
+ * apart (tile_capacity >= max_tokens * head_dim / 64, even), tile_off holds offsets into `packed` wherever the words
+ * of a 64-token block were put (the consumers only need the words of one block to be contiguous), and the number of
+ * cached tokens is read from device memory - min(*tokens_dev, max_tokens), a multiple of 64, may be 0 - while
+ * max_tokens sizes the launch and the workspace.  A call recorded into a HIP graph stays valid while chunks are
+ * appended between replays (the reference concatenates every array per chunk,
+ * models/llama_mustafar_quant_kernel.py:322-345). */
+int mstf_decode_attention_window_quant_pool(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed,
+                                            const uint32_t* k_tile_off, const mstf_half* k_scales,
+                                            const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed,
+                                            const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                            const mstf_half* v_zeros, const mstf_half* q, const mstf_half* k_win,
+                                            const mstf_half* v_win, int win_len, const int32_t* win_len_dev,
+                                            int win_stride, mstf_half* out, float* lse_out, int max_tokens,
+                                            const int32_t* tokens_dev, int64_t tile_capacity, int head_dim, int Bq,
+                                            int groups, int bit, int capacity, int dequant_mode, void* workspace,
+                                            size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ group-32 scale / zero option
  * No counterpart in the reference's kernels: its harness carries GROUP_SIZE = 32 (benchmark/mem_spd_test_quant.py:33,
  * 104) but the producer quantises per 64-element tile (kernel_quant/compression_quant.py:47-57, 209-210).  With

@@ -77,6 +77,8 @@ SIGNATURES = {
     "mstf_value_spmv_quant_grouped": (_i, [_vp] * 8 + [_i] * 9 + [_vp, _sz]),
     "mstf_decode_attention_quant_grouped": (_i, [_vp] * 14 + [_i] * 8 + [_vp, _sz]),
     "mstf_decode_attention_window_quant": (_i, [_vp] * 14 + [_i, _vp, _i, _vp, _vp] + [_i] * 7 + [_vp, _sz]),
+    "mstf_decode_attention_window_quant_pool": (_i, [_vp] * 14 + [_i, _vp, _i, _vp, _vp, _i, _vp, _i64] + [_i] * 6
+                                                + [_vp, _sz]),
 }
 
 

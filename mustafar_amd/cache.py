@@ -158,6 +158,77 @@ class CompressedPool:
         return self.nz[start:start + n]
 
 
+class QuantPool:
+    """One side (keys or values) of a quantised cache that grows in place.
+
+    Bitmaps, word offsets, counts, units, scales and zero-points are pre-allocated for max_tokens tokens
+    ([heads, tile_capacity] each) and so is the buffer of packed words, sized for the worst case (every element
+    kept).  A chunk is quantised straight into the next free region of that buffer - a region has room for the
+    chunk's worst case, so its start is known on the host and nothing is read back; the words a chunk does not need
+    stay unused, which the consumers allow: tile_off says where every tile's words are, and only the words of one
+    64-token block have to be contiguous - and its per-tile arrays are written behind the ones held, the offsets
+    shifted by the region's start.  No array ever moves (the reference concatenates all seven per chunk,
+    models/llama_mustafar_quant_kernel.py:322-345); the number of tokens held is mirrored in device memory
+    (tokens_dev) for consumers recorded into a HIP graph (mustafar_package_quant.decode_attention_window_quant_pool)."""
+
+    def __init__(self, heads, head_dim, max_tokens, is_value, bit, device):
+        assert max_tokens % 64 == 0 and bit in (2, 4, 8)
+        self.heads, self.head_dim, self.is_value, self.max_tokens, self.bit = heads, head_dim, is_value, max_tokens, bit
+        self.tile_capacity = max_tokens * head_dim // 64
+        T = self.tile_capacity
+
+        def store(dtype):
+            return torch.zeros((heads, T), dtype=dtype, device=device)
+
+        self.bmp_store, self.off_store = store(torch.int64), store(torch.int32)
+        self.counts_store, self.units_store = store(torch.int32), store(torch.int32)
+        self.scales_store, self.zeros_store = store(torch.float16), store(torch.float16)
+        self.packed = torch.zeros(heads * max_tokens * head_dim * bit // 32, dtype=torch.int32, device=device)
+        self.reserved = 0            # words handed out to chunks so far
+        self.tokens_dev = torch.zeros(1, dtype=torch.int32, device=device)
+        self.tokens = 0
+        self._totals = []            # the producers' word totals (device tensors), looked at by check()
+
+    @property
+    def tiles(self):
+        return self.tokens * self.head_dim // 64
+
+    def append(self, x, kth, ws=None):
+        """x: [heads, M, head_dim] fp16, M % 64 == 0, pruned here to rank kth (0: already pruned)."""
+        from . import compression_quant as cq
+        B, M, N = x.shape
+        assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
+        region = B * M * N * self.bit // 32
+        room = self.packed[self.reserved:self.reserved + region]
+        bmp, off, _, counts, units, scales, zeros, total = cq._produce(x, self.is_value, self.bit, kth, 64, ws, room)
+        T0, Tc = self.tiles, bmp.shape[1]
+        self.bmp_store[:, T0:T0 + Tc] = bmp
+        self.off_store[:, T0:T0 + Tc] = off + self.reserved
+        self.counts_store[:, T0:T0 + Tc] = counts
+        self.units_store[:, T0:T0 + Tc] = units
+        self.scales_store[:, T0:T0 + Tc] = scales
+        self.zeros_store[:, T0:T0 + Tc] = zeros
+        self.reserved += region
+        self.tokens += M
+        self.tokens_dev += M
+        self._totals.append(total)
+
+    def check(self):
+        """Raises if a producer call gave up (one host read per call since the last check)."""
+        from . import compression_quant as cq
+        for t in self._totals:
+            cq.words_written(t)
+        self._totals = []
+
+    def view(self):
+        """The side as the reference's operators take it: [bitmaps, tile_offsets, packed, counts, units, scales,
+        zeros] with contiguous per-tile arrays of the tokens held (copies; the packed buffer is the pool's own)."""
+        T = self.tiles
+        return [self.bmp_store[:, :T].contiguous(), self.off_store[:, :T].contiguous(), self.packed,
+                self.counts_store[:, :T].contiguous(), self.units_store[:, :T].contiguous(),
+                self.scales_store[:, :T].contiguous(), self.zeros_store[:, :T].contiguous()]
+
+
 class SparseKVCache:
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False,
                  max_tokens=0, window_kernel=False):
@@ -186,13 +257,16 @@ class SparseKVCache:
             self.ws = ops.Workspace(device)
         return self.ws
 
+    def _make_pools(self, heads, D, device):
+        self.k_pool = CompressedPool(heads, D, self.max_tokens, False, device)
+        self.v_pool = CompressedPool(heads, D, self.max_tokens, True, device)
+
     def _grow(self, K, V):
         """Adds the tokens K, V [bs, n_kv, M, D] to the compressed part."""
         bs, n_kv, M, D = K.shape
         if self.max_tokens > 0:
             if self.k_pool is None:
-                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, K.device)
-                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, K.device)
+                self._make_pools(bs * n_kv, D, K.device)
             ws = self._workspace(K.device)
             self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
             self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
@@ -229,8 +303,7 @@ class SparseKVCache:
         Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
         if self.max_tokens > 0:
             if self.k_pool is None:
-                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, kx.device)
-                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, kx.device)
+                self._make_pools(bs * n_kv, D, kx.device)
             ws = self._workspace(kx.device)
             self.k_pool.append_proj(kx, self.kth_k, Lc, cos, sin, ws=ws)
             if Lc > 0:
@@ -259,9 +332,9 @@ class SparseKVCache:
         self.compressed_length, self.kv_len = Lc, L
         if self.window_kernel:
             bs, n_kv, _, D = K.shape
-            if self.max_tokens > 0 and self.k_pool is None:   # nothing compressed yet: the (empty) pools exist from the
-                self.k_pool = CompressedPool(bs * n_kv, D, self.max_tokens, False, K.device)   # start, so the attention
-                self.v_pool = CompressedPool(bs * n_kv, D, self.max_tokens, True, K.device)    # call never changes form
+            if self.max_tokens > 0 and self.k_pool is None:
+                # nothing compressed yet: the (empty) pools exist from the start, so the attention call never changes form
+                self._make_pools(bs * n_kv, D, K.device)
             cap = max(self.residual_length + CHUNK, L - Lc)   # the window never holds more before a chunk leaves
             self._kbuf = torch.empty((bs * n_kv, cap, D), dtype=torch.float16, device=K.device)
             self._vbuf = torch.empty_like(self._kbuf)
@@ -418,14 +491,21 @@ class QuantSparseKVCache(SparseKVCache):
     decode_attention_window_quant (three launches, capturable with decode_device / advance)."""
 
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, bit=2,
-                 dequant_mode=0, fused=False, window_kernel=False):
+                 dequant_mode=0, fused=False, window_kernel=False, max_tokens=0):
+        """max_tokens > 0: the compressed part lives in pre-allocated pools (QuantPool) and grows in place, pruning
+        fused into the producer; with window_kernel the attention reads the pools themselves and a captured decode
+        step stays valid across chunk appends."""
         super().__init__(groups, head_dim, k_sparsity, v_sparsity, residual_length, fused=fused,
-                         window_kernel=window_kernel)
+                         window_kernel=window_kernel, max_tokens=max_tokens)
         self.bit, self.dequant_mode = bit, dequant_mode
         # self.k / self.v: 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales, zeros]
 
     def _attend_device(self, q2):
         from . import mustafar_package_quant as mpq
+        if self.k_pool is not None:
+            return mpq.decode_attention_window_quant_pool(self.k_pool, self.v_pool, q2, self._kbuf, self._vbuf,
+                                                          self._kbuf.shape[1], self.groups, self.dequant_mode,
+                                                          win_len_dev=self._wlen_dev, ws=self._workspace(q2.device))
         return mpq.decode_attention_window_quant(self.k, self.v, q2, self._kbuf, self._vbuf, self._kbuf.shape[1],
                                                  self.groups, self.bit, self.dequant_mode, win_len_dev=self._wlen_dev,
                                                  ws=self._workspace(q2.device))
@@ -456,7 +536,23 @@ class QuantSparseKVCache(SparseKVCache):
                 torch.cat([old[3], new[3]], 1), torch.cat([old[4], new[4]], 1), torch.cat([old[5], new[5]], 1),
                 torch.cat([old[6], new[6]], 1)]
 
+    def _make_pools(self, heads, D, device):
+        self.k_pool = QuantPool(heads, D, self.max_tokens, False, self.bit, device)
+        self.v_pool = QuantPool(heads, D, self.max_tokens, True, self.bit, device)
+
     def _grow(self, K, V):
+        if self.max_tokens > 0:
+            bs, n_kv, M, D = K.shape
+            if self.k_pool is None:
+                self._make_pools(bs * n_kv, D, K.device)
+            ws = self._workspace(K.device)
+            self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
+            self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
+            self.k_pool.check()
+            self.v_pool.check()
+            if not self.window_kernel:
+                self.k, self.v = self.k_pool.view(), self.v_pool.view()
+            return
         ck, cv = self._compress(K, V)
         self.k = ck if self.k is None else self._append(self.k, ck)
         self.v = cv if self.v is None else self._append(self.v, cv)

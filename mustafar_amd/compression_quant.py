@@ -11,7 +11,10 @@ from . import ops
 from ._lib import check, lib
 
 
-def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
+def _produce(inputs, is_value, bit, kth=0, group_size=64, ws=None, room=None):
+    """One call of the producer.  room: int32 tensor that takes the packed words (tile offsets count from its start);
+    default: a fresh buffer with room for the worst case.  Returns the per-tile arrays, the buffer and the word total
+    as a device tensor (all ones should a wait of the one-pass producer have run out) - nothing is read on the host."""
     assert inputs.is_cuda
     assert inputs.dim() == 3
     B, M, N = inputs.shape
@@ -33,21 +36,31 @@ def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
     zeros = torch.empty(meta_shape, dtype=torch.float16, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
     ws = ops.workspace(dev, L.mstf_compress_quant_workspace_bytes(B, M, N), ws)
-    name = "mstf_compress_quant_grouped"
     st = torch.cuda.current_stream().cuda_stream
-    # one pass with room for the worst case (every element kept: 64 // capacity words per tile), then the used
-    # part is copied out so that the large buffer goes back to the allocator; the total is read once on the host, as
-    # the reference's .item() does
+    # one pass with room for the worst case (every element kept: 64 // capacity words per tile)
     cap_words = B * T * (64 * int(bit) // 32)
-    room = torch.empty((max(cap_words, 1),), dtype=torch.int32, device=dev)
+    if room is None:
+        room = torch.empty((max(cap_words, 1),), dtype=torch.int32, device=dev)
+    assert room.dtype == torch.int32 and room.is_contiguous() and room.numel() >= cap_words
     check(L.mstf_compress_quant_grouped(st, x.data_ptr(), int(bool(is_value)), B, M, N, int(kth), int(bit), int(group_size),
                                         bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(), units.data_ptr(),
                                         scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,
-                                        ws.data_ptr(), ws.numel()), name)
+                                        ws.data_ptr(), ws.numel()), "mstf_compress_quant_grouped")
+    return bmp, tile_off, room, counts, units, scales, zeros, total
+
+
+def words_written(total):
+    """The producer's word total on the host (one read, as the reference's .item()); raises if the producer gave up."""
     n = int(total.item())
     if n < 0:   # all ones: a workgroup of the one-pass producer gave up waiting (ruled out by the dispatch order)
         raise RuntimeError("the quantised producer gave up waiting for an earlier workgroup; the packed words are incomplete")
-    packed = room[:n].clone()
+    return n
+
+
+def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
+    bmp, tile_off, room, counts, units, scales, zeros, total = _produce(inputs, is_value, bit, kth, group_size, ws)
+    # the used part is copied out so that the large buffer goes back to the allocator
+    packed = room[:words_written(total)].clone()
     return bmp, tile_off, packed, counts, units, scales, zeros
 
 

@@ -34,8 +34,18 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
     const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros, const uint64_t* __restrict__ v_bmp,
     const uint32_t* v_packed, const uint32_t* __restrict__ v_off, const uint32_t* v_off_dma, const uint16_t* v_scales,
     const uint16_t* v_zeros, const _Float16* q, _Float16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int Lc, int groups, int nblk, int nsplit, int write_final, float sqrt_d, int mode)
+    float* __restrict__ part_ml, size_t tstride, int groups, int nblk, int nsplit, int write_final, float sqrt_d, int mode,
+    const int* __restrict__ tokens_dev, int heads_fastest)
 {
+    // tstride: tiles between the per-tile rows of two heads - the tile count of the cached tokens unless the arrays are
+    // pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read from device memory, at most
+    // nblk blocks of it; the launch is then sized for the capacity and the wavefronts beyond the valid blocks leave
+    // neutral partials.  heads_fastest: the heads vary fastest over the workgroup index, so that the workgroups beyond
+    // the valid blocks are dispatched last instead of standing in front of working ones.
+    if (tokens_dev) {
+        const int valid = *tokens_dev / 64;
+        nblk = valid < nblk ? valid : nblk;
+    }
     using F = QFmt<BIT>;
     constexpr int D = kFusedD;
     // query and weight rows sit 16 bytes further apart than their length: the four rows that the lanes of a group read
@@ -53,12 +63,12 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
     __shared__ __attribute__((aligned(16))) char lds_all[kFusedWaves * kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
-    const int split = (int)blockIdx.x;
-    const int kv = (int)blockIdx.y;
+    const int split = heads_fastest ? (int)blockIdx.y : (int)blockIdx.x;
+    const int kv = heads_fastest ? (int)blockIdx.x : (int)blockIdx.y;
     const int tb = split * kFusedWaves + wave;
     const bool active = tb < nblk;  // wave-uniform
     const int j = lane & 3;
-    const size_t T = (size_t)Lc * D / 64;
+    const size_t T = tstride;
     char* my = lds_all + wave * kWaveLds;
     char* wordbuf = my + kImgBytes + 16;
     char* metabuf = wordbuf + 2 * F::kWordBuf;
@@ -185,16 +195,18 @@ static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp
                                 const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_off,
                                 const uint16_t* v_scales, const uint16_t* v_zeros, const _Float16* q, _Float16* out,
                                 float* part_o, float* part_ml, int tokens, int groups, int ns, int write_final, float sq,
-                                int mode, int group_size)
+                                int mode, int group_size, size_t tstride, const int32_t* tokens_dev, int heads_fastest)
 {
     if (group_size == 32)
         hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
                            k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
-                           out, part_o, part_ml, tokens, groups, tokens / 64, ns, write_final, sq, mode);
+                           out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
+                           heads_fastest);
     else
         hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
                            k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
-                           out, part_o, part_ml, tokens, groups, tokens / 64, ns, write_final, sq, mode);
+                           out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
+                           heads_fastest);
 }
 
 }  // namespace mstf
@@ -229,12 +241,15 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
                         const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
                         const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
                         int groups, int bit, int dequant_mode, void* workspace, int nst, int write_final,
-                        int group_size = 64)
+                        int group_size = 64, size_t tile_stride = 0, const int32_t* tokens_dev = nullptr)
 {
+    // tile_stride / tokens_dev: a cache pre-allocated for `tokens` tokens that holds *tokens_dev of them (see the kernel)
     const int Bkv = Bq / groups, ns = fused_nsplit(tokens);
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * nst * head_dim;
-    const dim3 grid((unsigned)ns, (unsigned)Bkv);
+    const int heads_fastest = tokens_dev ? 1 : 0;
+    const dim3 grid = heads_fastest ? dim3((unsigned)Bkv, (unsigned)ns) : dim3((unsigned)ns, (unsigned)Bkv);
+    const size_t tstride = tile_stride ? tile_stride : (size_t)tokens * head_dim / 64;
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
     _Float16* oh = reinterpret_cast<_Float16*>(out);
     const float sq = sqrtf((float)head_dim);
@@ -244,7 +259,8 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
     const uint16_t* vz = reinterpret_cast<const uint16_t*>(v_zeros);
 #define MSTF_FQ(NMV, BITV)                                                                                             \
     launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, ks, kz, v_bmp, v_packed, v_tile_off, vs, vz, \
-                                   qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode, group_size)
+                                   qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode, group_size, \
+                                   tstride, tokens_dev, heads_fastest)
     if (groups <= 4) {
         if (bit == 2) MSTF_FQ(1, 2); else if (bit == 4) MSTF_FQ(1, 4); else MSTF_FQ(1, 8);
     } else {
@@ -338,6 +354,42 @@ extern "C" int mstf_decode_attention_window_quant(
                           v_zeros, q, nullptr, tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, nst, 0);
         if (rc != MSTF_OK) return rc;
     }
+    if ((rc = window_launch(st, k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq, groups, nst,
+                            ns)) != MSTF_OK)
+        return rc;
+    return merge_splits(st, workspace, out, lse_out, nst, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_attention_window_quant_pool(
+    void* stream, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off, const mstf_half* k_scales,
+    const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+    const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q, const mstf_half* k_win,
+    const mstf_half* v_win, int win_len, const int32_t* win_len_dev, int win_stride, mstf_half* out, float* lse_out,
+    int max_tokens, const int32_t* tokens_dev, int64_t tile_capacity, int head_dim, int Bq, int groups, int bit,
+    int capacity, int dequant_mode, void* workspace, size_t workspace_bytes)
+{
+    if (!q || !k_win || !v_win || !out || !tokens_dev) return MSTF_EINVAL;
+    if (max_tokens <= 0 || win_len <= 0 || win_stride < win_len || Bq <= 0 || groups <= 0 || Bq % groups != 0)
+        return MSTF_EINVAL;
+    if (head_dim != kFusedD || max_tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (tile_capacity < (int64_t)max_tokens * head_dim / 64) return MSTF_EINVAL;
+    if (!aligned_to(q, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)) || !aligned_to(tokens_dev, 4))
+        return MSTF_EALIGN;
+    // rows of the per-tile arrays start tile_capacity entries apart: the two-byte ones keep their four-byte alignment
+    if (tile_capacity % 2 != 0) return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    hipStream_t st = as_stream(stream);
+    const int ns = fused_nsplit(max_tokens), nst = ns + window_blocks(win_len);
+    int rc = quant_check(k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
+                         max_tokens, head_dim, Bq, groups, bit, capacity, dequant_mode);
+    if (rc != MSTF_OK) return rc;
+    rc = quant_launch(st, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros, q,
+                      nullptr, max_tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, nst, 0, 64,
+                      (size_t)tile_capacity, tokens_dev);
+    if (rc != MSTF_OK) return rc;
     if ((rc = window_launch(st, k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq, groups, nst,
                             ns)) != MSTF_OK)
         return rc;

@@ -131,7 +131,7 @@ class Decoder:
                                          max_tokens=max_tokens, window_kernel=True) for _ in range(c.layers)]
         elif cache in ("sparse_quant2", "sparse_quant4"):
             self.caches = [QuantSparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length,
-                                              bit=int(cache[-1]), fused=True, window_kernel=True)
+                                              bit=int(cache[-1]), fused=True, window_kernel=True, max_tokens=max_tokens)
                            for _ in range(c.layers)]
         else:
             self.caches = [DenseMaskedCache(groups, c.head_dim, sparsity, sparsity, residual_length)

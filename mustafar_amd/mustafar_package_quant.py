@@ -183,6 +183,34 @@ def decode_attention_window_quant(key_side, value_side, q, k_win, v_win, win_len
     return o
 
 
+def decode_attention_window_quant_pool(k_pool, v_pool, q, k_win, v_win, win_len, num_key_value_groups, dequant_mode=0,
+                                       out=None, lse=None, win_len_dev=None, ws=None):
+    """decode_attention_window_quant over two cache.QuantPool sides that grow in place: the pools' pre-allocated
+    per-tile arrays are read with their row stride and the number of compressed tokens comes from the pool's device
+    counter, so nothing about the call changes when a chunk is appended (a HIP graph holding it stays valid)."""
+    assert q.dtype == torch.float16 and q.is_contiguous()
+    assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
+    assert k_pool.max_tokens == v_pool.max_tokens and k_pool.bit == v_pool.bit
+    D = q.shape[-1]
+    Bq = q.numel() // D
+    L = lib()
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q.device) if out is None else out
+    ws = ops.workspace(q.device, L.mstf_decode_attention_window_workspace_bytes(k_pool.max_tokens, int(win_len), D, Bq,
+                                                                                int(num_key_value_groups)), ws)
+    ptrs = []
+    for p in (k_pool, v_pool):
+        ptrs += [p.bmp_store.data_ptr(), p.packed.data_ptr(), p.off_store.data_ptr(), p.scales_store.data_ptr(),
+                 p.zeros_store.data_ptr()]
+    bit = int(k_pool.bit)
+    check(L.mstf_decode_attention_window_quant_pool(
+        torch.cuda.current_stream().cuda_stream, *ptrs, q.data_ptr(), k_win.data_ptr(), v_win.data_ptr(), int(win_len),
+        win_len_dev.data_ptr() if win_len_dev is not None else None, int(k_win.shape[1]), o.data_ptr(),
+        lse.data_ptr() if lse is not None else None, k_pool.max_tokens, k_pool.tokens_dev.data_ptr(),
+        k_pool.tile_capacity, D, Bq, int(num_key_value_groups), bit, 32 // bit, int(dequant_mode), ws.data_ptr(),
+        ws.numel()), "mstf_decode_attention_window_quant_pool")
+    return o
+
+
 # aliases the reference exports for its model code (pybind_quant.cpp:96-176)
 mustafar_quant_sparse_forward = mustafar_key_formulation_quant
 mustafar_quant_sparse_forward_meta = mustafar_key_formulation_quant_meta

@@ -104,9 +104,11 @@ def test_short_prompt_stays_dense_until_first_chunk(window_kernel):
     assert torch.isfinite(out).all()
 
 
-@pytest.mark.parametrize("fused,bit,window_kernel", [(False, 2, False), (True, 2, False), (True, 4, False),
-                                                     (True, 2, True), (True, 8, True)])
-def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
+@pytest.mark.parametrize("fused,bit,window_kernel,pooled", [(False, 2, False, False), (True, 2, False, False),
+                                                            (True, 4, False, False), (True, 2, True, False),
+                                                            (True, 8, True, False), (False, 2, False, True),
+                                                            (True, 2, True, True), (True, 4, True, True)])
+def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel, pooled):
     """The quantised caller's state machine: after the prefill and two chunk appends (the reference's append: words
     behind the old ones, offsets shifted) every checked decode step matches dense masked attention over
     [oracle-dequantised compressed part | dense window] within 1e-2, and the per-tile arrays equal a one-shot
@@ -121,7 +123,9 @@ def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
     Q = rng.standard_normal((steps, bs * n_kv * g, D)).astype(np.float16)
     Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, total, D)
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, total, D)
-    cache = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=fused, window_kernel=window_kernel)
+    # pooled: pre-allocated per-tile arrays and word buffer filled in place, pruning fused into the producer
+    cache = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=fused, window_kernel=window_kernel,
+                               max_tokens=768 if pooled else 0)
     cache.prefill(Kt[:, :, :L0], Vt[:, :, :L0])
     assert cache.compressed_length == 256
 
@@ -146,7 +150,8 @@ def test_quantised_cache_prefill_decode_append(fused, bit, window_kernel):
     assert cache.compressed_length == 512 and cache.kv_len == total and checked >= 6
     # per-tile arrays equal a one-shot quantisation; the packed words are the same words, chunk by chunk
     Lc = cache.compressed_length
-    for side, src, is_value in ((cache.k, K, 0), (cache.v, V, 1)):
+    sides = (cache.k_pool.view(), cache.v_pool.view()) if pooled else (cache.k, cache.v)
+    for side, src, is_value in ((sides[0], K, 0), (sides[1], V, 1)):
         ref = orc.compress_quant(orc.prune_rows(np.ascontiguousarray(src[:, :Lc]), 89), is_value, bit)
         for i in (0, 3, 4):
             assert np.array_equal(side[i].cpu().numpy(), ref[i])

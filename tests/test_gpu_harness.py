@@ -80,3 +80,27 @@ def test_prefill_from_the_projection_output_fills_the_same_cache():
     assert torch.equal(ca.k_win.view(torch.int16), cb.k_win.view(torch.int16))
     assert torch.equal(ca.v_win.view(torch.int16), cb.v_win.view(torch.int16))
     assert float((la - lb).abs().max() / la.abs().max()) < 1e-2
+
+
+def test_graphed_loop_over_the_quantised_pooled_cache_needs_one_capture():
+    """The quantised cache in pooled form (per-tile arrays and packed words pre-allocated, chunks quantised in place):
+    the graphed loop generates the eager loop's tokens with ONE capture across a chunk append."""
+    from mustafar_amd.harness import Config, Decoder, GraphedGreedyLoop, generate
+    dev = torch.device("cuda:0")
+    cfg = Config(hidden=512, layers=2, n_q=4, n_kv=2, head_dim=128, ffn=1024, vocab=1000)
+    g = torch.Generator(device=dev)
+    g.manual_seed(6)
+    bs, prompt, new = 2, 600, 200                      # a chunk is appended at kv_len 768, between two replays
+    ids = torch.randint(0, cfg.vocab, (bs, prompt), generator=g, device=dev)
+    eager = Decoder(cfg, dev, seed=23, cache="sparse_quant2", max_tokens=1024)
+    toks, _ = generate(eager, ids, new)
+    graphed = Decoder(cfg, dev, seed=23, cache="sparse_quant2", max_tokens=1024)
+    logits = graphed.prefill(ids)
+    loop = GraphedGreedyLoop(graphed, logits[:, -1].argmax(-1, keepdim=True), prompt)
+    got = [loop.ids.clone()]
+    for t in range(new - 1):
+        loop.step()
+        got.append(loop.ids.clone())
+    got = torch.cat(got, 1)
+    assert loop.captures == 1 and graphed.caches[0].compressed_length == eager.caches[0].compressed_length == 512
+    assert torch.equal(got, toks)
