@@ -275,7 +275,7 @@ def quant_record(torch, ops, dev, gen, bs, L, sparsity, bit, group_size, reps):
             "bytes_per_token_per_kv_head": {"key": round(kb / Bkv / L, 2), "value": round(vb / Bkv / L, 2)}}
 
 
-def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens):
+def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens, cache="sparse"):
     """configs[4], shortened: random-init Llama-3-8B shape, greedy decoding with the step replayed from a HIP graph
     (tokens/s) and a few eager steps with events around the cache's attention (its share of the step)."""
     import time as _time
@@ -283,7 +283,7 @@ def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens):
     from mustafar_amd.harness import Config, Decoder, GraphedGreedyLoop
     cfg = Config(layers=layers)
     max_tokens = ((prompt + new_tokens + 16 + CHUNK - 1) // CHUNK) * CHUNK
-    dec = Decoder(cfg, dev, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=max_tokens)
+    dec = Decoder(cfg, dev, cache=cache, sparsity=0.7, residual_length=256, max_tokens=max_tokens)
     g = torch.Generator(device=dev)
     g.manual_seed(1)
     ids = torch.randint(0, cfg.vocab, (batch, prompt), generator=g, device=dev)
@@ -314,7 +314,8 @@ def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens):
         loop.step()
     torch.cuda.synchronize()
     t_step = (_time.perf_counter() - t0) / new_tokens
-    return {"layers": layers, "batch": batch, "prompt": prompt, "new_tokens_timed": new_tokens, "prefill_s": round(t_prefill, 3),
+    return {"cache": cache, "layers": layers, "batch": batch, "prompt": prompt, "new_tokens_timed": new_tokens,
+            "prefill_s": round(t_prefill, 3),
             "graphed_decode_ms_per_step": round(1e3 * t_step, 3), "tokens_per_s": round(batch / t_step, 1),
             "graph_captures": loop.captures, "eager_decode_ms_per_step": round(1e3 * t_eager, 3),
             "eager_attention_over_cache_ms_per_step": round(attn_ms, 3),
@@ -499,8 +500,12 @@ def main():
         if args.loop_layers > 0:
             try:
                 configs["configs4_decode_loop"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 32)
+                torch.cuda.empty_cache()
+                configs["configs4_decode_loop_2bit"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 32,
+                                                                          cache="sparse_quant2")
             except Exception as e:  # pragma: no cover - e.g. out of memory on a shared box; reported, not fatal
-                configs["configs4_decode_loop"] = {"error": str(e)[:200]}
+                configs.setdefault("configs4_decode_loop", {"error": str(e)[:200]})
+                configs.setdefault("configs4_decode_loop_2bit", {"error": str(e)[:200]})
         torch.cuda.empty_cache()
 
     # a copy of known size, so that a counter run of this same command can be calibrated (outside every timed region)
