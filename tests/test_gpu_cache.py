@@ -104,6 +104,30 @@ def test_short_prompt_stays_dense_until_first_chunk(window_kernel):
     assert torch.isfinite(out).all()
 
 
+def test_short_prompt_on_the_pooled_quantised_cache_matches_the_concatenating_one():
+    """Nothing compressed after the prefill: the pooled quantised cache attends with empty pools (token count 0 on the
+    device), then quantises its first chunk in place; every step equals the cache that appends by concatenation."""
+    from mustafar_amd.cache import QuantSparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D = 1, 2, 2, 128
+    K, V = orc.make_kv(8, bs * n_kv, 320, D)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, 320, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, 320, D)
+    a = QuantSparseKVCache(g, D, 0.7, 0.7, 32, bit=2, fused=True, window_kernel=True)
+    b = QuantSparseKVCache(g, D, 0.7, 0.7, 32, bit=2, fused=True, window_kernel=True, max_tokens=512)
+    for c in (a, b):
+        c.prefill(Kt[:, :, :200], Vt[:, :, :200])
+        assert c.compressed_length == 0
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4)
+    for pos in range(200, 320):
+        q = torch.randn((bs, n_kv * g, 1, D), generator=gen, device=dev, dtype=torch.float16)
+        oa = a.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
+        ob = b.decode(q, Kt[:, :, pos:pos + 1], Vt[:, :, pos:pos + 1])
+        assert torch.equal(oa.view(torch.int16), ob.view(torch.int16)), pos
+    assert a.compressed_length == b.compressed_length == 256
+
+
 @pytest.mark.parametrize("fused,bit,window_kernel,pooled", [(False, 2, False, False), (True, 2, False, False),
                                                             (True, 4, False, False), (True, 2, True, False),
                                                             (True, 8, True, False), (False, 2, False, True),
