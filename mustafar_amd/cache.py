@@ -55,7 +55,7 @@ class CompressedPool:
 
     Every head owns a slab of the packed-value pool (nz_off[b] = start of slab b, which the format allows); a chunk
     is compressed straight to the end of each head's values by mstf_append_*_f16, so appending re-copies no packed
-    values, reads nothing back to the host and launches the same three kernels whatever the cache holds.  The per-tile
+    values, reads nothing back to the host and launches the same kernels whatever the cache holds.  The per-tile
     arrays are pre-allocated for max_tokens too (bmp_store [heads, tile_capacity], idx_store [heads, tile_capacity + 1])
     and a chunk's bitmaps and offsets are written behind the ones that are there, so no array of the pool ever moves;
     the number of tokens held is mirrored in device memory (tokens_dev) for consumers recorded into a HIP graph
