@@ -174,6 +174,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     __shared__ uint32_t slabs[W][kHalfSlabDw];
     __shared__ uint32_t wave_total[W];
     __shared__ uint64_t bases[W][2];
+    __shared__ uint32_t coop_words[W][16];  // the packed words of a tile quantised by the whole wavefront (64 * bit / 32 <= 16)
     const int lane = lane_id();
     const int wave = wave_id();
     const int nblk = M / 64;
@@ -320,34 +321,74 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
         __builtin_amdgcn_wave_barrier();
         const uint64_t m = bm[h];
         const uint64_t off = off_h[h];
-        if (off + u[h] > capacity_words) continue;  // would not fit: leave untouched
-        uint32_t cur = 0;
-        int pos = 0;
-        uint32_t w = 0;
-        // the kept elements first to last; the coming element is read from LDS while the current one is quantised
-        auto at = [&](int i) { return (float)sh[IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane)]; };
-        uint64_t rem = m;
-        int i = rem != 0ull ? __builtin_clzll(rem) : 0;
-        float v = at(i);
-        while (rem != 0ull) {
-            rem &= ~(0x8000000000000000ull >> i);
-            const int i_next = rem != 0ull ? __builtin_clzll(rem) : i;
-            const float v_next = at(i_next);
-            const float sc = (G32 && i >= 32) ? scg[h][NG - 1] : scg[h][0];   // the element's position picks the pair
-            const float zp = (G32 && i >= 32) ? zpg[h][NG - 1] : zpg[h][0];
+        const bool fits = off + u[h] <= capacity_words;  // a tile that would not fit is left untouched
+        // Key tiles with many survivors - a channel of outliers keeps all of its 64 tokens - would make the whole
+        // wavefront loop as often as they have elements; the few of them (at most kCoopMax, else none) are left to the
+        // cooperative pass below, where the 64 lanes quantise the tile's 64 positions together.
+        constexpr uint32_t kCoopOver = 48, kCoopMax = 8;
+        uint64_t coop = 0;
+        if (!IS_VALUE) {
+            coop = __ballot(fits && (uint32_t)__popcll(m) > kCoopOver);
+            if ((uint32_t)__popcll(coop) > kCoopMax) coop = 0;
+        }
+        if (fits && ((coop >> lane) & 1ull) == 0ull) {
+            uint32_t cur = 0;
+            int pos = 0;
+            uint32_t w = 0;
+            // the kept elements first to last; the coming element is read from LDS while the current one is quantised
+            auto at = [&](int i) { return (float)sh[IS_VALUE ? (lane * (2 * kHalfRowDw) + i) : (i * (2 * kHalfRowDw) + lane)]; };
+            uint64_t rem = m;
+            int i = rem != 0ull ? __builtin_clzll(rem) : 0;
+            float v = at(i);
+            while (rem != 0ull) {
+                rem &= ~(0x8000000000000000ull >> i);
+                const int i_next = rem != 0ull ? __builtin_clzll(rem) : i;
+                const float v_next = at(i_next);
+                const float sc = (G32 && i >= 32) ? scg[h][NG - 1] : scg[h][0];   // the element's position picks the pair
+                const float zp = (G32 && i >= 32) ? zpg[h][NG - 1] : zpg[h][0];
+                float q = floorf(v / sc + 0.5f) + zp;
+                q = fminf(fmaxf(q, 0.f), maxq);
+                cur |= (uint32_t)q << pos;
+                pos += bit;
+                if (pos == 32) {
+                    packed[off + w++] = cur;
+                    cur = 0;
+                    pos = 0;
+                }
+                v = v_next;
+                i = i_next;
+            }
+            if (pos > 0) packed[off + w] = cur;
+        }
+        // cooperative pass: lane = token; the tile's bitmap, parameters and word offset come from its owner lane
+        while (coop != 0ull) {
+            const int c = __builtin_ctzll(coop);
+            coop &= coop - 1ull;
+            const uint64_t mc = u64_of((uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)m, c),
+                                       (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(m >> 32), c));
+            const uint64_t offc = u64_of((uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)off, c),
+                                         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(off >> 32), c));
+            auto from_owner = [&](float x) {
+                return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), c));
+            };
+            const float sc0 = from_owner(scg[h][0]), zp0 = from_owner(zpg[h][0]);
+            const float sc1 = from_owner(scg[h][NG - 1]), zp1 = from_owner(zpg[h][NG - 1]);
+            const float sc = (G32 && lane >= 32) ? sc1 : sc0, zp = (G32 && lane >= 32) ? zp1 : zp0;
+            const uint64_t ml = lanes_of(mc);                    // bit i <=> token i
+            const bool keep = ((ml >> lane) & 1ull) != 0ull;
+            const float v = keep ? (float)sh[lane * (2 * kHalfRowDw) + c] : 0.f;
             float q = floorf(v / sc + 0.5f) + zp;
             q = fminf(fmaxf(q, 0.f), maxq);
-            cur |= (uint32_t)q << pos;
-            pos += bit;
-            if (pos == 32) {
-                packed[off + w++] = cur;
-                cur = 0;
-                pos = 0;
-            }
-            v = v_next;
-            i = i_next;
+            const uint32_t rank = rank_below(ml);
+            const uint32_t word = rank / (uint32_t)cap, shift = (rank % (uint32_t)cap) * (uint32_t)bit;
+            if (lane < 16) coop_words[wave][lane] = 0u;
+            __builtin_amdgcn_wave_barrier();
+            if (keep) atomicOr(&coop_words[wave][word], (uint32_t)q << shift);
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t nwords = ((uint32_t)__popcll(mc) + (uint32_t)cap - 1u) / (uint32_t)cap;
+            if ((uint32_t)lane < nwords) packed[offc + lane] = coop_words[wave][lane];
+            __builtin_amdgcn_wave_barrier();
         }
-        if (pos > 0) packed[off + w] = cur;
     }
 }
 
