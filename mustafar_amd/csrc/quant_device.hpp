@@ -77,13 +77,18 @@ __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uin
     constexpr int kTilesPerHalfPass = 64 / kHalfSlots;
     constexpr int kHalfPasses = kSubTiles / kTilesPerHalfPass;
     static_assert(kSubTiles == 32, "lanes 0..31 test the 32 tiles of the stage");
-    bool need_high;
+    // Tiles with more words than the first half covers: a few of them (a key stage typically holds one channel of
+    // outliers, which keeps all 64 tokens) are finished one by one after the first half, lane = rank (dequant_tile_by_rank
+    // below: a dozen instructions per tile); only with more than kDirectMax of them does the stage take the second half.
+    constexpr int kDirectMax = 4;
+    uint32_t long_tiles;
     {
         const uint32_t t = (uint32_t)(lane < 32 ? lane : 31);
         const uint32_t o = lds_load_u32(meta + t * 4u);
         const uint32_t nx = lane < 31 ? lds_load_u32(meta + t * 4u + 4u) : end_word;
-        need_high = __ballot(lane < 32 && nx - o > (uint32_t)kHalfSlots) != 0ull;
+        long_tiles = (uint32_t)__ballot(lane < 32 && nx - o > (uint32_t)kHalfSlots);
     }
+    const bool need_high = __builtin_popcount(long_tiles) > kDirectMax;
 #pragma unroll
     for (int hp = 0; hp < 2 * kHalfPasses; hp++) {
         const int half = hp / kHalfPasses, p = hp % kHalfPasses;
@@ -170,6 +175,30 @@ __device__ __forceinline__ void dequant_stage(uint32_t meta, uint32_t words, uin
                     dequant_exact(q, (sc >> sel) & 0xffffu, (zp >> sel) & 0xffffu, mode);
             }
         }
+    }
+    if (need_high) return;
+    // the long tiles one by one: lane = rank r reads code r of the tile and writes image slot r (the slots of the first
+    // half are written again with the same values; ranks beyond the tile's count land in slots no gather points to)
+    while (long_tiles != 0u) {
+        const uint32_t tl = (uint32_t)__builtin_ctz(long_tiles);
+        long_tiles &= long_tiles - 1u;
+        const uint32_t off = lds_load_u32(meta + tl * 4u);
+        const uint32_t sc = G32 ? lds_load_u32(meta + 128u + tl * 4u) : lds_load_u16(meta + 128u + tl * 2u);
+        const uint32_t zp = G32 ? lds_load_u32(meta + 256u + tl * 4u) : lds_load_u16(meta + 192u + tl * 2u);
+        const uint32_t r = (uint32_t)lane;
+        const uint32_t w = lds_load_u32(words + (off - start_word + (r >> F::kCapShift)) * 4u);
+        const uint32_t q = (w >> ((r & (uint32_t)(F::kCap - 1)) * (uint32_t)BIT)) & ((1u << BIT) - 1u);
+        uint32_t sel = 0u;  // G32: the first popcount(upper bitmap half) codes belong to the first pair
+        if (G32) sel = r >= (uint32_t)__builtin_popcount(lds_load_u32(meta + 384u + tl * 4u)) ? 16u : 0u;
+        const uint32_t s1 = (sc >> sel) & 0xffffu, z1 = (zp >> sel) & 0xffffu;
+        _Float16 val;
+        if ((z1 & 0x7fffu) <= 0x6400u) {
+            const _Float16 nb = (_Float16)(-1024.0f) - as_h((uint16_t)z1);  // exact: |zero| <= 1024
+            val = (as_h((uint16_t)(0x6400u | q)) + nb) * as_h((uint16_t)s1);
+        } else {
+            val = dequant_exact(q, s1, z1, mode);
+        }
+        *(MSTF_LDS _Float16*)(uintptr_t)(img + tl * (uint32_t)kImgStride + r * 2u) = val;
     }
 }
 

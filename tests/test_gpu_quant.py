@@ -160,14 +160,17 @@ def test_quant_decode_attention_against_dense_masked_oracle(bit, groups, Bkv, Lc
 @pytest.mark.parametrize("group_size", [64, 32])
 @pytest.mark.parametrize("bit", [2, 4, 8])
 @pytest.mark.parametrize("dequant_mode", [0, 1])
-def test_quant_dequantised_values_bit_exact(bit, dequant_mode, group_size):
+@pytest.mark.parametrize("kth", [89, 38])
+def test_quant_dequantised_values_bit_exact(bit, dequant_mode, group_size, kth):
     """One-hot query rows / probability rows turn the SpMVs into a read-out of the dequantised cache: every
     output is a single product value * 1, so it must equal the oracle's decode bit for bit.  Some tiles sit far
-    from zero (zero-point beyond +-1024), which takes the kernels' literal per-mode arithmetic."""
+    from zero (zero-point beyond +-1024), which takes the kernels' literal per-mode arithmetic.  kth 89: a stage
+    holds a few tiles with more than 32 survivors (outlier channels, the full tiles set below), finished one by one;
+    kth 38: most tiles have more than 32 and the stage takes the second half of the dequantisation."""
     from mustafar_amd import compression_quant as cq
     from mustafar_amd import mustafar_package_quant as mpq
     B, M, D, groups = 2, 128, 128, 4
-    Kp, Vp = pruned(57 + bit, B, M)
+    Kp, Vp = pruned(57 + bit, B, M, kth)
     k = np.arange(64)
     steps = {2: 3, 4: 10, 8: 64}[bit]          # spread chosen so that |zero| lands between 1024 and 8192
     Kp[1, :64, 5] = (300.0 + (k % steps) * (0.25 if bit < 8 else 0.5)).astype(np.float16)     # zero << -1024
