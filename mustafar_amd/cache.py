@@ -522,11 +522,10 @@ class QuantSparseKVCache(SparseKVCache):
     def _compress(self, K, V):
         from . import compression_quant as cq
         bs, n_kv, M, D = K.shape
-        Kp = ops.prune_rows(K.reshape(-1, D).contiguous(), self.kth_k).view(bs * n_kv, M, D)
-        Vp = ops.prune_rows(V.reshape(-1, D).contiguous(), self.kth_v).view(bs * n_kv, M, D)
-        ws = self._workspace(K.device)
-        return (list(cq.convert_key_batched_quant(Kp, return_metadata=True, bit=self.bit, ws=ws)),
-                list(cq.convert_value_batched_quant(Vp, bit=self.bit, ws=ws)))
+        ws = self._workspace(K.device)   # the pruning runs inside the producer: one read of the dense rows
+        return (list(cq.convert_key_batched_quant(K.reshape(bs * n_kv, M, D), return_metadata=True, bit=self.bit, ws=ws,
+                                                  kth=self.kth_k)),
+                list(cq.convert_value_batched_quant(V.reshape(bs * n_kv, M, D), bit=self.bit, ws=ws, kth=self.kth_v)))
 
     @staticmethod
     def _append(old, new):

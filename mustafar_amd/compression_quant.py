@@ -3,7 +3,7 @@ convert_value_batched_quant :425-529): same arguments and return tuples.  The re
 2-bit codes; `bit` is exposed here as an extra keyword (2, 4 or 8; capacity = 32 // bit), and `group_size`
 (64 = one scale / zero pair per tile as in the reference; 32 = two, scales and zeros then [B, T, 2]).
 
-inputs: [B, M, N] fp16 on the GPU, already pruned, M % 64 == 0.
+inputs: [B, M, N] fp16 on the GPU, already pruned (or pruned here: `kth`), M % 64 == 0.
 """
 import torch
 
@@ -65,12 +65,14 @@ def _convert(inputs, is_value, bit, kth=0, group_size=64, ws=None):
 
 
 def convert_key_batched_quant(inputs: torch.Tensor, return_metadata: bool = False, bit: int = 2, group_size: int = 64,
-                              ws=None):
-    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit, group_size=group_size, ws=ws)
+                              ws=None, kth: int = 0):
+    """kth > 0 (an extra of this build): the rows are pruned to that rank inside the producer, as dh_prune_key would
+    have done in front of it (models/llama_mustafar_quant_kernel.py), with one read of the dense rows."""
+    bmp, tile_off, packed, counts, units, scales, zeros = _convert(inputs, False, bit, kth, group_size, ws)
     if return_metadata:
         return bmp, tile_off, packed, counts, units, scales, zeros
     return bmp, tile_off, packed, scales, zeros
 
 
-def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2, group_size: int = 64, ws=None):
-    return _convert(inputs, True, bit, group_size=group_size, ws=ws)
+def convert_value_batched_quant(inputs: torch.Tensor, bit: int = 2, group_size: int = 64, ws=None, kth: int = 0):
+    return _convert(inputs, True, bit, kth, group_size, ws)
