@@ -183,7 +183,9 @@ class QuantPool:
         self.bmp_store, self.off_store = store(torch.int64), store(torch.int32)
         self.counts_store, self.units_store = store(torch.int32), store(torch.int32)
         self.scales_store, self.zeros_store = store(torch.float16), store(torch.float16)
-        self.packed = torch.zeros(heads * max_tokens * head_dim * bit // 32, dtype=torch.int32, device=device)
+        words = heads * max_tokens * head_dim * bit // 32
+        assert words < 2 ** 31, "tile offsets are 32-bit word offsets into one buffer, as in the reference's format"
+        self.packed = torch.zeros(words, dtype=torch.int32, device=device)
         self.reserved = 0            # words handed out to chunks so far
         self.tokens_dev = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens = 0
