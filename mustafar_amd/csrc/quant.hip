@@ -419,6 +419,8 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
     if (B <= 0 || M <= 0 || N <= 0 || kth < 0 || kth > N) return MSTF_EINVAL;
     if (cap_shift_of(bit) < 0) return MSTF_EUNSUPPORTED;
     if (N != kD || M % 64 != 0 || M / 64 > 8192 || (int64_t)B * (M / 64) > 0x7FFFFFFF) return MSTF_EUNSUPPORTED;
+    // tile offsets are 32-bit word offsets into one buffer (the reference's format): the worst case has to fit
+    if ((uint64_t)B * (uint64_t)M * (uint64_t)N / 64u * (uint64_t)(64 * bit / 32) > 0xFFFFFFFFull) return MSTF_EUNSUPPORTED;
     if (!aligned_to(x, 16) || !aligned_to(bmp, 8) || !aligned_to(tile_off, 4) || !aligned_to(counts, 4) ||
         !aligned_to(units, 4) || !aligned_to(scales, G32 ? 4 : 2) || !aligned_to(zeros, G32 ? 4 : 2) || !aligned_to(total_words, 8) ||
         (packed && !aligned_to(packed, 4)))
