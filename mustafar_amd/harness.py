@@ -197,6 +197,12 @@ class Decoder:
     def step(self, ids, position, timed=False):
         """ids: [bs, 1] -> logits [bs, 1, vocab]."""
         pos = torch.tensor([position], device=self.dev)
+        if all(getattr(c, "window_kernel", False) for c in self.caches):
+            # the caches take the projection output as it is (one launch for rotation, query layout and window append)
+            logits = self._layers(ids, pos, timed, None, from_proj=True)
+            for cache in self.caches:
+                cache.advance()
+            return logits
         return self._layers(ids, pos, timed, lambda cache, q, k, v: cache.decode(q, k, v))
 
     def _layers(self, ids, pos, timed, attend, from_proj=False):
