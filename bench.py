@@ -11,8 +11,8 @@ reads come from HBM, not from the 256 MB Infinity Cache.  Prints exactly one JSO
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sparsity 0.7] [--no-cpu] [--unfused] [--no-configs]
 
 Beside the headline the line carries `configs`: the other benchmark configurations measured in the same run
-(configs[1] at 50 %, configs[2] compressors at batch 16, configs[3] quantised decode at batch 32, a short configs[4]
-decode loop); every kernel time in the line is the GPU time of launches replayed from HIP graphs on rotating caches.
+(configs[1] at 50 %, configs[2] compressors at batch 16, configs[3] quantised decode at batch 32, the configs[4]
+decode loop over its 256 new tokens); every kernel time in the line is the GPU time of launches replayed from HIP graphs on rotating caches.
 """
 import argparse
 import json
@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_attention_bs8_ctx4096_s70_traffic.txt")
+KSTATS_FILE = os.path.join(ROOT, "profiles", "decode_attention_bs8_ctx4096_s70_kernel_stats.md")
 
 
 def measured_traffic(args):
@@ -36,6 +37,17 @@ def measured_traffic(args):
     for line in open(TRAFFIC_FILE):
         if line.startswith("traffic_bytes_per_launch:"):
             return int(float(line.split(":", 1)[1]))
+    return None
+
+
+def profiled_launch_us(args):
+    """Average duration of the fused kernel in the committed rocprofv3 --kernel-trace --stats summary of this command
+    (default workload only): carried in the line beside the live HIP-event average."""
+    if (args.batch, args.ctx, args.sparsity, args.unfused) != (8, 4096, 0.7, False) or not os.path.exists(KSTATS_FILE):
+        return None
+    for line in open(KSTATS_FILE):
+        if line.startswith("rocprof_avg_launch_us:"):
+            return float(line.split(":", 1)[1])
     return None
 
 
@@ -276,14 +288,15 @@ def quant_record(torch, ops, dev, gen, bs, L, sparsity, bit, group_size, reps):
 
 
 def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens, cache="sparse"):
-    """configs[4], shortened: random-init Llama-3-8B shape, greedy decoding with the step replayed from a HIP graph
-    (tokens/s) and a few eager steps with events around the cache's attention (its share of the step)."""
+    """configs[4]: random-init Llama-3-8B shape, greedy decoding of new_tokens tokens with the step replayed from a
+    HIP graph (tokens/s; the 256-token chunk that the window sheds on the way is pruned, compressed and appended
+    inside the timed region) and a few eager steps with events around the cache's attention (its share of the step)."""
     import time as _time
-    from mustafar_amd.cache import CHUNK
-    from mustafar_amd.harness import Config, Decoder, GraphedGreedyLoop
+    from mustafar_amd.harness import Config, Decoder, GraphedGreedyLoop, pool_tokens
     cfg = Config(layers=layers)
-    max_tokens = ((prompt + new_tokens + 16 + CHUNK - 1) // CHUNK) * CHUNK
-    dec = Decoder(cfg, dev, cache=cache, sparsity=0.7, residual_length=256, max_tokens=max_tokens)
+    eager_steps, warm_eager, warm_graph = 6, 2, 4
+    total = prompt + warm_eager + eager_steps + warm_graph + new_tokens
+    dec = Decoder(cfg, dev, cache=cache, sparsity=0.7, residual_length=256, max_tokens=pool_tokens(total))
     g = torch.Generator(device=dev)
     g.manual_seed(1)
     ids = torch.randint(0, cfg.vocab, (batch, prompt), generator=g, device=dev)
@@ -295,18 +308,18 @@ def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens, cache="spa
     torch.cuda.synchronize()
     t_prefill = _time.perf_counter() - t0
     nxt = logits[:, -1].argmax(-1, keepdim=True)
-    eager_steps = 6
-    for t in range(2):
+    for t in range(warm_eager):
         nxt = dec.step(nxt, prompt + t)[:, -1].argmax(-1, keepdim=True)
     torch.cuda.synchronize()
     t0 = _time.perf_counter()
-    for t in range(2, 2 + eager_steps):
+    for t in range(warm_eager, warm_eager + eager_steps):
         nxt = dec.step(nxt, prompt + t, timed=True)[:, -1].argmax(-1, keepdim=True)
     torch.cuda.synchronize()
     t_eager = (_time.perf_counter() - t0) / eager_steps
     attn_ms = sum(a.elapsed_time(b) for a, b in dec.attn_events) / eager_steps
-    loop = GraphedGreedyLoop(dec, nxt, prompt + 2 + eager_steps)
-    for _ in range(4):
+    loop = GraphedGreedyLoop(dec, nxt, prompt + warm_eager + eager_steps)
+    loop.append_events = []
+    for _ in range(warm_graph):
         loop.step()
     torch.cuda.synchronize()
     t0 = _time.perf_counter()
@@ -314,13 +327,26 @@ def decode_loop_record(torch, dev, layers, batch, prompt, new_tokens, cache="spa
         loop.step()
     torch.cuda.synchronize()
     t_step = (_time.perf_counter() - t0) / new_tokens
+    appends = [a.elapsed_time(b) for a, b in loop.append_events]
+    pool_b = sum(c.kv_bytes()[0] for c in dec.caches)
+    win_b = sum(c.kv_bytes()[1] for c in dec.caches)
+    heads = batch * cfg.n_kv
+    dense_pool = 2 * layers * heads * dec.caches[0].max_tokens * cfg.head_dim * 2       # the pools' token capacity, dense
+    dense_all = 2 * layers * heads * total * cfg.head_dim * 2        # every token of the run, dense
     return {"cache": cache, "layers": layers, "batch": batch, "prompt": prompt, "new_tokens_timed": new_tokens,
             "prefill_s": round(t_prefill, 3),
             "graphed_decode_ms_per_step": round(1e3 * t_step, 3), "tokens_per_s": round(batch / t_step, 1),
             "graph_captures": loop.captures, "eager_decode_ms_per_step": round(1e3 * t_eager, 3),
             "eager_attention_over_cache_ms_per_step": round(attn_ms, 3),
             "eager_attention_share": round(attn_ms / (1e3 * t_eager), 4),
-            "compressed_tokens_at_end": dec.caches[0].compressed_length}
+            "chunk_appends_in_timed_region": len(appends),
+            "chunk_append_ms_all_layers": [round(a, 3) for a in appends],
+            "compressed_tokens_at_end": dec.caches[0].compressed_length,
+            "kv_bytes_allocated": int(pool_b), "kv_bytes_dense": int(dense_pool),
+            "kv_allocated_over_dense": round(pool_b / dense_pool, 4),
+            "kv_bytes_window_buffers": int(win_b),
+            "kv_pools_plus_windows_over_dense_of_all_tokens": round((pool_b + win_b) / dense_all, 4),
+            "pool_growths": sum(c.k_pool.generation + c.v_pool.generation for c in dec.caches)}
 
 
 def main():
@@ -472,8 +498,20 @@ def main():
             Kd, Vd = dense[i]
             return F.scaled_dot_product_attention(q4, Kd.view(bs, nkv, L, D), Vd.view(bs, nkv, L, D), enable_gqa=True)
 
+        # the floor any dense kernel has: a plain read of the same K and V bytes (16 bytes per lane, nothing else)
+        from mustafar_amd._lib import lib as _lib_, check as _check_
+        sink = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+        nb = Bkv * L * D * 2
+
+        def dense_read(i):
+            st = torch.cuda.current_stream().cuda_stream
+            for t in dense[i]:
+                _check_(_lib_().mstf_probe_read(st, t.data_ptr(), nb, sink.data_ptr(), 4096), "mstf_probe_read")
+
         dense_us = {"matmul_softmax_matmul": round(ring_time_us(torch, dense_matmul, args.caches, reps), 2),
-                    "sdpa": round(ring_time_us(torch, dense_sdpa, args.caches, reps), 2), "bytes": int(2 * Bkv * L * D * 2)}
+                    "sdpa": round(ring_time_us(torch, dense_sdpa, args.caches, reps), 2),
+                    "plain_read_of_k_and_v": round(ring_time_us(torch, dense_read, args.caches, reps), 2),
+                    "bytes": int(2 * Bkv * L * D * 2)}
     del dense
 
     quant_here = {}
@@ -499,9 +537,9 @@ def main():
         torch.cuda.empty_cache()
         if args.loop_layers > 0:
             try:
-                configs["configs4_decode_loop"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 32)
+                configs["configs4_decode_loop"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 256)
                 torch.cuda.empty_cache()
-                configs["configs4_decode_loop_2bit"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 32,
+                configs["configs4_decode_loop_2bit"] = decode_loop_record(torch, dev, args.loop_layers, 16, 4096, 256,
                                                                           cache="sparse_quant2")
             except Exception as e:  # pragma: no cover - e.g. out of memory on a shared box; reported, not fatal
                 configs.setdefault("configs4_decode_loop", {"error": str(e)[:200]})
@@ -559,6 +597,8 @@ def main():
         "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
                       "prune_compress_key_ctx": comp["key"]["us"], "prune_compress_value_ctx": comp["value"]["us"]},
+        # BASELINE configs[1] asks for the compression of the cached context timed with the step: their sum
+        "configs1_total_us": round(comp["key"]["us"] + comp["value"]["us"] + wall_us, 2),
         "compress": comp,
         "quant_stages_us": quant_here,
         "dense_fp16_attention_us": dense_us,
@@ -570,7 +610,11 @@ def main():
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args),
                      "traffic_source": "profiles/decode_attention_bs8_ctx4096_s70_traffic.txt (rocprofv3 --pmc runs of this "
                                        "command, calibrated on the copy this run ends with)",
-                     "algorithmic_bytes": int(dom_bytes), "avg_launch_us": round(dom_us, 2)},
+                     "algorithmic_bytes": int(dom_bytes), "avg_launch_us": round(dom_us, 2),
+                     "avg_launch_us_source": "HIP events over graph replays in this run",
+                     "rocprof_avg_launch_us": profiled_launch_us(args),
+                     "rocprof_source": "profiles/decode_attention_bs8_ctx4096_s70_kernel_stats.md (rocprofv3 "
+                                       "--kernel-trace --stats of this command)"},
         "configs": configs,
     }
     if not args.no_cpu:

@@ -53,6 +53,11 @@ int mstf_version(void);
  * practically impossible case that the xor of all data read by a workgroup hits a fixed constant).  Timing it gives the
  * plain-read time of a buffer of that size on the box at hand. */
 int mstf_probe_read(void* stream, const void* src, size_t bytes, uint32_t* sink, int workgroups);
+/* Test aid (no counterpart in the reference): the number of polls a workgroup of the one-pass producers
+ * (mstf_compress_*, mstf_append_*, mstf_compress_*_quant*) spends on a wait before it gives up and marks the call.
+ * polls < 0 restores the default (2^20).  Process-wide, read at every launch; nothing in the environment changes it.
+ * A test sets it to 0 to drive the give-up path from the host while every kernel still runs to its end. */
+void mstf_test_set_spin_limit(int64_t polls);
 
 /* ------------------------------------------------------------------ pruning (A1)
  * Replaces dh_prune_key / dh_prune_value (models/llama_mustafar_kernel.py:194-274):
@@ -71,8 +76,10 @@ int mstf_prune_rows_f16(void* stream, const mstf_half* x, mstf_half* y, int64_t 
  * mstf_compress_*_f16 produces everything with one read of x (status words in the workspace order
  * the workgroups; they are cleared by the call itself); with nz == NULL it runs phase 1 only.  Tiles
  * whose values would not fit in nz_capacity_halfs are not written (compare *total_halfs afterwards).
- * A workgroup waits for the totals of the workgroups launched before it; should such a wait ever run
- * out of its (bounded) polls, no values are written for it and *total_halfs reads as all ones. */
+ * A workgroup waits for the totals of the workgroups launched before it; should such a wait of ANY workgroup
+ * ever run out of its (bounded) polls, that workgroup writes no values and *total_halfs reads as all ones
+ * (the call clears *total_halfs first and raises it with atomic maxima, so the marker survives whichever
+ * workgroup finishes last). */
 size_t mstf_compress_workspace_bytes(int B, int M, int N);
 int mstf_compress_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp,
                           uint32_t* idx, uint32_t* nz_off, uint64_t* total_halfs, mstf_half* nz,
@@ -91,8 +98,14 @@ int mstf_scatter_value_f16(void* stream, const mstf_half* x, int B, int M, int N
  * nz + 16 * dst_off[b] and must end at or before nz + 16 * dst_limit[b] (both in 16-byte units).  With one slab
  * per head and dst_off[b] = slab start + idx_so_far[b][T] / 4 the cache grows in place; the format's nz_off[b]
  * is the slab start.  bmp[B, M*N/64] and idx[B, M*N/64 + 1] receive the chunk's bitmaps and its offsets counted
- * from the chunk's first value (add idx_so_far[b][T]).  A unit that would pass its head's limit is not written
- * and *overflow (sticky, zeroed by the caller) is set to 1.  Workspace as for mstf_compress_*_f16. */
+ * from the chunk's first value (add idx_so_far[b][T]).  *overflow is a sticky flag word zeroed by the caller:
+ * bit 0 (MSTF_APPEND_OVERFLOW) is set when a unit would pass its head's limit - that unit's values are not
+ * written; the chunk's bitmaps and offsets are, and appending the same chunk again with larger slabs repairs it -
+ * and bit 1 (MSTF_APPEND_GAVE_UP) when a workgroup's bounded wait for the workgroups in front of it ran out, in
+ * which case it wrote no values (the marker *total_halfs carries in the compress contract).  A caller must look
+ * at the word before it trusts the appended chunk.  Workspace as for mstf_compress_*_f16. */
+#define MSTF_APPEND_OVERFLOW 1u
+#define MSTF_APPEND_GAVE_UP 2u
 int mstf_append_key_f16(void* stream, const mstf_half* x, int B, int M, int N, int kth, uint64_t* bmp, uint32_t* idx,
                         const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow,
                         void* workspace, size_t workspace_bytes);
@@ -275,7 +288,8 @@ int mstf_window_append_f16(void* stream, const mstf_half* q_in, int64_t q_stride
  *   zero = floor(-min / scale + 0.5); code = clamp(floor(v / scale + 0.5) + zero, 0, 2^bit - 1);
  *   code j of a tile sits at bits bit*(j % capacity) of word j / capacity.
  * kth as in mstf_compress_*_f16.  packed == NULL runs the sizing phase only; with packed the input is read once and
- * the workgroups are ordered as in mstf_compress_*_f16 (*total_words reads as all ones should a bounded wait run out). */
+ * the workgroups are ordered as in mstf_compress_*_f16 (*total_words reads as all ones should a bounded wait of any
+ * workgroup run out). */
 size_t mstf_compress_quant_workspace_bytes(int B, int M, int N);
 int mstf_compress_key_quant(void* stream, const mstf_half* x, int B, int M, int N, int kth, int bit, uint64_t* bmp,
                             uint32_t* tile_off, uint32_t* counts, uint32_t* units, mstf_half* scales,

@@ -35,6 +35,7 @@ SIGNATURES = {
     "mstf_last_hip_error": (_i, []),
     "mstf_version": (_i, []),
     "mstf_probe_read": (_i, [_vp, _vp, _sz, _vp, _i]),
+    "mstf_test_set_spin_limit": (None, [_i64]),
     "mstf_prune_rows_f16": (_i, [_vp, _vp, _vp, _i64, _i, _i]),
     "mstf_compress_workspace_bytes": (_sz, [_i, _i, _i]),
     "mstf_compress_key_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _sz]),

@@ -50,35 +50,52 @@ def append_compressed(old, new):
                             total)
 
 
+def slab_fraction_for(kth, head_dim):
+    """Slab size, relative to the dense size, that holds any cache pruned to rank kth whose rows have no ties at the
+    threshold: D - kth + 1 survivors per row plus the worst padding of every 64-element tile (7 values).  Ties add
+    survivors (an all-equal row keeps everything), so a pool this size can still overflow: it then grows."""
+    keep = (head_dim - int(kth) + 1) / head_dim if kth > 0 else 1.0
+    return min(1.0, keep + 7.0 / 64.0)
+
+
 class CompressedPool:
     """One side (keys or values) of a compressed cache that grows in place.
 
     Every head owns a slab of the packed-value pool (nz_off[b] = start of slab b, which the format allows); a chunk
     is compressed straight to the end of each head's values by mstf_append_*_f16, so appending re-copies no packed
-    values, reads nothing back to the host and launches the same kernels whatever the cache holds.  The per-tile
-    arrays are pre-allocated for max_tokens too (bmp_store [heads, tile_capacity], idx_store [heads, tile_capacity + 1])
-    and a chunk's bitmaps and offsets are written behind the ones that are there, so no array of the pool ever moves;
-    the number of tokens held is mirrored in device memory (tokens_dev) for consumers recorded into a HIP graph
-    (ops.decode_attention_window_pool).
+    values and launches the same kernels whatever the cache holds.  The per-tile arrays are pre-allocated for
+    max_tokens too (bmp_store [heads, tile_capacity], idx_store [heads, tile_capacity + 1]) and a chunk's bitmaps and
+    offsets are written behind the ones that are there; the number of tokens held is mirrored in device memory
+    (tokens_dev) for consumers recorded into a HIP graph (ops.decode_attention_window_pool).
 
-    slab_fraction: slab size relative to the dense size of max_tokens tokens (1.0 can never overflow; smaller
-    saves memory and is guarded by the sticky `overflow` flag: check_overflow() raises once it is set)."""
+    slab_fraction: slab size relative to the dense size of max_tokens tokens.  1.0 can never overflow; smaller saves
+    memory (slab_fraction_for(kth, head_dim) holds every cache without ties at the pruning threshold: 0.42 of dense at
+    70 % sparsity, so that values + bitmaps + offsets come to 0.52 of the dense bytes).  Every append reads the call's
+    flag word back once (the host is between two decode steps there anyway): a chunk that did not fit a head's slab
+    makes the pool grow - new, larger slabs, the old ones copied over, the same chunk appended again - and
+    `generation` counts such moves (a HIP graph that holds the pool's addresses must then be captured again); a
+    producer workgroup that gave up its bounded wait raises."""
 
     def __init__(self, heads, head_dim, max_tokens, is_value, device, slab_fraction=1.0):
-        assert max_tokens % 64 == 0
+        assert max_tokens % 64 == 0 and 0.0 < slab_fraction <= 1.0
         self.heads, self.head_dim, self.is_value, self.max_tokens = heads, head_dim, is_value, max_tokens
-        self.slab_fraction = slab_fraction
-        slab16 = (int(math.ceil(max_tokens * head_dim * 2 * slab_fraction)) + 15) // 16
-        self.slab16 = slab16
-        self.nz = torch.zeros(heads * slab16 * 8, dtype=torch.float16, device=device)
-        self.nz_off = (torch.arange(heads, device=device, dtype=torch.int64) * slab16).to(torch.int32)
-        self.limit = (self.nz_off.to(torch.int64) + slab16).to(torch.int32)
+        self.device = device
+        self.dense16 = max_tokens * head_dim * 2 // 16
+        self.generation = 0
+        self._alloc_slabs(max(1, min(self.dense16, (int(math.ceil(max_tokens * head_dim * 2 * slab_fraction)) + 15) // 16)))
         self.tile_capacity = max_tokens * head_dim // 64
         self.bmp_store = torch.zeros((heads, self.tile_capacity), dtype=torch.int64, device=device)
         self.idx_store = torch.zeros((heads, self.tile_capacity + 1), dtype=torch.int32, device=device)
         self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens_dev = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens = 0
+
+    def _alloc_slabs(self, slab16):
+        self.slab16 = slab16
+        self.slab_fraction = slab16 / self.dense16
+        self.nz = torch.zeros(self.heads * slab16 * 8, dtype=torch.float16, device=self.device)
+        self.nz_off = (torch.arange(self.heads, device=self.device, dtype=torch.int64) * slab16).to(torch.int32)
+        self.limit = (self.nz_off.to(torch.int64) + slab16).to(torch.int32)
 
     @property
     def tiles(self):
@@ -93,6 +110,10 @@ class CompressedPool:
     def idx(self):
         return self.idx_store[:, :self.tiles + 1]
 
+    def allocated_bytes(self):
+        """Device bytes the pool holds: packed values, bitmaps, offsets."""
+        return self.nz.numel() * 2 + self.bmp_store.numel() * 8 + self.idx_store.numel() * 4 + self.nz_off.numel() * 8
+
     def _publish(self, bmp_c, idx_c, M):
         """Writes a chunk's bitmaps and offsets (counted from the chunk's first value) behind the ones held."""
         T0, Tc = self.tiles, bmp_c.shape[1]
@@ -101,11 +122,38 @@ class CompressedPool:
         self.tokens += M
         self.tokens_dev += M
 
-    def check_overflow(self):
-        """Raises if a chunk did not fit into a head's slab (possible only with slab_fraction < 1; one host read)."""
-        if self.slab_fraction < 1.0 and int(self.overflow) != 0:
-            raise RuntimeError("compressed pool overflow: a head's packed values outgrew its slab "
-                               "(slab_fraction %.2f); the cache is no longer usable" % self.slab_fraction)
+    def _grow_slabs(self):
+        """After a chunk that did not fit: slabs large enough for what the heads hold now (the chunk's offsets were
+        published although its values were not written), scaled to the capacity in tokens, at least a quarter more."""
+        need16 = (int(self.idx_store[:, self.tiles].max().item()) + 3) // 4
+        scaled = int(math.ceil(need16 * (self.max_tokens / self.tokens) * 1.0625))
+        new16 = min(self.dense16, max(scaled, int(math.ceil(self.slab16 * 1.25)), need16))
+        if new16 <= self.slab16:
+            raise RuntimeError("compressed pool overflow at the dense slab size: the appended rows are not [*, %d] fp16 "
+                               "tokens of this pool" % self.head_dim)
+        old, old16 = self.nz, self.slab16
+        self._alloc_slabs(new16)
+        self.nz.view(self.heads, new16 * 8)[:, :old16 * 8].copy_(old.view(self.heads, old16 * 8))
+        self.generation += 1
+
+    def _append_checked(self, launch, M):
+        """launch(): one append call for the chunk at the pool's current end, published.  Reads the flag word back,
+        grows and appends again on overflow."""
+        launch()
+        for attempt in range(2):
+            flag = int(self.overflow.item())
+            if flag & 2:
+                raise RuntimeError("the compressor gave up waiting for an earlier workgroup; the appended chunk is "
+                                   "incomplete and the pool is no longer usable")
+            if not (flag & 1):
+                return
+            if attempt == 1:
+                raise RuntimeError("compressed pool overflow after growing")
+            self.overflow.zero_()
+            self._grow_slabs()
+            self.tokens -= M          # the chunk is appended again at the same place
+            self.tokens_dev -= M
+            launch()
 
     def append(self, x, kth, ws=None):
         """x: [heads, M, head_dim] fp16, M % 64 == 0.  ws: the caller's ops.Workspace (default: the stream's)."""
@@ -114,15 +162,19 @@ class CompressedPool:
         x = x.contiguous()
         L = lib()
         Tc = M * N // 64
-        bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
-        idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
-        dst = self.nz_off + self.idx_store[:, self.tiles] // 4          # 16-byte units; idx counts 4-byte units
-        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, M, N), ws)
+        wsb = L.mstf_compress_workspace_bytes(B, M, N)
         fn = L.mstf_append_value_f16 if self.is_value else L.mstf_append_key_f16
-        check(fn(torch.cuda.current_stream().cuda_stream, x.data_ptr(), B, M, N, int(kth), bmp_c.data_ptr(),
-                 idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(), self.overflow.data_ptr(),
-                 ws.data_ptr(), ws.numel()), "mstf_append_f16")
-        self._publish(bmp_c, idx_c, M)
+
+        def launch():
+            bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
+            idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
+            dst = self.nz_off + self.idx_store[:, self.tiles] // 4          # 16-byte units; idx counts 4-byte units
+            w = ops.workspace(x.device, wsb, ws)
+            check(fn(torch.cuda.current_stream().cuda_stream, x.data_ptr(), B, M, N, int(kth), bmp_c.data_ptr(),
+                     idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(), self.overflow.data_ptr(),
+                     w.data_ptr(), w.numel()), "mstf_append_f16")
+            self._publish(bmp_c, idx_c, M)
+        self._append_checked(launch, M)
 
     def append_proj(self, x, kth, M, cos=None, sin=None, rot=None, ws=None):
         """The first M tokens of x [batch, rows, heads per batch entry, head_dim] (a view of the projection output,
@@ -134,16 +186,27 @@ class CompressedPool:
         assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
         L = lib()
         Tc = M * N // 64
-        bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
-        idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
-        dst = self.nz_off + self.idx_store[:, self.tiles] // 4
-        ws = ops.workspace(x.device, L.mstf_compress_workspace_bytes(B, max(M, 64), N), ws)
-        check(L.mstf_append_proj_f16(torch.cuda.current_stream().cuda_stream, ctypes.byref(src), int(self.is_value), M, N,
-                                     int(kth), bmp_c.data_ptr(), idx_c.data_ptr(), dst.data_ptr(), self.limit.data_ptr(),
-                                     self.nz.data_ptr(), self.overflow.data_ptr(), ws.data_ptr(), ws.numel()),
-              "mstf_append_proj_f16")
+        wsb = L.mstf_compress_workspace_bytes(B, max(M, 64), N)
+        state = {"src": src}
+
+        def launch():
+            bmp_c = torch.empty((B, Tc), dtype=torch.int64, device=x.device)
+            idx_c = torch.empty((B, Tc + 1), dtype=torch.int32, device=x.device)
+            dst = self.nz_off + self.idx_store[:, self.tiles] // 4
+            w = ops.workspace(x.device, wsb, ws)
+            check(L.mstf_append_proj_f16(torch.cuda.current_stream().cuda_stream, ctypes.byref(state["src"]),
+                                         int(self.is_value), M, N, int(kth), bmp_c.data_ptr(), idx_c.data_ptr(),
+                                         dst.data_ptr(), self.limit.data_ptr(), self.nz.data_ptr(),
+                                         self.overflow.data_ptr(), w.data_ptr(), w.numel()), "mstf_append_proj_f16")
+            if M > 0:
+                self._publish(bmp_c, idx_c, M)
+            # a second attempt (after growing) finds the rows already rotated where `rot` put them
+            if cos is not None:
+                state["src"], _ = ops.proj_source(rot)
         if M > 0:
-            self._publish(bmp_c, idx_c, M)
+            self._append_checked(launch, M)
+        else:
+            launch()
         return rot
 
     def view(self):
@@ -158,21 +221,38 @@ class CompressedPool:
         return self.nz[start:start + n]
 
 
+def packed_fraction_for(kth, head_dim, bit):
+    """Word-buffer size of a QuantPool, relative to the worst case (every element kept), that holds any cache pruned
+    to rank kth without ties at the threshold: per 64-token block 64 * (D - kth + 1) codes in D tiles, each tile
+    rounded up to whole words of 32 / bit codes."""
+    if kth <= 0:
+        return 1.0
+    cap = 32 // bit
+    tiles = head_dim                # tiles of one side of a 64-token block
+    codes = 64 * (head_dim - int(kth) + 1)
+    words = codes / cap + tiles * (cap - 1) / cap
+    return min(1.0, words / (tiles * 64 / cap))
+
+
 class QuantPool:
     """One side (keys or values) of a quantised cache that grows in place.
 
     Bitmaps, word offsets, counts, units, scales and zero-points are pre-allocated for max_tokens tokens
-    ([heads, tile_capacity] each) and so is the buffer of packed words, sized for the worst case (every element
-    kept).  A chunk is quantised straight into the next free region of that buffer - a region has room for the
-    chunk's worst case, so its start is known on the host and nothing is read back; the words a chunk does not need
-    stay unused, which the consumers allow: tile_off says where every tile's words are, and only the words of one
-    64-token block have to be contiguous - and its per-tile arrays are written behind the ones held, the offsets
-    shifted by the region's start.  No array ever moves (the reference concatenates all seven per chunk,
-    models/llama_mustafar_quant_kernel.py:322-345); the number of tokens held is mirrored in device memory
-    (tokens_dev) for consumers recorded into a HIP graph (mustafar_package_quant.decode_attention_window_quant_pool)."""
+    ([heads, tile_capacity] each) and so is the buffer of packed words, sized `packed_fraction` of the worst case
+    (every element kept; packed_fraction_for(kth, head_dim, bit) holds every cache without ties at the pruning
+    threshold: 0.55 of the worst case for 2-bit codes at 70 % sparsity).  A chunk is quantised straight behind the
+    words of the chunks before it - the producer's word total is read back once per append, which also tells a
+    producer that gave up - and its per-tile arrays are written behind the ones held, the offsets shifted by the
+    chunk's start.  A chunk that does not fit makes the buffer grow (a larger one, the old words copied, the chunk
+    quantised again; `generation` counts such moves); otherwise no array ever moves (the reference concatenates all
+    seven per chunk, models/llama_mustafar_quant_kernel.py:322-345).  The number of tokens held is mirrored in device
+    memory (tokens_dev) for consumers recorded into a HIP graph
+    (mustafar_package_quant.decode_attention_window_quant_pool)."""
 
-    def __init__(self, heads, head_dim, max_tokens, is_value, bit, device):
-        assert max_tokens % 64 == 0 and bit in (2, 4, 8)
+    SLACK_WORDS = 64     # behind the last word: the consumers fetch a block's words in 16-byte pieces
+
+    def __init__(self, heads, head_dim, max_tokens, is_value, bit, device, packed_fraction=1.0):
+        assert max_tokens % 64 == 0 and bit in (2, 4, 8) and 0.0 < packed_fraction <= 1.0
         self.heads, self.head_dim, self.is_value, self.max_tokens, self.bit = heads, head_dim, is_value, max_tokens, bit
         self.tile_capacity = max_tokens * head_dim // 64
         T = self.tile_capacity
@@ -183,26 +263,50 @@ class QuantPool:
         self.bmp_store, self.off_store = store(torch.int64), store(torch.int32)
         self.counts_store, self.units_store = store(torch.int32), store(torch.int32)
         self.scales_store, self.zeros_store = store(torch.float16), store(torch.float16)
-        words = heads * max_tokens * head_dim * bit // 32
-        assert words < 2 ** 31, "tile offsets are 32-bit word offsets into one buffer, as in the reference's format"
-        self.packed = torch.zeros(words, dtype=torch.int32, device=device)
-        self.reserved = 0            # words handed out to chunks so far
+        self.worst_words = heads * max_tokens * head_dim * bit // 32
+        assert self.worst_words < 2 ** 31, "tile offsets are 32-bit word offsets into one buffer, as in the reference's format"
+        self.capacity_words = max(1, min(self.worst_words, int(math.ceil(self.worst_words * packed_fraction))))
+        self.packed = torch.zeros(self.capacity_words + self.SLACK_WORDS, dtype=torch.int32, device=device)
+        self.generation = 0
+        self.reserved = 0            # words in use
         self.tokens_dev = torch.zeros(1, dtype=torch.int32, device=device)
         self.tokens = 0
-        self._totals = []            # the producers' word totals (device tensors), looked at by check()
 
     @property
     def tiles(self):
         return self.tokens * self.head_dim // 64
+
+    def allocated_bytes(self):
+        """Device bytes the pool holds: packed words and the six per-tile arrays."""
+        per_tile = sum(t.numel() * t.element_size() for t in (self.bmp_store, self.off_store, self.counts_store,
+                                                               self.units_store, self.scales_store, self.zeros_store))
+        return self.packed.numel() * 4 + per_tile
+
+    def _grow_packed(self, need_words, tokens_after):
+        scaled = int(math.ceil(need_words * (self.max_tokens / tokens_after) * 1.0625))
+        new_cap = min(self.worst_words, max(scaled, int(math.ceil(self.capacity_words * 1.25)), need_words))
+        if new_cap < need_words:
+            raise RuntimeError("quantised pool overflow at the worst-case buffer size")
+        old = self.packed
+        self.packed = torch.zeros(new_cap + self.SLACK_WORDS, dtype=torch.int32, device=old.device)
+        self.packed[:self.reserved].copy_(old[:self.reserved])
+        self.capacity_words = new_cap
+        self.generation += 1
 
     def append(self, x, kth, ws=None):
         """x: [heads, M, head_dim] fp16, M % 64 == 0, pruned here to rank kth (0: already pruned)."""
         from . import compression_quant as cq
         B, M, N = x.shape
         assert B == self.heads and N == self.head_dim and M % 64 == 0 and self.tokens + M <= self.max_tokens
-        region = B * M * N * self.bit // 32
-        room = self.packed[self.reserved:self.reserved + region]
-        bmp, off, _, counts, units, scales, zeros, total = cq._produce(x, self.is_value, self.bit, kth, 64, ws, room)
+        for attempt in range(2):
+            room = self.packed[self.reserved:self.capacity_words]
+            bmp, off, _, counts, units, scales, zeros, total = cq._produce(x, self.is_value, self.bit, kth, 64, ws, room)
+            words = cq.words_written(total)      # one host read; raises if the producer gave up
+            if words <= room.numel():
+                break
+            if attempt == 1:
+                raise RuntimeError("quantised pool overflow after growing")
+            self._grow_packed(self.reserved + words, self.tokens + M)   # the tiles that did not fit were left unwritten
         T0, Tc = self.tiles, bmp.shape[1]
         self.bmp_store[:, T0:T0 + Tc] = bmp
         self.off_store[:, T0:T0 + Tc] = off + self.reserved
@@ -210,17 +314,12 @@ class QuantPool:
         self.units_store[:, T0:T0 + Tc] = units
         self.scales_store[:, T0:T0 + Tc] = scales
         self.zeros_store[:, T0:T0 + Tc] = zeros
-        self.reserved += region
+        self.reserved += words
         self.tokens += M
         self.tokens_dev += M
-        self._totals.append(total)
 
     def check(self):
-        """Raises if a producer call gave up (one host read per call since the last check)."""
-        from . import compression_quant as cq
-        for t in self._totals:
-            cq.words_written(t)
-        self._totals = []
+        """Kept for callers of the earlier interface: every append already checks its own producer call."""
 
     def view(self):
         """The side as the reference's operators take it: [bitmaps, tile_offsets, packed, counts, units, scales,
@@ -233,10 +332,13 @@ class QuantPool:
 
 class SparseKVCache:
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, fused=False,
-                 max_tokens=0, window_kernel=False):
+                 max_tokens=0, window_kernel=False, pool_fraction=None):
         """fused: the compressed part of a decode step is one launch (ops.decode_attention) whose (max, sum) joins
         the dense window under one softmax, instead of the reference's key SpMV / softmax / value SpMV sequence.
         max_tokens > 0: the compressed part lives in pre-allocated pools (CompressedPool) and grows in place.
+        pool_fraction: size of the pools' value buffers relative to the dense / worst-case size (None: what the
+        sparsities need when no row has ties at its threshold - slab_fraction_for / packed_fraction_for; a pool that
+        turns out too small grows, see CompressedPool).
         window_kernel: the dense window lives in a pre-allocated buffer and the whole attention of a step - compressed
         tokens and window - is ops.decode_attention_window (three launches, no torch operators)."""
         self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
@@ -245,6 +347,8 @@ class SparseKVCache:
         self._kbuf = self._vbuf = None      # [bs * n_kv, residual_length + CHUNK, D], first _wlen tokens valid
         self._wlen = 0
         self.max_tokens = max_tokens
+        self.pool_fraction = pool_fraction
+        self._pool_gen = (0, 0)
         self.k_pool = self.v_pool = None
         self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
         self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
@@ -260,8 +364,23 @@ class SparseKVCache:
         return self.ws
 
     def _make_pools(self, heads, D, device):
-        self.k_pool = CompressedPool(heads, D, self.max_tokens, False, device)
-        self.v_pool = CompressedPool(heads, D, self.max_tokens, True, device)
+        fk = self.pool_fraction if self.pool_fraction is not None else slab_fraction_for(self.kth_k, D)
+        fv = self.pool_fraction if self.pool_fraction is not None else slab_fraction_for(self.kth_v, D)
+        self.k_pool = CompressedPool(heads, D, self.max_tokens, False, device, fk)
+        self.v_pool = CompressedPool(heads, D, self.max_tokens, True, device, fv)
+
+    def pools_moved(self):
+        """True once after a pool replaced its value buffer (it had to grow): addresses a HIP graph captured are stale."""
+        gen = (self.k_pool.generation, self.v_pool.generation) if self.k_pool is not None else (0, 0)
+        moved = gen != self._pool_gen
+        self._pool_gen = gen
+        return moved
+
+    def kv_bytes(self):
+        """(bytes the compressed part holds on the device, bytes of the dense window buffers)."""
+        pool = self.k_pool.allocated_bytes() + self.v_pool.allocated_bytes() if self.k_pool is not None else 0
+        win = 2 * self._kbuf.numel() * 2 if self._kbuf is not None else 0
+        return pool, win
 
     def _grow(self, K, V):
         """Adds the tokens K, V [bs, n_kv, M, D] to the compressed part."""
@@ -279,10 +398,8 @@ class SparseKVCache:
         self.v = cv if self.v is None else append_compressed(self.v, cv)
 
     def _pool_views(self):
-        """After an append to the pools.  With window_kernel the attention reads the pools themselves (nothing moved,
-        nothing to rebuild); the operator-by-operator paths take contiguous per-tile arrays, copied here."""
-        self.k_pool.check_overflow()
-        self.v_pool.check_overflow()
+        """After an append to the pools.  With window_kernel the attention reads the pools themselves (nothing to
+        rebuild); the operator-by-operator paths take contiguous per-tile arrays, copied here."""
         if self.window_kernel:
             self.k, self.v = self.k_pool, self.v_pool
         else:
@@ -402,7 +519,8 @@ class SparseKVCache:
     def advance(self):
         """Host-side bookkeeping after decode_device (or a replay of it): counts the token and, when the window holds
         residual_length + 256 tokens, compresses its oldest 256.  Returns True when arrays of the compressed part moved
-        (a captured graph must then be captured again): never with pools (max_tokens > 0), which grow in place."""
+        (a captured graph must then be captured again): with pools (max_tokens > 0), which grow in place, only when a
+        pool's value buffer turned out too small and was replaced by a larger one."""
         bs, n_kv, D = self._shape
         self.kv_len += 1
         self._wlen += 1
@@ -417,7 +535,7 @@ class SparseKVCache:
             self._wlen = rest
             self._wlen_dev.fill_(rest)
             self.compressed_length += CHUNK
-            grew = self.k_pool is None
+            grew = self.k_pool is None or self.pools_moved()
         self._window_views()
         return grew
 
@@ -493,12 +611,12 @@ class QuantSparseKVCache(SparseKVCache):
     decode_attention_window_quant (three launches, capturable with decode_device / advance)."""
 
     def __init__(self, groups, head_dim=128, k_sparsity=0.7, v_sparsity=0.7, residual_length=256, bit=2,
-                 dequant_mode=0, fused=False, window_kernel=False, max_tokens=0):
+                 dequant_mode=0, fused=False, window_kernel=False, max_tokens=0, pool_fraction=None):
         """max_tokens > 0: the compressed part lives in pre-allocated pools (QuantPool) and grows in place, pruning
         fused into the producer; with window_kernel the attention reads the pools themselves and a captured decode
         step stays valid across chunk appends."""
         super().__init__(groups, head_dim, k_sparsity, v_sparsity, residual_length, fused=fused,
-                         window_kernel=window_kernel, max_tokens=max_tokens)
+                         window_kernel=window_kernel, max_tokens=max_tokens, pool_fraction=pool_fraction)
         self.bit, self.dequant_mode = bit, dequant_mode
         # self.k / self.v: 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales, zeros]
 
@@ -538,8 +656,10 @@ class QuantSparseKVCache(SparseKVCache):
                 torch.cat([old[6], new[6]], 1)]
 
     def _make_pools(self, heads, D, device):
-        self.k_pool = QuantPool(heads, D, self.max_tokens, False, self.bit, device)
-        self.v_pool = QuantPool(heads, D, self.max_tokens, True, self.bit, device)
+        fk = self.pool_fraction if self.pool_fraction is not None else packed_fraction_for(self.kth_k, D, self.bit)
+        fv = self.pool_fraction if self.pool_fraction is not None else packed_fraction_for(self.kth_v, D, self.bit)
+        self.k_pool = QuantPool(heads, D, self.max_tokens, False, self.bit, device, fk)
+        self.v_pool = QuantPool(heads, D, self.max_tokens, True, self.bit, device, fv)
 
     def _grow(self, K, V):
         if self.max_tokens > 0:
@@ -549,8 +669,6 @@ class QuantSparseKVCache(SparseKVCache):
             ws = self._workspace(K.device)
             self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
             self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
-            self.k_pool.check()
-            self.v_pool.check()
             if not self.window_kernel:
                 self.k, self.v = self.k_pool.view(), self.v_pool.view()
             return

@@ -12,7 +12,8 @@ from ._lib import check, lib
 
 
 def _produce(inputs, is_value, bit, kth=0, group_size=64, ws=None, room=None):
-    """One call of the producer.  room: int32 tensor that takes the packed words (tile offsets count from its start);
+    """One call of the producer.  room: int32 tensor that takes the packed words (tile offsets count from its start;
+    a tile whose words would pass its end is not written, and the total then exceeds room.numel());
     default: a fresh buffer with room for the worst case.  Returns the per-tile arrays, the buffer and the word total
     as a device tensor (all ones should a wait of the one-pass producer have run out) - nothing is read on the host."""
     assert inputs.is_cuda
@@ -41,7 +42,9 @@ def _produce(inputs, is_value, bit, kth=0, group_size=64, ws=None, room=None):
     cap_words = B * T * (64 * int(bit) // 32)
     if room is None:
         room = torch.empty((max(cap_words, 1),), dtype=torch.int32, device=dev)
-    assert room.dtype == torch.int32 and room.is_contiguous() and room.numel() >= cap_words
+    else:
+        cap_words = room.numel()
+    assert room.dtype == torch.int32 and room.is_contiguous()
     check(L.mstf_compress_quant_grouped(st, x.data_ptr(), int(bool(is_value)), B, M, N, int(kth), int(bit), int(group_size),
                                         bmp.data_ptr(), tile_off.data_ptr(), counts.data_ptr(), units.data_ptr(),
                                         scales.data_ptr(), zeros.data_ptr(), total.data_ptr(), room.data_ptr(), cap_words,

@@ -21,8 +21,6 @@
 //                    In the fused call it also turns the unit-local tile offsets in idx into final ones.
 #include "compress_common.hpp"
 
-#include <cstdlib>
-
 namespace mstf {
 
 // ------------------------------------------------------------------------------- count
@@ -298,8 +296,10 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 // trip, until every word is set, and adds them up; the others wait at the barrier.
 // A workgroup publishes its total before it waits for anything and waits only for workgroups of a lower index, which
 // the dispatcher has started before it: every wait ends.  The waits are bounded all the same (kSpinLimit polls); a
-// workgroup that gives up sets the flag word behind the workgroup words, writes no values, and *total_halfs reads as
-// all ones.  onepass_init_kernel clears the words before the launch.
+// workgroup that gives up writes no values and marks the call itself (mark_gave_up): the flag word behind the
+// workgroup words, *total_halfs raised to all ones (packed layout: the last workgroup raises it to the sum with the
+// same atomic maximum, so the order of the two does not matter) and bit 1 of *overflow (pooled layout).
+// onepass_init_kernel clears the words and *total_halfs before the launch.
 // Compacts half h of a unit into the LDS image at img (tile offsets relative to the half's first tile).
 //   r     : this lane's token, raw fp16 pairs;  kept: its keep words (see select_kth_planes)
 //   key   : tile c = channel 64h + c over the 64 tokens - the lanes that keep the channel write at the tile's running
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
         in_head += bases[w][1];
         ok = ok && bases[w][2] != 0ull;
     }
-    if (!ok && threadIdx.x == 0) agent_store(gave_up, 1ull);
+    if (!ok && threadIdx.x == 0) mark_gave_up(gave_up, total_halfs, overflow);
     const uint32_t base = (uint32_t)in_head + in_group;
     const uint32_t end = base + total;
 
@@ -478,13 +478,14 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     if (lane == 0) {
         if (tb == nblk - 1) io[kD] = end;
         if (tb == 0 && nz_off) nz_off[b] = (uint32_t)(H >> 2);
-        if (u == units - 1 && total_halfs) *total_halfs = ok ? 2ull * (H + end) : ~0ull;
+        if (u == units - 1 && total_halfs && ok)
+            atomicMax(reinterpret_cast<unsigned long long*>(total_halfs), 2ull * (H + end));
     }
     if (!ok) return;
     const uint64_t head_half0 = dst_off ? 8ull * dst_off[b] : 2ull * H;
     if (head_half0 + 2ull * end > nz_capacity_halfs) return;  // would not fit: leave untouched (wave-uniform)
     if (dst_limit && head_half0 + 2ull * end > 8ull * dst_limit[b]) {
-        if (lane == 0) atomicOr(overflow, 1u);
+        if (lane == 0) atomicOr(overflow, kFlagOverflow);
         return;
     }
     char* dst = nz + (head_half0 + 2ull * base) * 2ull;
@@ -552,10 +553,9 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, const ProjArgs& pr
     const int groups = units / W;
     uint64_t* state = reinterpret_cast<uint64_t*>(ws);
     const int words = groups + 1;
-    const char* limit_env = getenv("MSTF_COMPRESS_SPIN_LIMIT");  // read per call: a test lowers it to force the give-up path
-    const uint32_t spin_limit = limit_env ? (uint32_t)strtoul(limit_env, nullptr, 10) : kSpinLimit;
+    const uint32_t spin_limit = onepass_spin_limit();
     hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
-                       dim3(256), 0, st, state, words);
+                       dim3(256), 0, st, state, words, total_halfs);
     int rc = check_launch();
     if (rc != MSTF_OK) return rc;
 #define MSTF_OP(WV)                                                                                                   \
@@ -678,6 +678,10 @@ static int proj_impl(void* stream, const mstf_proj_source* s, int is_value, int 
                                rope ? s->rot_stride_token : 0, rope ? s->rot_stride_head : 0};
     for (int64_t v : strides)
         if (v < 0 || v % 8 != 0) return MSTF_EINVAL;
+    // the loaders address the 64 rows of a unit with 32-bit byte offsets from the unit's first row
+    const int64_t tok_strides[] = {s->stride_token, rope ? s->rope_stride_token : 0, rope ? s->rot_stride_token : 0};
+    for (int64_t v : tok_strides)
+        if (v * 2 * 64 > 0xFFFFFFFFll) return MSTF_EUNSUPPORTED;
     if (!aligned_to(s->x, 16) || (rope && (!aligned_to(s->cos, 16) || !aligned_to(s->sin, 16) || !aligned_to(s->rot, 16))))
         return MSTF_EALIGN;
     const int64_t B64 = (int64_t)s->batch * s->heads;

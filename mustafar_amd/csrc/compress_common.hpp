@@ -475,11 +475,27 @@ __device__ __forceinline__ uint64_t sum_before(const uint32_t* ut, size_t before
 // ------------------------------------------------------------------------------- one-pass ordering
 // Status words of the one-pass producers (compress.hip describes the protocol): cleared by onepass_init_kernel,
 // one word per workgroup = bit 63 | total, published with an agent-scope store, polled by the workgroups behind.
-constexpr uint32_t kSpinLimit = 1u << 20;  // default; the host passes the limit in (MSTF_COMPRESS_SPIN_LIMIT overrides it for tests)
+constexpr uint32_t kSpinLimit = 1u << 20;  // the default of onepass_spin_limit() (runtime.hip)
+// The limit the launchers pass: kSpinLimit unless mstf_test_set_spin_limit (runtime.hip) lowered it - a test's way
+// to force the give-up path from the host while every kernel still exits normally.  The environment has no say.
+uint32_t onepass_spin_limit();
 
-static __global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n)
+// Clears the status words and the caller's total (nullable): the kernel raises the total with atomic maxima - the
+// last workgroup to the sum, a workgroup that gave up to all ones - so whichever comes last, a give-up stays visible.
+static __global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n,
+                                                                  uint64_t* __restrict__ total)
 {
     for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < n; i += (int)(gridDim.x * 256)) state[i] = 0ull;
+    if (total && blockIdx.x == 0 && threadIdx.x == 0) *total = 0ull;
+}
+// The marker of a workgroup whose wait ran out, from one thread: the flag word behind the status words, all ones in
+// the caller's total (compress contract) or bit 1 of the caller's sticky flag (append contract).
+constexpr uint32_t kFlagOverflow = 1u, kFlagGaveUp = 2u;
+__device__ __forceinline__ void mark_gave_up(uint64_t* flag_word, uint64_t* total, uint32_t* sticky)
+{
+    __hip_atomic_store(flag_word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (total) atomicMax(reinterpret_cast<unsigned long long*>(total), ~0ull);
+    if (sticky) atomicOr(sticky, kFlagGaveUp);
 }
 
 __device__ __forceinline__ uint64_t agent_load(const uint64_t* p)

@@ -9,8 +9,6 @@
 #include "compress_common.hpp"
 #include "spmv_common.hpp"
 
-#include <cstdlib>
-
 namespace mstf {
 
 #pragma clang fp contract(off)
@@ -306,8 +304,9 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
         before += bases[w][0];
         ok = ok && bases[w][1] != 0ull;
     }
-    if (!ok && threadIdx.x == 0) agent_store(state + groups_total, 1ull);
-    if (lane == 0 && unit == nunits - 1) *total_words = ok ? before + totA + totB : ~0ull;
+    if (!ok && threadIdx.x == 0) mark_gave_up(state + groups_total, total_words, nullptr);
+    if (lane == 0 && unit == nunits - 1 && ok)
+        atomicMax(reinterpret_cast<unsigned long long*>(total_words), before + totA + totB);
     const uint64_t off_h[2] = {before + eA, before + totA + eB};
     tile_off[tile0 + lane] = (uint32_t)off_h[0];
     tile_off[tile0 + 64 + lane] = (uint32_t)off_h[1];
@@ -443,10 +442,9 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
         const int groups = units_all / W;
         uint64_t* state = reinterpret_cast<uint64_t*>(ws);
         const int words = groups + 1;
-        const char* limit_env = getenv("MSTF_COMPRESS_SPIN_LIMIT");
-        const uint32_t spin_limit = limit_env ? (uint32_t)strtoul(limit_env, nullptr, 10) : kSpinLimit;
+        const uint32_t spin_limit = onepass_spin_limit();
         hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
-                           dim3(256), 0, st, state, words);
+                           dim3(256), 0, st, state, words, total_words);
         if ((rc = check_launch()) != MSTF_OK) return rc;
 #define MSTF_QOP(WV)                                                                                                  \
     hipLaunchKernelGGL((quant_onepass_kernel<IS_VALUE, G32, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \

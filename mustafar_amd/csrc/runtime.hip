@@ -6,7 +6,22 @@
 namespace mstf {
 static std::atomic<int> g_last_hip_error{0};
 void set_last_hip_error(int e) { g_last_hip_error.store(e); }
+
+// Polls a one-pass producer's workgroup spends on a wait before it gives up (0 in the atomic = the default).
+static std::atomic<uint32_t> g_spin_limit{0u};
+static std::atomic<bool> g_spin_limit_set{false};
+uint32_t onepass_spin_limit() { return g_spin_limit_set.load() ? g_spin_limit.load() : (1u << 20); }
 }  // namespace mstf
+
+extern "C" void mstf_test_set_spin_limit(int64_t polls)
+{
+    if (polls < 0) {
+        mstf::g_spin_limit_set.store(false);
+        return;
+    }
+    mstf::g_spin_limit.store(polls > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)polls);
+    mstf::g_spin_limit_set.store(true);
+}
 
 extern "C" const char* mstf_strerror(int code)
 {

@@ -32,14 +32,25 @@ class Config:
 
 
 class DenseMaskedCache:
-    """Same state machine as SparseKVCache with the compressed range kept as pruned dense tensors."""
+    """Same state machine as SparseKVCache with the compressed range kept as pruned dense tensors.  The tokens live in
+    buffers that grow geometrically (a decode step appends one row instead of re-concatenating the cache) and the
+    query heads of a KV head are multiplied as one batch, so K and V are read once per KV head."""
 
-    def __init__(self, groups, head_dim, k_sparsity, v_sparsity, residual_length):
+    def __init__(self, groups, head_dim, k_sparsity, v_sparsity, residual_length, capacity=0):
         self.groups, self.head_dim, self.residual_length = groups, head_dim, residual_length
         self.kth_k = ops.kth_from_sparsity(k_sparsity, head_dim)
         self.kth_v = ops.kth_from_sparsity(v_sparsity, head_dim)
-        self.k = self.v = None
+        self.capacity = capacity
+        self._k = self._v = None
         self.compressed_length = self.kv_len = 0
+
+    @property
+    def k(self):
+        return self._k[:, :, :self.kv_len]
+
+    @property
+    def v(self):
+        return self._v[:, :, :self.kv_len]
 
     @staticmethod
     def _prune(x, kth):
@@ -47,27 +58,44 @@ class DenseMaskedCache:
         thr = torch.kthvalue(a, kth, dim=-1, keepdim=True).values
         return torch.where(a >= thr, x, torch.zeros_like(x))
 
+    def _compressed_form(self, K, V):
+        """What the cache holds for a range of tokens that leaves the dense window: K, V [bs, n_kv, M, D], M % 256 == 0."""
+        return self._prune(K, self.kth_k), self._prune(V, self.kth_v)
+
+    def _room(self, n):
+        if self._k is not None and self._k.shape[2] >= n:
+            return
+        cap = max(n, self.capacity, int(1.5 * self._k.shape[2]) if self._k is not None else 0)
+        for name in ("_k", "_v"):
+            old = getattr(self, name)
+            new = torch.empty(old.shape[:2] + (cap,) + old.shape[3:], dtype=old.dtype, device=old.device)
+            new[:, :, :self.kv_len] = old[:, :, :self.kv_len]
+            setattr(self, name, new)
+
     def prefill(self, K, V):
         L = K.shape[2]
         Lc = ((L - self.residual_length) // CHUNK) * CHUNK if L > self.residual_length else 0
-        self.k, self.v = K.clone(), V.clone()
+        cap = max(L, self.capacity)
+        self._k = torch.empty(K.shape[:2] + (cap, K.shape[3]), dtype=K.dtype, device=K.device)
+        self._v = torch.empty_like(self._k)
+        self._k[:, :, :L], self._v[:, :, :L] = K, V
         if Lc > 0:
-            self.k[:, :, :Lc] = self._prune(K[:, :, :Lc], self.kth_k)
-            self.v[:, :, :Lc] = self._prune(V[:, :, :Lc], self.kth_v)
+            self._k[:, :, :Lc], self._v[:, :, :Lc] = self._compressed_form(K[:, :, :Lc], V[:, :, :Lc])
         self.compressed_length, self.kv_len = Lc, L
 
     def decode(self, q, k_new, v_new):
         D, g = self.head_dim, self.groups
+        bs, n_q = q.shape[0], q.shape[1]
+        self._room(self.kv_len + 1)
+        self._k[:, :, self.kv_len], self._v[:, :, self.kv_len] = k_new[:, :, 0], v_new[:, :, 0]
         self.kv_len += 1
-        self.k = torch.cat([self.k, k_new], dim=2)
-        self.v = torch.cat([self.v, v_new], dim=2)
-        s = torch.matmul(q, _repeat_kv(self.k, g).transpose(2, 3))
+        s = torch.matmul(q.view(bs, n_q // g, g, D), self.k.transpose(2, 3))
         p = torch.softmax((s / math.sqrt(D)).float(), -1).half()
-        out = torch.matmul(p, _repeat_kv(self.v, g))
+        out = torch.matmul(p, self.v).view(bs, n_q, 1, D)
         Lc = self.compressed_length
         if (self.kv_len - self.residual_length - Lc) % CHUNK == 0 and self.kv_len - Lc >= CHUNK:
-            self.k[:, :, Lc:Lc + CHUNK] = self._prune(self.k[:, :, Lc:Lc + CHUNK], self.kth_k)
-            self.v[:, :, Lc:Lc + CHUNK] = self._prune(self.v[:, :, Lc:Lc + CHUNK], self.kth_v)
+            kc, vc = self._compressed_form(self._k[:, :, Lc:Lc + CHUNK], self._v[:, :, Lc:Lc + CHUNK])
+            self._k[:, :, Lc:Lc + CHUNK], self._v[:, :, Lc:Lc + CHUNK] = kc, vc
             self.compressed_length += CHUNK
         return out
 
@@ -94,12 +122,27 @@ def _rope(x, tables):
 
 class Decoder:
     def __init__(self, cfg, device, seed=0, cache="sparse", sparsity=0.7, residual_length=256, max_tokens=0,
-                 proj_prefill=True):
+                 proj_prefill=True, weights_of=None, dense_cache=None):
         """proj_prefill: the sparse caches take the keys and values of the prompt straight from the projection output
         (keys rotated by the compressor's own kernel; the fp16 cache also compresses them where they lie, without
-        transposed or contiguous copies)."""
+        transposed or contiguous copies).  max_tokens: capacity of the compressed part of the sparse caches (0: caches
+        that re-concatenate), of all tokens for the dense cache.  weights_of: another Decoder whose weight tensors
+        this one shares.  dense_cache: class used for cache="dense_masked" (default DenseMaskedCache).
+        shadow (attribute, a list of caches, one per layer): every layer's attention inputs - the projection output of
+        the step, the prompt's keys and values - are also given to these caches and shadow_check(layer, output of the
+        model's cache, output of the shadow cache) is called; the model goes on with its own cache's output, so the
+        shadow caches are teacher-forced layer by layer."""
         self.cfg, self.dev = cfg, device
         self.proj_prefill = proj_prefill
+        self.shadow, self.shadow_check = None, None
+        self._dense_cache = dense_cache or DenseMaskedCache
+        if weights_of is not None:
+            self.embed, self.layers, self.norm, self.lm_head = (weights_of.embed, weights_of.layers, weights_of.norm,
+                                                                weights_of.lm_head)
+            self._cache_args = (cache, sparsity, residual_length, max_tokens)
+            self.reset_caches()
+            self.attn_events = []
+            return
         g = torch.Generator(device=device)
         g.manual_seed(seed)
 
@@ -123,19 +166,23 @@ class Decoder:
 
     def reset_caches(self):
         """Fresh, empty caches for every layer (a new prompt)."""
+        self.caches = self.make_caches(*self._cache_args)
+
+    def make_caches(self, cache, sparsity=0.7, residual_length=256, max_tokens=0):
+        """One cache per layer of the kind `cache` (what reset_caches installs; also how a shadow set is made)."""
         c = self.cfg
-        cache, sparsity, residual_length, max_tokens = self._cache_args
         groups = c.n_q // c.n_kv
         if cache == "sparse":
-            self.caches = [SparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length, fused=True,
+            return [SparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length, fused=True,
                                          max_tokens=max_tokens, window_kernel=True) for _ in range(c.layers)]
-        elif cache in ("sparse_quant2", "sparse_quant4"):
-            self.caches = [QuantSparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length,
-                                              bit=int(cache[-1]), fused=True, window_kernel=True, max_tokens=max_tokens)
-                           for _ in range(c.layers)]
-        else:
-            self.caches = [DenseMaskedCache(groups, c.head_dim, sparsity, sparsity, residual_length)
-                           for _ in range(c.layers)]
+        if cache in ("sparse_quant2", "sparse_quant4"):
+            return [QuantSparseKVCache(groups, c.head_dim, sparsity, sparsity, residual_length,
+                                       bit=int(cache[-1]), fused=True, window_kernel=True, max_tokens=max_tokens)
+                    for _ in range(c.layers)]
+        # the dense cache holds every token: the compressed capacity plus the largest window
+        total = max_tokens + residual_length + CHUNK if max_tokens > 0 else 0
+        return [self._dense_cache(groups, c.head_dim, sparsity, sparsity, residual_length, capacity=total)
+                for _ in range(c.layers)]
 
     def _mlp(self, lw, x):
         # two products over the halves of the stacked weight: both results are contiguous, so the activation and
@@ -144,7 +191,8 @@ class Decoder:
         gate, up = F.linear(x, lw["gate_up"][:ffn]), F.linear(x, lw["gate_up"][ffn:])
         return F.linear(F.silu(gate) * up, lw["down"])
 
-    def _qkv(self, lw, x, tables):
+    def _qkv(self, lw, x, tables, proj=None):
+        """proj: the projection output of x, if the caller already has it (decode steps)."""
         c = self.cfg
         bs, L, _ = x.shape
         if L == 1:
@@ -156,7 +204,8 @@ class Decoder:
                 cos = torch.cat([cos.expand(c.n_q + c.n_kv, -1), one], 0)
                 sin = torch.cat([sin.expand(c.n_q + c.n_kv, -1), torch.zeros_like(one)], 0)
                 tables[0], tables[1] = cos, sin        # built by the first layer of the step, reused by the others
-            qkv = _rope(F.linear(x, lw["qkv"]).view(bs, H, c.head_dim), (cos, sin)).unsqueeze(2)
+            proj = F.linear(x, lw["qkv"]) if proj is None else proj
+            qkv = _rope(proj.view(bs, H, c.head_dim), (cos, sin)).unsqueeze(2)
             return qkv[:, : c.n_q], qkv[:, c.n_q: c.n_q + c.n_kv], qkv[:, c.n_q + c.n_kv:]
         qkv = F.linear(x, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim).transpose(1, 2)
         qk = _rope(qkv[:, : c.n_q + c.n_kv], tables)   # query and key heads in one pass; contiguous [bs, heads, L, D]
@@ -171,12 +220,16 @@ class Decoder:
         half = c.head_dim // 2
         usin = torch.cat([-tables[1][:, :half], tables[1][:, half:]], -1)   # sin itself: the kernel rotates with rotate_half
         x = self.embed[ids]
-        for lw, cache in zip(self.layers, self.caches):
+        for li, (lw, cache) in enumerate(zip(self.layers, self.caches)):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            if self.proj_prefill and isinstance(cache, SparseKVCache):
+            # every cache of the layer gets the same keys and values: the model's own and, if set, its shadow
+            takers = [cache] + ([self.shadow[li]] if self.shadow is not None else [])
+            from_proj = [t for t in takers if self.proj_prefill and isinstance(t, SparseKVCache)]
+            if from_proj:
                 qkv = F.linear(h, lw["qkv"]).view(bs, L, c.n_q + 2 * c.n_kv, c.head_dim)
                 q = _rope(qkv[:, :, : c.n_q].transpose(1, 2), tables)
-                k, v = cache.prefill_proj(qkv[:, :, c.n_q: c.n_q + c.n_kv], qkv[:, :, c.n_q + c.n_kv:], tables[0], usin)
+                k, v = from_proj[0].prefill_proj(qkv[:, :, c.n_q: c.n_q + c.n_kv], qkv[:, :, c.n_q + c.n_kv:], tables[0],
+                                                 usin)
             else:
                 q, k, v = self._qkv(lw, h, tables)
                 k = k.contiguous()
@@ -185,8 +238,9 @@ class Decoder:
                 outs.append(F.scaled_dot_product_attention(q[b0:b0 + seq_chunk], k[b0:b0 + seq_chunk], v[b0:b0 + seq_chunk],
                                                            is_causal=True, enable_gqa=True))
             a = torch.cat(outs, 0).transpose(1, 2).reshape(bs, L, c.n_q * c.head_dim)
-            if not (self.proj_prefill and isinstance(cache, SparseKVCache)):
-                cache.prefill(k, v)
+            for t in takers:
+                if not (from_proj and t is from_proj[0]):
+                    t.prefill(k, v)      # (rotated keys)
             x = x + F.linear(a, lw["o"])
             h = _rms_norm(x, lw["ln2"], c.rms_eps)
             for b0 in range(0, bs, seq_chunk):
@@ -202,25 +256,29 @@ class Decoder:
             logits = self._layers(ids, pos, timed, None, from_proj=True)
             for cache in self.caches:
                 cache.advance()
-            return logits
-        return self._layers(ids, pos, timed, lambda cache, q, k, v: cache.decode(q, k, v))
+        else:
+            logits = self._layers(ids, pos, timed, lambda cache, q, k, v: cache.decode(q, k, v))
+        for cache in self.shadow or ():
+            cache.advance()
+        return logits
 
     def _layers(self, ids, pos, timed, attend, from_proj=False):
         """from_proj: the cache takes the new token's projection output as it is (decode_device_proj: rotation, window
         append and query layout in one launch); otherwise q, k, v are rotated here and handed over as tensors."""
         c = self.cfg
         tables = list(_rope_tables(pos, c.head_dim, c.rope_theta, torch.float16))   # once per step, shared by the layers
-        if from_proj:
+        shadow = self.shadow
+        if from_proj or shadow is not None:
             half, nq, nk = c.head_dim // 2, c.n_q * c.head_dim, c.n_kv * c.head_dim
             cos = tables[0]
             usin = torch.cat([-tables[1][:, :half], tables[1][:, half:]], -1)   # sin itself, for rotate_half
         x = self.embed[ids]
-        for lw, cache in zip(self.layers, self.caches):
+        for li, (lw, cache) in enumerate(zip(self.layers, self.caches)):
             h = _rms_norm(x, lw["ln1"], c.rms_eps)
-            if from_proj:
-                qkv = F.linear(h, lw["qkv"]).view(x.shape[0], -1)
-            else:
-                q, k, v = self._qkv(lw, h, tables)
+            proj = F.linear(h, lw["qkv"])
+            qkv = proj.view(x.shape[0], -1)
+            if not from_proj:
+                q, k, v = self._qkv(lw, h, tables, proj=proj)
             if timed:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
@@ -231,6 +289,9 @@ class Decoder:
             if timed:
                 e1.record()
                 self.attn_events.append((e0, e1))
+            if shadow is not None:
+                sa = shadow[li].decode_device_proj(qkv[:, :nq], qkv[:, nq: nq + nk], qkv[:, nq + nk:], cos, usin)
+                self.shadow_check(li, a, sa)
             x = x + F.linear(a.transpose(1, 2).reshape(x.shape[0], 1, c.n_q * c.head_dim), lw["o"])
             x = x + self._mlp(lw, _rms_norm(x, lw["ln2"], c.rms_eps))
         return F.linear(_rms_norm(x, self.norm, c.rms_eps), self.lm_head)
@@ -251,6 +312,7 @@ class GraphedGreedyLoop:
         self.pos = torch.tensor([position], device=dec.dev)
         self.graph = None
         self.captures = 0
+        self.append_events = None    # a list: (start, end) HIP events around every chunk append are collected in it
         # the layers' windows grow in lockstep: one device counter, advanced by the first layer's cache
         for cache in dec.caches[1:]:
             cache.share_clock(dec.caches[0])
@@ -263,8 +325,15 @@ class GraphedGreedyLoop:
 
     def _advance(self):
         grew = False
+        before = self.dec.caches[0].compressed_length
+        if self.append_events is not None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
         for cache in self.dec.caches:
             grew |= cache.advance()
+        if self.append_events is not None and self.dec.caches[0].compressed_length != before:
+            e1.record()
+            self.append_events.append((e0, e1))
         if grew:
             self.graph = None
 
@@ -284,6 +353,12 @@ class GraphedGreedyLoop:
             return
         self.graph.replay()
         self._advance()
+
+
+def pool_tokens(total_tokens, residual_length=256):
+    """Capacity of the compressed part of a cache that will hold total_tokens tokens: the compressed length is a
+    multiple of the chunk and leaves at least residual_length tokens dense."""
+    return max(CHUNK, ((total_tokens - residual_length) // CHUNK) * CHUNK)
 
 
 def generate(dec, prompt_ids, new_tokens, forced=None):
@@ -315,7 +390,7 @@ def main():
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = Config(layers=args.layers)
-    max_tokens = ((args.prompt + args.new_tokens + CHUNK - 1) // CHUNK) * CHUNK
+    max_tokens = pool_tokens(args.prompt + args.new_tokens, args.residual)
     dec = Decoder(cfg, dev, cache=args.cache, sparsity=args.sparsity, residual_length=args.residual, max_tokens=max_tokens,
                   proj_prefill=not args.copy_prefill)
     g = torch.Generator(device=dev)

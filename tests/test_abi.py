@@ -65,6 +65,13 @@ def test_argument_validation_returns_before_any_launch(lib):
     assert L.mstf_compress_proj_f16(None, None, 0, 64, 128, 89, None, None, None, None, None, 0, None, 0) == -1
     assert L.mstf_compress_proj_f16(None, ctypes.byref(src), 0, 64, 128, 89, None, None, None, None, None, 0, None, 0) == -1
     assert L.mstf_append_proj_f16(None, ctypes.byref(src), 1, 64, 128, 89, None, None, None, None, None, None, None, 0) == -1
+    # a row stride whose 64-row span does not fit the loaders' 32-bit byte offsets is refused, not wrapped
+    wide = _lib.ProjSource()
+    wide.x, wide.batch, wide.heads, wide.rows = 256, 1, 1, 64
+    wide.stride_batch, wide.stride_head, wide.stride_token = 0, 128, 1 << 25
+    assert L.mstf_compress_proj_f16(None, ctypes.byref(wide), 1, 64, 128, 89, 256, 256, 256, 256, 256, 8192, 256, 1 << 20) == -3
+    L.mstf_test_set_spin_limit(0)       # host-side state only
+    L.mstf_test_set_spin_limit(-1)
     assert L.mstf_decode_attention_f16(None, *([None] * 11), 64, 128, 4, 4, None, 0) == -1
     # the entry point on the library's fixed scratch buffer refuses, on the host, what does not fit into it
     assert L.mstf_decode_attention_static_f16(None, *([256] * 10), None, 4096, 128, 1012, 4) == -6

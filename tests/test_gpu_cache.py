@@ -67,7 +67,10 @@ def test_prefill_decode_append_matches_one_shot_and_oracle(fused, pooled, window
         assert torch.equal(one.packed(), cache.k.packed())
 
 
-def test_pool_overflow_is_flagged_and_leaves_other_heads_alone():
+def test_pool_that_overflows_grows_and_ends_up_like_one_that_never_did():
+    """A chunk that does not fit a head's slab sets bit 0 of the flag word and writes none of the unit's values; what
+    was there stays.  The pool then grows - larger slabs, old values copied, the chunk appended again - and holds
+    exactly what a pool with dense-size slabs holds (and what the oracle packs)."""
     from mustafar_amd.cache import CompressedPool
     dev = torch.device("cuda:0")
     heads, D = 3, 128
@@ -75,15 +78,73 @@ def test_pool_overflow_is_flagged_and_leaves_other_heads_alone():
     Kt = torch.from_numpy(K).to(dev)
     pool = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)    # 30 % survive: 64 tokens fit, 256 do not
     pool.append(Kt[:, :64], 89)
-    assert int(pool.overflow) == 0
-    before = pool.nz.clone()
+    assert int(pool.overflow) == 0 and pool.generation == 0
+    before, off_before, seen = pool.nz.clone(), pool.nz_off.clone(), []
+    grow = pool._grow_slabs
+
+    def watched_grow():
+        # at this point the failed append has run: flag read by the pool, old values untouched
+        for b in range(heads):
+            n = 2 * int(pool.idx_store[b, 128])
+            s0 = 8 * int(off_before[b])
+            assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
+        seen.append(pool.slab16)
+        grow()
+    pool._grow_slabs = watched_grow
     pool.append(Kt[:, 64:256], 89)
-    assert int(pool.overflow) == 1
-    # what was there stays: the values of the first 64 tokens of every head
+    assert seen and pool.generation == 1 and pool.slab16 > seen[0] and int(pool.overflow) == 0 and pool.tokens == 256
+    ref = CompressedPool(heads, D, 256, False, dev, slab_fraction=1.0)
+    ref.append(Kt[:, :64], 89)
+    ref.append(Kt[:, 64:256], 89)
+    assert ref.generation == 0
+    assert torch.equal(pool.bmp, ref.bmp) and torch.equal(pool.idx, ref.idx)
+    rb, ri, rnz, roff = orc.compress(orc.prune_rows(K, 89), 0)
+    assert np.array_equal(pool.bmp.cpu().numpy(), rb) and np.array_equal(pool.idx.cpu().numpy(), ri)
     for b in range(heads):
-        n = 2 * int(pool.idx[b, 128])
-        s0 = 8 * int(pool.nz_off[b])
-        assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
+        assert torch.equal(pool.head_values(b).view(torch.int16), ref.head_values(b).view(torch.int16))
+        want = rnz[8 * int(roff[b]):8 * int(roff[b]) + 2 * int(ri[b, -1])]
+        assert np.array_equal(pool.head_values(b).cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_quantised_pool_that_overflows_grows_and_ends_up_like_one_that_never_did():
+    from mustafar_amd.cache import QuantPool
+    dev = torch.device("cuda:0")
+    heads, D = 3, 128
+    _, V = orc.make_kv(19, heads, 256, D)
+    Vt = torch.from_numpy(V).to(dev)
+    pool = QuantPool(heads, D, 256, True, 2, dev, packed_fraction=0.2)     # 64 tokens fit, 256 do not
+    ref = QuantPool(heads, D, 256, True, 2, dev)
+    for p in (pool, ref):
+        p.append(Vt[:, :64], 89)
+    assert pool.generation == 0
+    for p in (pool, ref):
+        p.append(Vt[:, 64:256], 89)
+    assert pool.generation == 1 and ref.generation == 0 and pool.reserved == ref.reserved and pool.tokens == 256
+    for a, b in zip(pool.view(), ref.view()):
+        if a.dim() == 1:
+            assert torch.equal(a[:pool.reserved], b[:ref.reserved])
+        else:
+            assert torch.equal(a, b)
+
+
+def test_default_pool_sizes_hold_the_seeded_cache_without_growing():
+    """slab_fraction_for / packed_fraction_for: 70 % sparsity, K with outlier channels - no growth, and the bytes held
+    are the fractions of the dense bytes the docstrings state."""
+    from mustafar_amd.cache import QuantSparseKVCache, SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D, L = 2, 2, 4, 128, 1024 + 256
+    K, V = orc.make_kv(23, bs * n_kv, L, D)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, L, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, L, D)
+    dense = 2 * bs * n_kv * 1024 * D * 2
+    for cache, bound in ((SparseKVCache(g, D, 0.7, 0.7, 256, fused=True, window_kernel=True, max_tokens=1024), 0.55),
+                         (QuantSparseKVCache(g, D, 0.7, 0.7, 256, bit=2, fused=True, window_kernel=True, max_tokens=1024),
+                          0.30)):
+        cache.prefill(Kt, Vt)
+        assert cache.compressed_length == 1024
+        assert cache.k_pool.generation == 0 and cache.v_pool.generation == 0
+        pool_bytes, _ = cache.kv_bytes()
+        assert pool_bytes <= bound * dense, (pool_bytes / dense, bound)
 
 
 @pytest.mark.parametrize("window_kernel", [False, True])

@@ -270,30 +270,81 @@ def test_config0_shape_against_oracle():
                 fused=ops.decode_attention(ck, cv, qg, groups))
 
 
-def test_one_pass_compressor_flags_a_wait_that_ran_out(monkeypatch):
+@pytest.fixture
+def no_polls():
+    """Forces the one-pass producers' bounded waits to zero polls from the host (every kernel still runs to its end);
+    the default comes back afterwards."""
+    from mustafar_amd._lib import lib
+    lib().mstf_test_set_spin_limit(0)
+    yield
+    lib().mstf_test_set_spin_limit(-1)
+
+
+def test_one_pass_compressor_flags_a_wait_that_ran_out(no_polls):
     """The one-pass compressor orders its workgroups through status words and bounds every wait.  With the bound forced
     to zero polls from the host, a workgroup whose predecessors have not published yet gives up: then the total must
-    read as all ones (and the host layer must raise), otherwise everything must be exactly right - never a silently
-    wrong result.  Every kernel still runs to its end."""
+    read as all ones whichever workgroup it was (and the host layer must raise), otherwise everything must be exactly
+    right - never a silently wrong result."""
     from mustafar_amd import ops
+    from mustafar_amd._lib import lib
     dev = torch.device("cuda:0")
     K, _ = orc.make_kv(31, 16, 1024, 128)
     Kt = torch.from_numpy(K).to(dev)
     rb, ri, rnz, roff = orc.compress(orc.prune_rows(K, 89), 0)
-    monkeypatch.setenv("MSTF_COMPRESS_SPIN_LIMIT", "0")
-    gave_up = 0
     for _ in range(4):
         ck = ops.compress(Kt, False, kth=89, capacity_halfs=Kt.numel())
         torch.cuda.synchronize()
         if int(ck.total_halfs) == -1:
-            gave_up += 1
             with pytest.raises(RuntimeError, match="gave up"):
                 ck.packed()
         else:
             assert int(ck.total_halfs) == rnz.size
             assert np.array_equal(ck.bmp.cpu().numpy(), rb) and np.array_equal(ck.idx.cpu().numpy(), ri)
             assert np.array_equal(ck.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
-    monkeypatch.delenv("MSTF_COMPRESS_SPIN_LIMIT")
+    lib().mstf_test_set_spin_limit(-1)
     ck = ops.compress(Kt, False, kth=89, capacity_halfs=Kt.numel())
     assert int(ck.total_halfs) == rnz.size
     assert np.array_equal(ck.packed().cpu().numpy().view(np.uint16), rnz.view(np.uint16))
+
+
+def test_append_flags_a_wait_that_ran_out(no_polls):
+    """The pooled append has no total to carry the marker: a workgroup that gives up sets bit 1 of the flag word and
+    the pool raises; an append that is not flagged is exact."""
+    from mustafar_amd.cache import CompressedPool
+    dev = torch.device("cuda:0")
+    heads, M, D = 16, 1024, 128
+    K, _ = orc.make_kv(32, heads, M, D)
+    Kt = torch.from_numpy(K).to(dev)
+    rb, ri, rnz, roff = orc.compress(orc.prune_rows(K, 89), 0)
+    for _ in range(4):
+        pool = CompressedPool(heads, D, M, False, dev)
+        try:
+            pool.append(Kt, 89)
+        except RuntimeError as e:
+            assert "gave up" in str(e) and int(pool.overflow) & 2
+            continue
+        assert int(pool.overflow) == 0
+        assert np.array_equal(pool.bmp.cpu().numpy(), rb) and np.array_equal(pool.idx.cpu().numpy(), ri)
+        for b in range(heads):
+            want = rnz[8 * int(roff[b]):8 * int(roff[b]) + 2 * int(ri[b, -1])]
+            assert np.array_equal(pool.head_values(b).cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_quantised_producer_flags_a_wait_that_ran_out(no_polls):
+    from mustafar_amd import compression_quant as cq
+    dev = torch.device("cuda:0")
+    _, V = orc.make_kv(33, 16, 1024, 128)
+    Vp = orc.prune_rows(V, 89)
+    ref = orc.compress_quant(Vp, 1, 2)
+    Vt = torch.from_numpy(Vp).to(dev)
+    for gs in (64, 32):
+        for _ in range(3):
+            out = cq._produce(Vt, True, 2, 0, gs)
+            total = out[-1]
+            torch.cuda.synchronize()
+            if int(total) == -1:
+                with pytest.raises(RuntimeError, match="gave up"):
+                    cq.words_written(total)
+            elif gs == 64:
+                n = cq.words_written(total)
+                assert np.array_equal(out[2][:n].cpu().numpy().view(np.uint32), ref[2].view(np.uint32))

@@ -210,25 +210,26 @@ def test_random_layouts_against_oracle(seed):
     check_compressed(c, comp)
 
 
-def test_append_proj_overflow_is_flagged():
+def test_append_proj_overflow_grows_and_does_not_rotate_twice():
+    """A chunk from the projection layout that does not fit: the pool grows and appends it again; the keys, rotated
+    in place by the first attempt, are not rotated a second time."""
     from mustafar_amd.cache import CompressedPool
     dev = torch.device("cuda:0")
     batch, heads, rows = 1, 3, 256
     K, _ = orc.make_kv(9, batch * heads, rows, D)
-    x = torch.from_numpy(np.ascontiguousarray(K.reshape(batch, heads, rows, D).transpose(0, 2, 1, 3))).to(dev)
+    kx = np.ascontiguousarray(K.reshape(batch, heads, rows, D).transpose(0, 2, 1, 3))
+    cos, sin = orc.rope_tables(np.arange(rows))
+    rot_ref, comp = oracle_side(kx, rows, 89, False, cos, sin)
+    x = torch.from_numpy(kx).to(dev)
     pool = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)    # 64 tokens fit, 256 do not
-    pool.append_proj(x[:, :64], 89, 64)
-    assert int(pool.overflow) == 0 and pool.tokens == 64
-    ref = CompressedPool(heads, D, 256, False, dev, slab_fraction=0.2)
-    ref.append(x[:, :64].transpose(1, 2).reshape(heads, 64, D), 89)
-    assert torch.equal(pool.nz.view(torch.int16), ref.nz.view(torch.int16)) and torch.equal(pool.idx, ref.idx)
-    before = pool.nz.clone()
-    pool.append_proj(x[:, 64:], 89, 192)
-    assert int(pool.overflow) == 1
+    r = pool.append_proj(x, 89, rows, torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev))
+    assert pool.generation == 1 and int(pool.overflow) == 0 and pool.tokens == rows
+    assert np.array_equal(bits(r.cpu().numpy()), bits(rot_ref))
+    rb, ri, rnz, roff = comp
+    assert np.array_equal(pool.bmp.cpu().numpy(), rb) and np.array_equal(pool.idx.cpu().numpy(), ri)
     for b in range(heads):
-        n = 2 * int(pool.idx[b, 128])
-        s0 = 8 * int(pool.nz_off[b])
-        assert torch.equal(pool.nz[s0:s0 + n], before[s0:s0 + n])
+        want = rnz[8 * int(roff[b]):8 * int(roff[b]) + 2 * int(ri[b, -1])]
+        assert np.array_equal(pool.head_values(b).cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
 def test_short_prompt_through_prefill_proj_is_only_rotated():
