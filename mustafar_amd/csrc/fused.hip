@@ -39,6 +39,11 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     // from device memory, at most nblk blocks of it; the launch is then sized for the capacity and the wavefronts
     // beyond the valid blocks leave neutral partials, so a recorded launch stays valid while the cache grows.
     constexpr int D = kFusedD;
+    // every argument in registers before anything else: left alone, the compiler fetches them where they are first
+    // used, three dependent round trips in front of the first load of data
+    asm volatile("" ::"s"(k_bmp), "s"(k_nz), "s"(k_idx), "s"(k_nz_off), "s"(v_bmp), "s"(v_nz), "s"(v_idx), "s"(v_nz_off),
+                 "s"(q), "s"(out), "s"(part_o), "s"(part_ml), "s"(tstride), "s"(groups), "s"(nblk), "s"(nsplit),
+                 "s"(write_final), "s"(sqrt_d), "s"(bpw), "s"(tokens_dev));
     if (tokens_dev) {
         const int valid = *tokens_dev / 64;
         nblk = valid < nblk ? valid : nblk;
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
         // nc, woffc: stage index and byte offset of the stage's first weight from wbase, as constants (they end up in
         // immediate operands)
         auto stage_batches = [&](auto nc, uint32_t buf, uint32_t wbase, auto woffc, uint32_t wgroup, f4_t (&acc)[NM],
-                                 int adv) {
+                                 f4_t (&acc2)[NM], int adv) {
             constexpr int n = decltype(nc)::value;
             constexpr int woff = decltype(woffc)::value;
             const uint32_t rel = buf - cur.ov[0] * 4u;  // idx counts 4-byte units from the start of the head's values
@@ -160,14 +165,14 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
                 constexpr int wo = woff + g * 16;
                 Batch nxt;
                 if constexpr (g1 < kSideBatches)
-                    batch_step_exec<NM, true, g1 * 64, g1 * 32, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc);
+                    batch_step_exec<NM, true, g1 * 64, g1 * 32, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc, acc2);
                 else if constexpr (g1 < 2 * kSideBatches)
-                    batch_step_exec<NM, true, (g1 - kSideBatches) * 64, (g1 - kSideBatches) * 32, wo>(cur, nxt, bmV, ixV, rel,
-                                                                                                    zaddr, wbase, wgroup, acc);
+                    batch_step_exec<NM, true, (g1 - kSideBatches) * 64, (g1 - kSideBatches) * 32, wo>(
+                        cur, nxt, bmV, ixV, rel, zaddr, wbase, wgroup, acc, acc2);
                 else if constexpr (MULTI)
-                    batch_step_exec<NM, true, 0, 0, wo>(cur, nxt, bmK + adv, ixK + adv, rel, zaddr, wbase, wgroup, acc);
+                    batch_step_exec<NM, true, 0, 0, wo>(cur, nxt, bmK + adv, ixK + adv, rel, zaddr, wbase, wgroup, acc, acc2);
                 else
-                    batch_step_exec<NM, false, 0, 0, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc);
+                    batch_step_exec<NM, false, 0, 0, wo>(cur, nxt, bmK, ixK, rel, zaddr, wbase, wgroup, acc, acc2);
                 cur = nxt;
             });
         };
@@ -176,9 +181,12 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
         for (int r = 0; r < (MULTI ? nb : 1); r++) {
             const int adv = (MULTI && r + 1 < nb) ? D : 0;  // tiles to the coming block of this wavefront
             f4_t acc_k[NM], blk_v[NM][2];
+            f4_t acc2[NM];  // the second set of sums of the gather statements (batch_step_dual), folded in per phase
             float m_blk[NM], l_blk[NM];
+            constexpr bool kDual = NM == 1 && MSTF_DUAL_ACC;
 #pragma unroll
             for (int m = 0; m < NM; m++) {
+                acc2[m] = f4_t{0.f, 0.f, 0.f, 0.f};
                 acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
                 blk_v[m][0] = f4_t{0.f, 0.f, 0.f, 0.f};
                 blk_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
@@ -194,9 +202,14 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
                 const uint32_t buf = lbase + (uint32_t)(n & 1) * kSubBytes;
                 if constexpr (n < kKeySubs) {
                     stage_batches(nc, buf, qrow, std::integral_constant<int, n * kSubTiles * 2>{}, (uint32_t)D * 8u, acc_k,
-                                  adv);
+                                  acc2, adv);
                 } else {
                     if constexpr (n == kKeySubs) {
+                        if constexpr (kDual) {
+                            dual_settle(acc_k[0], acc2[0]);
+                            acc_k[0] += acc2[0];
+                            acc2[0] = f4_t{0.f, 0.f, 0.f, 0.f};
+                        }
                         block_softmax<NM>(acc_k, sqrt_d, 64, pl, lane, m_blk, l_blk);
                         // its latency is covered by the value phase; the wait of the next stage completes it
                         if (MULTI) bnd_next = boundaries(ixK + adv, ixV + adv);
@@ -208,7 +221,12 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
 #pragma unroll
                     for (int m = 0; m < NM; m++) tmp[m] = blk_v[m][half];
                     stage_batches(nc, buf, prow, std::integral_constant<int, (vs % kSubsPerHalf) * kSubTiles * 2>{},
-                                  4u * kPRow, tmp, adv);
+                                  4u * kPRow, tmp, acc2, adv);
+                    if constexpr (kDual && vs % kSubsPerHalf == kSubsPerHalf - 1) {  // the half is complete
+                        dual_settle(tmp[0], acc2[0]);
+                        tmp[0] += acc2[0];
+                        acc2[0] = f4_t{0.f, 0.f, 0.f, 0.f};
+                    }
 #pragma unroll
                     for (int m = 0; m < NM; m++) blk_v[m][half] = tmp[m];
                 }

@@ -155,12 +155,16 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         const uint32_t qrow = lds_addr(ql) + (uint32_t)j * kQRow;
         const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
 
+        constexpr bool kDual = NM == 1 && MSTF_DUAL_ACC;
+        f4_t acc2[NM];  // second set of sums of the gather statements (batch_step_img_dual), folded in per phase
+#pragma unroll
+        for (int m = 0; m < NM; m++) acc2[m] = f4_t{0.f, 0.f, 0.f, 0.f};
         auto stage = [&](int n, uint2 bits, uint32_t waddr, uint32_t wgroup, f4_t (&acc)[NM]) {
             const QSide& S = n < kKeySubs ? K : V;
             const int t = (n < kKeySubs ? n : n - kKeySubs) * kSubTiles;
             dequant_stage<BIT, G32>(lds_addr(metabuf) + (uint32_t)(n & 1) * kMetaBytes,
                                lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, start_of(n), end_of(n), lane, mode);
-            stage_img_exec<NM>(S.bmp + t, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc);
+            stage_img_exec<NM>(S.bmp + t, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc, acc2);
         };
 
 #pragma unroll
@@ -171,7 +175,14 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             if (n < kKeySubs) {
                 stage(n, bits, qrow + (uint32_t)n * kSubTiles * 2u, 4u * kQRow, acc_k);
             } else {
-                if (n == kKeySubs) block_softmax<NM, kPRow>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
+                if (n == kKeySubs) {
+                    if constexpr (kDual) {
+                        dual_settle(acc_k[0], acc2[0]);
+                        acc_k[0] += acc2[0];
+                        acc2[0] = f4_t{0.f, 0.f, 0.f, 0.f};
+                    }
+                    block_softmax<NM, kPRow>(acc_k, sqrt_d, 64, pl, lane, m_run, l_run);
+                }
                 const int vs = n - kKeySubs;  // value stage: half = vs / 2, tokens (vs % 2) * 32..
                 constexpr int kSubsPerHalf = 64 / kSubTiles;
                 const int half = vs / kSubsPerHalf;
@@ -179,6 +190,11 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
 #pragma unroll
                 for (int m = 0; m < NM; m++) tmp[m] = acc_v[m][half];
                 stage(n, bits, prow + (uint32_t)(vs % kSubsPerHalf) * kSubTiles * 2u, 4u * kPRow, tmp);
+                if (kDual && vs % kSubsPerHalf == kSubsPerHalf - 1) {  // the half is complete
+                    dual_settle(tmp[0], acc2[0]);
+                    tmp[0] += acc2[0];
+                    acc2[0] = f4_t{0.f, 0.f, 0.f, 0.f};
+                }
 #pragma unroll
                 for (int m = 0; m < NM; m++) acc_v[m][half] = tmp[m];
             }

@@ -290,6 +290,60 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
     return m;
 }
 
+// batch_step_img_exec (below) for one accumulator group in the form without packing (batch_step_dual in
+// spmv_device.hpp: even tiles into the low halves, odd ones into the high halves of their registers, two sets of sums,
+// the gather registers cleared by vector moves, the weights in MSTF_GB0_3).
+template <bool PREFETCH, int BOFF, int IMG, int WOFF>
+__device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t& nxt, const uint64_t* bm, uint32_t img,
+                                                    uint32_t wbase, f4_t& acc, f4_t& acc2)
+{
+#define MSTF_TILE(I, LD, H, A)                                   \
+    "s_brev_b64 exec, %[m" #I "]\n\t"                            \
+    "v_mbcnt_lo_u32_b32 " A ", exec_lo, 0\n\t"                   \
+    "v_mbcnt_hi_u32_b32 " A ", exec_hi, " A "\n\t"               \
+    "v_lshl_add_u32 " A ", " A ", 1, %[img]\n\t"                 \
+    LD " " H ", " A " offset:%[i" #I "]\n\t"
+#define MSTF_LO "ds_read_u16"
+#define MSTF_HI "ds_read_u16_d16_hi"
+#define MSTF_GATHER                                                                                                  \
+    "ds_read_b128 " MSTF_GB0_3 ", %[wa] offset:%[woff]\n\t"                                                          \
+    "v_mov_b64 " MSTF_GV0_1 ", 0\n\tv_mov_b64 " MSTF_GV2_3 ", 0\n\tv_mov_b64 " MSTF_GV4_5 ", 0\n\tv_mov_b64 " MSTF_GV6_7 ", 0\n\t" \
+    MSTF_TILE(0, MSTF_LO, MSTF_GV0, MSTF_GV8) MSTF_TILE(1, MSTF_HI, MSTF_GV2, MSTF_GV9)                              \
+    MSTF_TILE(2, MSTF_LO, MSTF_GV1, MSTF_GV10) MSTF_TILE(3, MSTF_HI, MSTF_GV3, MSTF_GV11)                            \
+    MSTF_TILE(4, MSTF_LO, MSTF_GV4, MSTF_GV12) MSTF_TILE(5, MSTF_HI, MSTF_GV6, MSTF_GV13)                            \
+    MSTF_TILE(6, MSTF_LO, MSTF_GV5, MSTF_GV14) MSTF_TILE(7, MSTF_HI, MSTF_GV7, MSTF_GV15)                            \
+    "s_mov_b64 exec, -1\n\t"                                                                                         \
+    "s_waitcnt lgkmcnt(4)\n\t"                                                                                       \
+    "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV0_1 ", " MSTF_GB0_1 ", %[aa]\n\t"                                      \
+    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV2_3 ", " MSTF_GB0_1 ", %[ab]\n\t"                                      \
+    "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
+    "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV4_5 ", " MSTF_GB2_3 ", %[aa]\n\t"                                      \
+    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]"
+#define MSTF_IN                                                                                                      \
+    [m0] "s"(u64_of(mv[0], mv[1])), [m1] "s"(u64_of(mv[2], mv[3])), [m2] "s"(u64_of(mv[4], mv[5])),                  \
+        [m3] "s"(u64_of(mv[6], mv[7])), [m4] "s"(u64_of(mv[8], mv[9])), [m5] "s"(u64_of(mv[10], mv[11])),            \
+        [m6] "s"(u64_of(mv[12], mv[13])), [m7] "s"(u64_of(mv[14], mv[15])), [img] "s"(img), [wa] "v"(wbase),         \
+        [woff] "i"(WOFF), [i0] "i"(IMG), [i1] "i"(IMG + kImgStride), [i2] "i"(IMG + 2 * kImgStride),                 \
+        [i3] "i"(IMG + 3 * kImgStride), [i4] "i"(IMG + 4 * kImgStride), [i5] "i"(IMG + 5 * kImgStride),              \
+        [i6] "i"(IMG + 6 * kImgStride), [i7] "i"(IMG + 7 * kImgStride)
+#define MSTF_CLOBBER MSTF_GV_CLOBBER, MSTF_GB_CLOBBER, "memory"
+    if constexpr (PREFETCH) {
+        asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t" MSTF_GATHER
+                     : [aa] "+v"(acc), [ab] "+v"(acc2), [nm] "=&s"(nxt)
+                     : MSTF_IN, [nb] "s"(bm), [boff] "i"(BOFF)
+                     : MSTF_CLOBBER);
+    } else {
+        asm volatile(MSTF_GATHER : [aa] "+v"(acc), [ab] "+v"(acc2) : MSTF_IN : MSTF_CLOBBER);
+        nxt = mv;
+    }
+#undef MSTF_TILE
+#undef MSTF_LO
+#undef MSTF_HI
+#undef MSTF_GATHER
+#undef MSTF_IN
+#undef MSTF_CLOBBER
+}
+
 // Expands 8 tiles of the image and accumulates them, the gather under the tile's exec mask (see batch_step_exec in
 // spmv_device.hpp for the statement and the MFMA layout): one statement per batch of 8 tiles on fixed registers
 // (MSTF_GV0 .. 15 of spmv_device.hpp); the image slots of tile i sit at img + IMG + kImgStride * i, so the tile's
@@ -297,8 +351,13 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
 // requested first and completed by the statement's wait.
 template <int NM, bool PREFETCH, int BOFF, int IMG, int WOFF>
 __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t& nxt, const uint64_t* bm, uint32_t img,
-                                                    uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM])
+                                                    uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM],
+                                                    f4_t (&acc2)[NM])
 {
+    if constexpr (NM == 1 && MSTF_DUAL_ACC) {
+        batch_step_img_dual<PREFETCH, BOFF, IMG, WOFF>(mv, nxt, bm, img, wbase, acc[0], acc2[0]);
+        return;
+    }
     u32x4_t qm[NM];
 #pragma unroll
     for (int m = 1; m < NM; m++) qm[m] = *(MSTF_LDS const u32x4_t*)(uintptr_t)(wbase + (uint32_t)WOFF + (uint32_t)m * wgroup);
@@ -362,9 +421,12 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
 // into L2 one stage ahead) - the dequantisation in front has lane-dependent branches, so nothing scalar is carried
 // across it, and a scalar load here would be waited for on the spot; the other batches are requested one batch ahead.
 // img: LDS address of the stage's image; wbase: LDS address of w[lane & 3][first tile of the stage].
+// acc2: the second set of sums of the form without packing (one accumulator group): the caller adds it to acc when
+// its walk is over (dual_settle first).
 template <int NM>
 __device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t bm_lo, uint32_t bm_hi, uint32_t img,
-                                               uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM])
+                                               uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM],
+                                               f4_t (&acc2)[NM])
 {
     constexpr int G = kSubTiles / 8;
     u32x16_t cur;
@@ -376,7 +438,8 @@ __device__ __forceinline__ void stage_img_exec(const uint64_t* bm, uint32_t bm_l
     static_for<G>([&](auto gc) {
         constexpr int g = decltype(gc)::value;
         u32x16_t nxt;
-        batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 8 * kImgStride, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup, acc);
+        batch_step_img_exec<NM, (g + 1 < G), (g + 1) * 64, g * 8 * kImgStride, g * 16>(cur, nxt, bm, img, zaddr, wbase, wgroup,
+                                                                                       acc, acc2);
         cur = nxt;
     });
 }

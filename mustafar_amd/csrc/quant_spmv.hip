@@ -73,6 +73,9 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
         return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(c.bmp + t) + touch8);
     };
 
+    f4_t acc2[NM];  // second set of sums of the gather statements (batch_step_img_dual)
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc2[m] = f4_t{0.f, 0.f, 0.f, 0.f};
     size_t t_cur = tile_of(0);
     uint32_t s_cur, e_cur;
     bounds(t_cur, s_cur, e_cur);
@@ -97,8 +100,12 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
                            lds_addr(wordbuf) + (uint32_t)(n & 1) * F::kWordBuf, lbase, s_now, uni(e_now), lane, mode);
         const uint64_t* bm = c.bmp + t_now;
         const uint32_t waddr = waddr_of(n);
-        stage_img_exec<NM>(bm, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc);
+        stage_img_exec<NM>(bm, bits.x, bits.y, lbase, zaddr, waddr, wgroup, acc, acc2);
         wait_lgkm0();  // every read of the image and of the staged buffers is done before they are rewritten
+    }
+    if constexpr (NM == 1 && MSTF_DUAL_ACC) {
+        dual_settle(acc[0], acc2[0]);
+        acc[0] += acc2[0];
     }
 }
 
