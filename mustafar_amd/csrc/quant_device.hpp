@@ -318,7 +318,8 @@ __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t
     "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV2_3 ", " MSTF_GB0_1 ", %[ab]\n\t"                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
     "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV4_5 ", " MSTF_GB2_3 ", %[aa]\n\t"                                      \
-    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]"
+    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]\n\t"                                      \
+    "s_nop 4"
 #define MSTF_IN                                                                                                      \
     [m0] "s"(u64_of(mv[0], mv[1])), [m1] "s"(u64_of(mv[2], mv[3])), [m2] "s"(u64_of(mv[4], mv[5])),                  \
         [m3] "s"(u64_of(mv[6], mv[7])), [m4] "s"(u64_of(mv[8], mv[9])), [m5] "s"(u64_of(mv[10], mv[11])),            \

@@ -137,7 +137,9 @@ struct Batch {
 // over), so that two products on the same accumulator are always two instructions apart, which is what the matrix
 // pipeline asks for, and the first four tiles are multiplied while the last four are still on their way from LDS
 // (LDS reads return in order, and the scalar loads of the coming batch, on the same counter, can only make that
-// first wait longer).  The gather registers are cleared by four 64-bit vector moves instead of two 16-byte LDS reads
+// first wait longer).  The statement ends with the wait states the matrix pipeline's results need before an ordinary
+// vector instruction may read them: the compiler cannot see the products in here, and under register pressure it does
+// put such reads - copies of the sums - right behind the statement.  The gather registers are cleared by four 64-bit vector moves instead of two 16-byte LDS reads
 // of a zero slot (the LDS pipe moves 16 bytes per lane for each of those); the weights arrive in four more fixed
 // registers (MSTF_GB0_3).  Same-run comparisons at batch 8: 18.6 -> 18.1 us for the fused kernel.
 template <bool PREFETCH, int BOFF, int IOFF, int WOFF>
@@ -168,7 +170,8 @@ __device__ __forceinline__ void batch_step_dual(const Batch& b, Batch& nxt, cons
     "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV2_3 ", " MSTF_GB0_1 ", %[ab]\n\t"                                      \
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
     "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV4_5 ", " MSTF_GB2_3 ", %[aa]\n\t"                                      \
-    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]"
+    "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]\n\t"                                      \
+    "s_nop 4"
 #define MSTF_GATHER_IN                                                                                               \
     [m0] "s"(u64_of(b.mv[0], b.mv[1])), [m1] "s"(u64_of(b.mv[2], b.mv[3])), [m2] "s"(u64_of(b.mv[4], b.mv[5])),      \
         [m3] "s"(u64_of(b.mv[6], b.mv[7])), [m4] "s"(u64_of(b.mv[8], b.mv[9])), [m5] "s"(u64_of(b.mv[10], b.mv[11])), \
