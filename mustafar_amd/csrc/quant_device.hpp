@@ -290,12 +290,15 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
     return m;
 }
 
+#ifndef MSTF_Q_FORM
+#define MSTF_Q_FORM 1
+#endif
 // batch_step_img_exec (below) for one accumulator group in the form without packing (batch_step_dual in
 // spmv_device.hpp: even tiles into the low halves, odd ones into the high halves of their registers, two sets of sums,
 // the gather registers cleared by vector moves, the weights in MSTF_GB0_3).
 template <bool PREFETCH, int BOFF, int IMG, int WOFF>
 __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t& nxt, const uint64_t* bm, uint32_t img,
-                                                    uint32_t wbase, f4_t& acc, f4_t& acc2)
+                                                    uint32_t zaddr, uint32_t wbase, f4_t& acc, f4_t& acc2)
 {
 #define MSTF_TILE(I, LD, H, A)                                   \
     "s_brev_b64 exec, %[m" #I "]\n\t"                            \
@@ -305,9 +308,14 @@ __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t
     LD " " H ", " A " offset:%[i" #I "]\n\t"
 #define MSTF_LO "ds_read_u16"
 #define MSTF_HI "ds_read_u16_d16_hi"
+#if MSTF_Q_FORM == 1
+#define MSTF_QCLEAR "ds_read_b128 " MSTF_GV0_3 ", %[z]\n\tds_read_b128 " MSTF_GV4_7 ", %[z]\n\t"
+#else
+#define MSTF_QCLEAR "v_mov_b64 " MSTF_GV0_1 ", 0\n\tv_mov_b64 " MSTF_GV2_3 ", 0\n\tv_mov_b64 " MSTF_GV4_5 ", 0\n\tv_mov_b64 " MSTF_GV6_7 ", 0\n\t"
+#endif
 #define MSTF_GATHER                                                                                                  \
     "ds_read_b128 " MSTF_GB0_3 ", %[wa] offset:%[woff]\n\t"                                                          \
-    "v_mov_b64 " MSTF_GV0_1 ", 0\n\tv_mov_b64 " MSTF_GV2_3 ", 0\n\tv_mov_b64 " MSTF_GV4_5 ", 0\n\tv_mov_b64 " MSTF_GV6_7 ", 0\n\t" \
+    MSTF_QCLEAR \
     MSTF_TILE(0, MSTF_LO, MSTF_GV0, MSTF_GV8) MSTF_TILE(1, MSTF_HI, MSTF_GV2, MSTF_GV9)                              \
     MSTF_TILE(2, MSTF_LO, MSTF_GV1, MSTF_GV10) MSTF_TILE(3, MSTF_HI, MSTF_GV3, MSTF_GV11)                            \
     MSTF_TILE(4, MSTF_LO, MSTF_GV4, MSTF_GV12) MSTF_TILE(5, MSTF_HI, MSTF_GV6, MSTF_GV13)                            \
@@ -326,7 +334,7 @@ __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t
         [m6] "s"(u64_of(mv[12], mv[13])), [m7] "s"(u64_of(mv[14], mv[15])), [img] "s"(img), [wa] "v"(wbase),         \
         [woff] "i"(WOFF), [i0] "i"(IMG), [i1] "i"(IMG + kImgStride), [i2] "i"(IMG + 2 * kImgStride),                 \
         [i3] "i"(IMG + 3 * kImgStride), [i4] "i"(IMG + 4 * kImgStride), [i5] "i"(IMG + 5 * kImgStride),              \
-        [i6] "i"(IMG + 6 * kImgStride), [i7] "i"(IMG + 7 * kImgStride)
+        [i6] "i"(IMG + 6 * kImgStride), [i7] "i"(IMG + 7 * kImgStride), [z] "v"(zaddr)
 #define MSTF_CLOBBER MSTF_GV_CLOBBER, MSTF_GB_CLOBBER, "memory"
     if constexpr (PREFETCH) {
         asm volatile("s_load_dwordx16 %[nm], %[nb], %[boff]\n\t" MSTF_GATHER
@@ -340,6 +348,7 @@ __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t
 #undef MSTF_TILE
 #undef MSTF_LO
 #undef MSTF_HI
+#undef MSTF_QCLEAR
 #undef MSTF_GATHER
 #undef MSTF_IN
 #undef MSTF_CLOBBER
@@ -355,8 +364,8 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
                                                     uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM],
                                                     f4_t (&acc2)[NM])
 {
-    if constexpr (NM == 1 && MSTF_DUAL_ACC) {
-        batch_step_img_dual<PREFETCH, BOFF, IMG, WOFF>(mv, nxt, bm, img, wbase, acc[0], acc2[0]);
+    if constexpr (NM == 1 && MSTF_DUAL_ACC && MSTF_Q_FORM != 2) {
+        batch_step_img_dual<PREFETCH, BOFF, IMG, WOFF>(mv, nxt, bm, img, zaddr, wbase, acc[0], acc2[0]);
         return;
     }
     u32x4_t qm[NM];

@@ -124,7 +124,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
     __shared__ __attribute__((aligned(16))) char lds[4][kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
-    const int task = (int)blockIdx.x * 4 + wave;
+    // neighbouring token blocks on the same XCD: their packed words share cache lines
+    const int task = xcd_contiguous((int)blockIdx.x, (ntasks + 3) / 4) * 4 + wave;
     if (task >= ntasks) return;
     const int kv = task / nblk;
     const int tb = task - kv * nblk;
@@ -168,13 +169,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
 }
 
 // ------------------------------------------------------------------------------- value
-// grid = (token splits, D/64 halves, KV heads); see value_spmv_kernel.
+// grid = xcd_grid(token splits x D/64 halves x KV heads), halves fastest in the logical index: the two halves of a
+// token range read the same weights and interleaved cache lines, so they run on the same XCD; see value_spmv_kernel.
 template <int NW, int WAVES, int BIT, bool G32>
 __global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
     const uint64_t* __restrict__ bmp, const uint32_t* packed, const uint32_t* __restrict__ tile_off,
     const uint32_t* tile_off_dma, const uint16_t* scales, const uint16_t* zeros, const _Float16* P,
     _Float16* __restrict__ C, float* __restrict__ part, int Lc, int D, int nblk, int nbpw, int nsplit, int rows_per_kv,
-    int row0, int mode)
+    int row0, int mode, int nwg)
 {
     constexpr int NM = (NW + 3) / 4;
     constexpr int kWRow = kSubTiles * 2;
@@ -185,9 +187,12 @@ __global__ __launch_bounds__(WAVES * 64) void value_spmv_quant_kernel(
     __shared__ __attribute__((aligned(16))) char lds[WAVES][kWaveLds];
     const int lane = lane_id();
     const int wave = wave_id();
-    const int split = (int)blockIdx.x;
-    const int half = (int)blockIdx.y;
-    const int kv = (int)blockIdx.z;
+    const int nhalf = D / 64;
+    const int logical = xcd_contiguous((int)blockIdx.x, nwg);
+    if (logical >= nwg) return;  // (the whole workgroup: no barrier is left waiting)
+    const int half = logical % nhalf;
+    const int split = (logical / nhalf) % nsplit;
+    const int kv = logical / (nhalf * nsplit);
     const size_t T = (size_t)Lc * D / 64;
     const QCache c = {bmp, tile_off, tile_off_dma, scales, zeros, packed};
     const _Float16* wk = P + ((size_t)kv * rows_per_kv + row0) * Lc;
@@ -273,10 +278,10 @@ static void launch_key_q(hipStream_t st, const QArgs& a, const _Float16* Bm, _Fl
     const int nblk = Lc / 64;
     const int ntasks = Bkv * nblk;
     if (a.group_size == 32)
-        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, true>), dim3((ntasks + 3) / 4), dim3(256), 0, st, a.bmp, a.packed,
+        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, true>), dim3(xcd_grid((ntasks + 3) / 4)), dim3(256), 0, st, a.bmp, a.packed,
                            a.tile_off, a.tile_off, a.scales, a.zeros, Bm, C, Lc, D, nblk, ntasks, rows_per_kv, row0, a.mode);
     else
-        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, false>), dim3((ntasks + 3) / 4), dim3(256), 0, st, a.bmp, a.packed,
+        hipLaunchKernelGGL((key_spmv_quant_kernel<NW, BIT, false>), dim3(xcd_grid((ntasks + 3) / 4)), dim3(256), 0, st, a.bmp, a.packed,
                            a.tile_off, a.tile_off, a.scales, a.zeros, Bm, C, Lc, D, nblk, ntasks, rows_per_kv, row0, a.mode);
 }
 template <int NW>
@@ -295,14 +300,15 @@ template <int NW, int WAVES, int BIT>
 static void launch_value_q(hipStream_t st, const ValuePlan& pl, const QArgs& a, const _Float16* P, _Float16* C,
                            float* part, int Lc, int D, int Bkv, int rows_per_kv, int row0)
 {
+    const int nwg = pl.nsplit * (D / 64) * Bkv;
     if (a.group_size == 32)
-        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, true>), dim3(pl.nsplit, D / 64, Bkv), dim3(WAVES * 64), 0,
+        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, true>), dim3(xcd_grid(nwg)), dim3(WAVES * 64), 0,
                            st, a.bmp, a.packed, a.tile_off, a.tile_off, a.scales, a.zeros, P, C, part, Lc, D, Lc / 64,
-                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode);
+                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode, nwg);
     else
-        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, false>), dim3(pl.nsplit, D / 64, Bkv), dim3(WAVES * 64), 0,
+        hipLaunchKernelGGL((value_spmv_quant_kernel<NW, WAVES, BIT, false>), dim3(xcd_grid(nwg)), dim3(WAVES * 64), 0,
                            st, a.bmp, a.packed, a.tile_off, a.tile_off, a.scales, a.zeros, P, C, part, Lc, D, Lc / 64,
-                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode);
+                           pl.nbpw, pl.nsplit, rows_per_kv, row0, a.mode, nwg);
 }
 template <int NW, int WAVES>
 static void launch_value_q_bit(int bit, hipStream_t st, const ValuePlan& pl, const QArgs& a, const _Float16* P,

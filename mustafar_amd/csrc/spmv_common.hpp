@@ -29,6 +29,16 @@ inline int pick_nw(int left)
     return 1;
 }
 
+// Workgroups are handed to the chip's eight XCDs round-robin by their linear index, and every XCD has an L2 of its
+// own: two workgroups that share cache lines - neighbours in memory - fetch them twice when they sit on different
+// XCDs.  xcd_contiguous turns the linear index `id` of a launch of xcd_grid(n) workgroups into a logical index such
+// that every XCD works through one contiguous eighth of the n logical workgroups; indices >= n are surplus
+// workgroups that leave at once.  (Only traffic depends on the round-robin assumption, never results.)
+inline int xcd_grid(int n) { return 8 * ((n + 7) / 8); }
+#ifdef __HIPCC__
+__device__ __forceinline__ int xcd_contiguous(int id, int n) { return (id & 7) * ((n + 7) >> 3) + (id >> 3); }
+#endif
+
 struct ValuePlan {
     int waves;   // wavefronts per workgroup
     int nbpw;    // token blocks per wavefront

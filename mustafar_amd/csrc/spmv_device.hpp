@@ -126,6 +126,22 @@ struct Batch {
 #ifndef MSTF_DUAL_ACC
 #define MSTF_DUAL_ACC 1
 #endif
+#ifndef MSTF_TAIL_KIND
+#define MSTF_TAIL_KIND 0
+#endif
+#if MSTF_TAIL_KIND == 1
+#define MSTF_DUAL_TAIL "s_nop 7"
+#elif MSTF_TAIL_KIND == 2
+#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 1"
+#elif MSTF_TAIL_KIND == 3
+#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 7"
+#elif MSTF_TAIL_KIND == 4
+#define MSTF_DUAL_TAIL "s_nop 4\n\ts_sleep 1"
+#elif MSTF_TAIL_KIND == 5
+#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 7\n\ts_nop 7"
+#else
+#define MSTF_DUAL_TAIL "s_nop 4"
+#endif
 
 // batch_step_exec (below) for one accumulator group (at most four query heads per KV head), without the packing of
 // two tiles into one register: the tiles with an even index are gathered into the low half of their register, the odd
@@ -171,7 +187,7 @@ __device__ __forceinline__ void batch_step_dual(const Batch& b, Batch& nxt, cons
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
     "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV4_5 ", " MSTF_GB2_3 ", %[aa]\n\t"                                      \
     "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]\n\t"                                      \
-    "s_nop 4"
+    MSTF_DUAL_TAIL
 #define MSTF_GATHER_IN                                                                                               \
     [m0] "s"(u64_of(b.mv[0], b.mv[1])), [m1] "s"(u64_of(b.mv[2], b.mv[3])), [m2] "s"(u64_of(b.mv[4], b.mv[5])),      \
         [m3] "s"(u64_of(b.mv[6], b.mv[7])), [m4] "s"(u64_of(b.mv[8], b.mv[9])), [m5] "s"(u64_of(b.mv[10], b.mv[11])), \
