@@ -256,6 +256,32 @@ int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, c
                                           int max_tokens, const int32_t* tokens_dev, int64_t tile_capacity, int head_dim,
                                           int Bq, int groups, void* workspace, size_t workspace_bytes);
 
+/* The whole cache side of a decode step of one layer in two launches (models/llama_mustafar_kernel.py:363-374: views
+ * of the projection outputs and apply_rotary_pos_emb; :391, :430: torch.cat of the new key / value row onto the local
+ * windows; :391-441: key SpMV | q.K_win^T, / sqrt(d), softmax, value SpMV + P_win.V_win): what
+ * mstf_window_append_f16 followed by mstf_decode_attention_window_pool_f16 compute, bit for bit, with the rotation of
+ * the query heads, the rotation and append of the new key / value row and the attention over the dense window inside
+ * the launch of the compressed tokens (extra workgroups behind the token splits; the wavefront whose window block
+ * holds the new row rotates and stores it), then the merge.  A launch costs about 5 us on this GPU whatever it does,
+ * so a step of 32 layers is 0.3 ms shorter than with the four launches of the two calls.
+ * Arguments as for those two calls: q_in / k_in / v_in [bs][n_q * 128] / [bs][n_kv * 128] fp16 with their batch
+ * strides (not rotated), cos / sin [bs][128] (rope_stride; both NULL: no rotation), the window buffers
+ * [bs * n_kv][win_stride][128]; win_len bounds the count of valid window rows AFTER the step (it sizes the launch and
+ * the workspace) and, without win_len_dev, is that count; with win_len_dev the count is read on the device.  The new
+ * row goes to row count - 1; a count outside 1 .. win_stride appends nothing and sets *overflow (nullable, sticky).
+ * The compressed side is a pooled cache (tokens_dev, tile_capacity, max_tokens as for
+ * mstf_decode_attention_window_pool_f16).  out [bs * n_q][128].  Workspace:
+ * mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, 128, bs * n_q, n_q / n_kv). */
+int mstf_decode_step_pool_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                              const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
+                              const uint32_t* v_nz_off, const mstf_half* q_in, int64_t q_stride, const mstf_half* k_in,
+                              int64_t k_stride, const mstf_half* v_in, int64_t v_stride, int bs, int n_q, int n_kv,
+                              const mstf_half* cos, const mstf_half* sin, int64_t rope_stride, mstf_half* k_win,
+                              mstf_half* v_win, int win_stride, int win_len, const int32_t* win_len_dev,
+                              uint32_t* overflow, mstf_half* out, float* lse_out, int max_tokens,
+                              const int32_t* tokens_dev, int64_t tile_capacity, int head_dim, void* workspace,
+                              size_t workspace_bytes);
+
 /* The caller's per-token work in front of the attention call, in one launch (models/llama_mustafar_kernel.py:363-374:
  * the views of the projection outputs and apply_rotary_pos_emb; :391, :430: torch.cat of the new key / value row onto
  * the local windows):

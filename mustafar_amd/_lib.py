@@ -60,6 +60,8 @@ SIGNATURES = {
     "mstf_decode_attention_window_f16": (_i, [_vp] * 12 + [_i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp, _sz]),
     "mstf_decode_attention_window_pool_f16": (_i, [_vp] * 12 + [_i, _vp, _i, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp,
                                                    _sz]),
+    "mstf_decode_step_pool_f16": (_i, [_vp] * 9 + [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _i,
+                                       _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp, _sz]),
     "mstf_window_append_f16": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp, _vp, _i64, _vp, _vp, _vp, _i,
                                _i, _vp, _vp]),
     "mstf_compress_quant_workspace_bytes": (_sz, [_i, _i, _i]),

@@ -347,6 +347,9 @@ class SparseKVCache:
         self._kbuf = self._vbuf = None      # [bs * n_kv, residual_length + CHUNK, D], first _wlen tokens valid
         self._wlen = 0
         self.max_tokens = max_tokens
+        # decode_device_proj over a pooled cache as mstf_decode_step_pool_f16 (two launches) instead of the append call
+        # followed by the attention call (four); the results are identical
+        self.step_launch = True
         self.pool_fraction = pool_fraction
         self._pool_gen = (0, 0)
         self.k_pool = self.v_pool = None
@@ -503,6 +506,11 @@ class SparseKVCache:
         n_q = q_in.shape[1] // D
         if self._owns_clock:
             self._wlen_dev += 1
+        if self.step_launch and self.k_pool is not None:
+            # rotation, append and the attention over the window inside the launch of the compressed tokens
+            return ops.decode_step_pool(self.k_pool, self.v_pool, q_in, k_in, v_in, self._kbuf, self._vbuf,
+                                        self._kbuf.shape[1], cos, sin, win_len_dev=self._wlen_dev, overflow=self._wovf,
+                                        ws=self._workspace(q_in.device)).view(bs, n_q, 1, D)
         q2 = ops.window_append(k_in, v_in, self._kbuf, self._vbuf, self._wlen + 1, q_in=q_in, cos=cos, sin=sin,
                                win_len_dev=self._wlen_dev, overflow=self._wovf)
         return self._attend_device(q2).view(bs, n_q, 1, D)
@@ -618,6 +626,7 @@ class QuantSparseKVCache(SparseKVCache):
         super().__init__(groups, head_dim, k_sparsity, v_sparsity, residual_length, fused=fused,
                          window_kernel=window_kernel, max_tokens=max_tokens, pool_fraction=pool_fraction)
         self.bit, self.dequant_mode = bit, dequant_mode
+        self.step_launch = False    # (the one-launch step exists for the fp16 format only)
         # self.k / self.v: 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales, zeros]
 
     def _attend_device(self, q2):

@@ -13,10 +13,224 @@
 // (max, sum, output) triples through LDS; token splits across workgroups are combined by a small
 // merge kernel.  Scores and probabilities never touch HBM.
 #include "fused_common.hpp"
+#include "compress_common.hpp"
 
 #include <atomic>
 
 namespace mstf {
+
+// ------------------------------------------------------------------ the whole decode step in one launch
+// The new token of a decode step for the launch that does everything the caller has to do per layer and step on the
+// cache side (models/llama_mustafar_kernel.py:363-374, 391-441): rotary embedding of the new query and key heads, the
+// append of the new key / value row to the dense window, attention over the compressed tokens and over the window.
+// Workgroups 0 .. ns-1 of a KV head are the splits of the compressed tokens (the kernel below as it is, with the query
+// rows rotated on their way into LDS); the workgroups behind them take the window, one 64-token block per wavefront,
+// and the wavefront whose block holds the new row rotates / appends it.
+struct StepArgs {
+    const _Float16* q_in;  // projection outputs of the new token: [bs][n_q * 128], [bs][n_kv * 128] x 2, not rotated
+    const _Float16* k_in;
+    const _Float16* v_in;
+    int64_t q_stride, k_stride, v_stride;  // halfs between two batch entries
+    const _Float16* cos;                   // [bs][128] (rope_stride halfs apart; 0: one position for all), or null
+    const _Float16* sin;
+    int64_t rope_stride;
+    _Float16* k_win;  // [Bkv][win_stride][128]
+    _Float16* v_win;
+    const int32_t* win_len_dev;  // valid rows AFTER this step, the new token included (null: win_len)
+    uint32_t* overflow;          // sticky: a count outside 1 .. win_stride appends nothing
+    int win_len, win_stride, n_kv, ns;
+};
+
+// The query rows of KV head kv into LDS (ql: [4*NM][128] fp16), rotated: eight lanes per query head, a lane holds
+// channels c .. c+7 and their partners 64 channels on.
+__device__ __forceinline__ void stage_query_rotated(char* ql, const StepArgs& sa, int kv, int groups, int lane)
+{
+    const int b = kv / sa.n_kv, hk = kv - b * sa.n_kv;
+    const int h = lane >> 3, c = (lane & 7) * 8;
+    if (h < groups) {
+        const _Float16* xp = sa.q_in + b * sa.q_stride + (int64_t)(hk * groups + h) * kFusedD + c;
+        uint4 o0 = *reinterpret_cast<const uint4*>(xp);
+        uint4 o1 = *reinterpret_cast<const uint4*>(xp + 64);
+        if (sa.cos) {
+            const _Float16* cp = sa.cos + b * sa.rope_stride + c;
+            const _Float16* sp = sa.sin + b * sa.rope_stride + c;
+            const uint4 c0 = *reinterpret_cast<const uint4*>(cp), c1 = *reinterpret_cast<const uint4*>(cp + 64);
+            const uint4 s0 = *reinterpret_cast<const uint4*>(sp), s1 = *reinterpret_cast<const uint4*>(sp + 64);
+            const uint4 x0 = o0, x1 = o1;
+            rope_piece(x0, x1, c0, c1, s0, s1, o0, o1);
+        }
+        *reinterpret_cast<uint4*>(ql + h * (kFusedD * 2) + c * 2) = o0;
+        *reinterpret_cast<uint4*>(ql + h * (kFusedD * 2) + c * 2 + 128) = o1;
+    }
+}
+
+// One 64-token block (wblk) of the dense window of KV head kv, by one wavefront; leaves the block's (max, sum,
+// un-normalised output) in split slot sa.ns + wblk of every query row of the head, like a split of the compressed
+// tokens.  my: the wavefront's LDS (two 4 KB value buffers first, as in the compressed path), ql: the rotated query
+// rows, pl: room for the block's weights.
+//   key phase   : lane = token holds its whole key row in registers (sixteen 16-byte loads; the lane of the new row
+//                 reads the projection output instead, rotates it and stores it to the window), so the A operands of
+//                 the products are register pairs as they are;
+//   value phase : sixteen rows at a time go through LDS (LDS-direct loads, double buffered; the new row is patched in
+//                 from registers), lane = channel reads them column-wise.
+template <int NM>
+__device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, const StepArgs& sa, float* part_o,
+                                                 float* part_ml, int kv, int groups, int nst, int wblk, float sqrt_d,
+                                                 int lane)
+{
+    constexpr int D = kFusedD;
+    constexpr int kPRow = 64 * 2;
+    const int j = lane & 3;
+    int wlen = sa.win_len_dev ? *sa.win_len_dev : sa.win_len;
+    const bool fits = wlen >= 1 && wlen <= sa.win_stride;
+    if (!fits && sa.overflow && lane == 0 && wblk == 0) *sa.overflow = 1u;
+    const int new_row = fits ? wlen - 1 : -1;
+    wlen = wlen < 0 ? 0 : (wlen > sa.win_stride ? sa.win_stride : wlen);
+    if (sa.win_len < wlen) wlen = sa.win_len;  // (the launch and the split slots are sized for win_len)
+    const int row0 = wblk * 64;
+    auto slot_of = [&](int h) { return ((size_t)kv * groups + h) * nst + sa.ns + wblk; };
+    if (row0 >= wlen) {
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            const int h = 4 * m + j;
+            if (h < groups) {
+                const size_t slot = slot_of(h);
+                *reinterpret_cast<f4_t*>(part_o + slot * D + (lane & ~3)) = f4_t{0.f, 0.f, 0.f, 0.f};
+                *reinterpret_cast<f4_t*>(part_o + slot * D + 64 + (lane & ~3)) = f4_t{0.f, 0.f, 0.f, 0.f};
+                if (lane < 4) {
+                    part_ml[slot * 2] = -INFINITY;
+                    part_ml[slot * 2 + 1] = 0.f;
+                }
+            }
+        }
+        return;
+    }
+    const int nt = wlen - row0 > 64 ? 64 : wlen - row0;
+    const int b = kv / sa.n_kv, hk = kv - b * sa.n_kv;
+    const bool has_new = new_row >= row0 && new_row < row0 + 64;  // wave-uniform
+    const bool is_new = row0 + lane == new_row;
+
+    // ---- key rows into registers
+    uint4 kr[16];
+    {
+        const int t = lane < nt ? lane : nt - 1;
+        const _Float16* krow = is_new ? sa.k_in + b * sa.k_stride + (int64_t)hk * D
+                                      : sa.k_win + ((size_t)kv * sa.win_stride + row0 + t) * D;
+#pragma unroll
+        for (int i = 0; i < 16; i++) kr[i] = *reinterpret_cast<const uint4*>(krow + 8 * i);
+    }
+    if (has_new) {
+        if (sa.cos) {
+            // every lane runs the rotation on its row, the lane of the new row keeps the result
+            const _Float16* cp = sa.cos + b * sa.rope_stride;
+            const _Float16* sp = sa.sin + b * sa.rope_stride;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint4 c0 = *reinterpret_cast<const uint4*>(cp + 8 * i), c1 = *reinterpret_cast<const uint4*>(cp + 64 + 8 * i);
+                const uint4 s0 = *reinterpret_cast<const uint4*>(sp + 8 * i), s1 = *reinterpret_cast<const uint4*>(sp + 64 + 8 * i);
+                uint4 o0, o1;
+                rope_piece(kr[i], kr[i + 8], c0, c1, s0, s1, o0, o1);
+                if (is_new) {
+                    kr[i] = o0;
+                    kr[i + 8] = o1;
+                }
+            }
+        }
+        if (is_new) {
+            _Float16* dst = sa.k_win + ((size_t)kv * sa.win_stride + new_row) * D;
+#pragma unroll
+            for (int i = 0; i < 16; i++) *reinterpret_cast<uint4*>(dst + 8 * i) = kr[i];
+        }
+    }
+    if (lane >= nt) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) kr[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+
+    // ---- scores: channel c of the row x the query rows (B operand: the weights of accumulator lane & 3)
+    f4_t acc_k[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc_k[m] = f4_t{0.f, 0.f, 0.f, 0.f};
+    const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+            const u32x4_t w = *(MSTF_LDS const u32x4_t*)(uintptr_t)(qrow + (uint32_t)i * 16u + (uint32_t)m * (D * 8u));
+            acc_k[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(kr[i].x, kr[i].y), as_h4(w[0], w[1]), acc_k[m], 0, 0, 0);
+            acc_k[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(kr[i].z, kr[i].w), as_h4(w[2], w[3]), acc_k[m], 0, 0, 0);
+        }
+    }
+    float m_run[NM], l_run[NM];
+    block_softmax<NM>(acc_k, sqrt_d, nt, pl, lane, m_run, l_run);
+
+    // ---- values: sixteen rows (4 KB) at a time through LDS
+    f4_t acc_v[NM][2];
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc_v[m][0] = acc_v[m][1] = f4_t{0.f, 0.f, 0.f, 0.f};
+    uint4 vnew = make_uint4(0u, 0u, 0u, 0u);
+    if (has_new) {
+        vnew = *reinterpret_cast<const uint4*>(sa.v_in + b * sa.v_stride + (int64_t)hk * D + (lane & 15) * 8);
+        if (lane < 16) *reinterpret_cast<uint4*>(sa.v_win + ((size_t)kv * sa.win_stride + new_row) * D + lane * 8) = vnew;
+    }
+    const char* vsrc = reinterpret_cast<const char*>(sa.v_win + ((size_t)kv * sa.win_stride + row0) * D);
+    auto issue_rows = [&](int qd) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int row = qd * 16 + i * 4 + (lane >> 4);
+            if (row < nt) dma16(vsrc + (size_t)row * (D * 2) + (lane & 15) * 16, my + (qd & 1) * 4096 + i * 1024);
+        }
+    };
+    const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
+    issue_rows(0);
+#pragma unroll
+    for (int qd = 0; qd < 4; qd++) {
+        if (qd * 16 >= nt) break;  // wave-uniform
+        wait_vm0();
+        wait_lgkm0();  // the reads of the other buffer (two quarters back) are done before it is filled again
+        __builtin_amdgcn_sched_barrier(0);
+        if (qd + 1 < 4) issue_rows(qd + 1);
+        char* buf = my + (qd & 1) * 4096;
+        // the new row is not in the window buffer yet as far as this wavefront's loads can tell: from registers
+        if (has_new && new_row - row0 >= qd * 16 && new_row - row0 < qd * 16 + 16 && lane < 16)
+            *reinterpret_cast<uint4*>(buf + (new_row - row0 - qd * 16) * (D * 2) + lane * 16) = vnew;
+        // rows behind the window's end have weight 0, but what LDS holds there may be anything: zeros
+        for (int r = nt > qd * 16 ? nt : qd * 16; r < qd * 16 + 16; r++)
+            if (lane < 16) *reinterpret_cast<uint4*>(buf + (r - qd * 16) * (D * 2) + lane * 16) = make_uint4(0u, 0u, 0u, 0u);
+        const uint32_t vcol = lds_addr(buf) + (uint32_t)lane * 2u;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                _Float16 h[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) h[i] = lds_load_h(vcol + (uint32_t)((g4 * 4 + i) * D * 2 + half * 128));
+                const uint32_t v0 = pack_h2(h[0], h[1]), v1 = pack_h2(h[2], h[3]);
+#pragma unroll
+                for (int m = 0; m < NM; m++) {
+                    const u32x2_t w = *(MSTF_LDS const u32x2_t*)(uintptr_t)(prow + (uint32_t)(qd * 16 + g4 * 4) * 2u +
+                                                                             (uint32_t)m * (4u * kPRow));
+                    acc_v[m][half] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(v0, v1), as_h4(w[0], w[1]), acc_v[m][half], 0, 0, 0);
+                }
+            }
+        }
+    }
+    wait_vm0();
+    // lane 4b+j holds channels 4b..4b+3 of both halves for head 4m+j
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const int h = 4 * m + j;
+        if (h < groups) {
+            const size_t slot = slot_of(h);
+            *reinterpret_cast<f4_t*>(part_o + slot * D + (lane & ~3)) = acc_v[m][0];
+            *reinterpret_cast<f4_t*>(part_o + slot * D + 64 + (lane & ~3)) = acc_v[m][1];
+            if (lane < 4) {
+                part_ml[slot * 2] = m_run[m];
+                part_ml[slot * 2 + 1] = l_run[m];
+            }
+        }
+    }
+}
 
 // grid = (token splits, KV heads), kFusedWaves wavefronts; wavefront w of split s owns the bpw consecutive token
 // blocks (s*kFusedWaves + w)*bpw ...  NM = accumulator groups of four query heads (groups <= 4*NM).
@@ -26,13 +240,15 @@ namespace mstf {
 // (max, sum, output) into running ones before the workgroup combine.
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
-template <int NM, bool MULTI>
+// STEP: the launch is a whole decode step (StepArgs above): grid = (st.ns splits + workgroups for the window, KV heads),
+// the query rows come rotated out of the projection output instead of q.
+template <int NM, bool MULTI, bool STEP = false>
 __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(MSTF_FUSED_OCCUPANCY))) void decode_attention_kernel(
     const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
     _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, size_t tstride, int groups,
-    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev)
+    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev, StepArgs st)
 {
     // tstride: tiles between the bitmap rows of two heads (offsets: one more), which is the tile count of the cached
     // tokens unless the cache is pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read
@@ -77,6 +293,15 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     char* my = lds[wave];
     char* ql = my + kNzLds;
     char* pl = ql + kQLds;
+    if constexpr (STEP) {
+        if (split >= st.ns) {  // the workgroups of the dense window: one 64-token block per wavefront
+            stage_query_rotated(ql, st, kv, groups, lane);
+            const int wblk = (split - st.ns) * kFusedWaves + wave;
+            if (wblk < (st.win_len + 63) / 64)
+                step_window_wave<NM>(my, ql, pl, st, part_o, part_ml, kv, groups, nsplit, wblk, sqrt_d, lane);
+            return;
+        }
+    }
     const uint32_t lbase = lds_addr(my);
     const uint32_t zaddr = lbase + 2 * kSubBytes;
 
@@ -132,8 +357,10 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
             return touch_sub_flat(bmK + adv, ixK + adv, off8, off4);
         };
 
-        // the query rows of this KV head: groups x D fp16, contiguous
-        {
+        // the query rows of this KV head: groups x D fp16, contiguous (STEP: rotated out of the projection output)
+        if constexpr (STEP) {
+            stage_query_rotated(ql, st, kv, groups, lane);
+        } else {
             const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
             const uint32_t qbytes = (uint32_t)groups * D * 2u;
 #pragma unroll
@@ -552,7 +779,7 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
                          const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz, const uint32_t* v_idx,
                          const uint32_t* v_nz_off, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
                          int groups, void* workspace, int write_final, int nsplit_total = 0, size_t tile_stride = 0,
-                         const int32_t* tokens_dev = nullptr)
+                         const int32_t* tokens_dev = nullptr, const StepArgs* step = nullptr)
 {
     const size_t tstride = tile_stride ? tile_stride : (size_t)tokens * head_dim / 64;
     const int Bkv = Bq / groups, nblk = tokens / 64;
@@ -563,7 +790,14 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     const int nst = nsplit_total > 0 ? nsplit_total : ns;
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * nst * head_dim;
-    const dim3 grid((unsigned)ns, (unsigned)Bkv);
+    StepArgs sa = {};
+    unsigned extra = 0;  // workgroups per KV head behind the splits: the dense window of a whole-step launch
+    if (step) {
+        sa = *step;
+        sa.ns = ns;
+        extra = (unsigned)((window_blocks(sa.win_len) + kFusedWaves - 1) / kFusedWaves);
+    }
+    const dim3 grid((unsigned)ns + extra, (unsigned)Bkv);
     const char* knz = reinterpret_cast<const char*>(k_nz);
     const char* vnz = reinterpret_cast<const char*>(v_nz);
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
@@ -572,8 +806,17 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
 #define MSTF_FD(NMV, MULTIV)                                                                                         \
     hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, \
                        k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,    \
-                       write_final, sq, bpw, tokens_dev)
-    if (groups <= 4) {
+                       write_final, sq, bpw, tokens_dev, sa)
+    if (step) {  // (token count in device memory: the MULTI form)
+        if (groups <= 4)
+            hipLaunchKernelGGL((decode_attention_kernel<1, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx,
+                               k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
+                               write_final, sq, bpw, tokens_dev, sa);
+        else
+            hipLaunchKernelGGL((decode_attention_kernel<2, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx,
+                               k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
+                               write_final, sq, bpw, tokens_dev, sa);
+    } else if (groups <= 4) {
         if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
     } else {
         if (bpw == 1) MSTF_FD(2, false); else MSTF_FD(2, true);
@@ -804,5 +1047,61 @@ extern "C" int mstf_decode_attention_window_pool_f16(void* stream, const uint64_
     if ((rc = window_launch(as_stream(stream), k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq,
                             groups, nst, ns)) != MSTF_OK)
         return rc;
+    return merge_splits(as_stream(stream), workspace, out, lse_out, nst, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_step_pool_f16(void* stream, const uint64_t* k_bmp, const mstf_half* k_nz, const uint32_t* k_idx,
+                                         const uint32_t* k_nz_off, const uint64_t* v_bmp, const mstf_half* v_nz,
+                                         const uint32_t* v_idx, const uint32_t* v_nz_off, const mstf_half* q_in,
+                                         int64_t q_stride, const mstf_half* k_in, int64_t k_stride, const mstf_half* v_in,
+                                         int64_t v_stride, int bs, int n_q, int n_kv, const mstf_half* cos,
+                                         const mstf_half* sin, int64_t rope_stride, mstf_half* k_win, mstf_half* v_win,
+                                         int win_stride, int win_len, const int32_t* win_len_dev, uint32_t* overflow,
+                                         mstf_half* out, float* lse_out, int max_tokens, const int32_t* tokens_dev,
+                                         int64_t tile_capacity, int head_dim, void* workspace, size_t workspace_bytes)
+{
+    if (!q_in || !k_in || !v_in || !k_win || !v_win || !out || !tokens_dev) return MSTF_EINVAL;
+    if ((cos == nullptr) != (sin == nullptr)) return MSTF_EINVAL;
+    if (bs <= 0 || n_q <= 0 || n_kv <= 0 || n_q % n_kv != 0) return MSTF_EINVAL;
+    if (max_tokens <= 0 || win_len <= 0 || win_stride < win_len) return MSTF_EINVAL;
+    const int groups = n_q / n_kv;
+    const int64_t Bq64 = (int64_t)bs * n_q;
+    if (Bq64 > 0x7FFFFFF0) return MSTF_EUNSUPPORTED;
+    const int Bq = (int)Bq64;
+    if (head_dim != kFusedD || max_tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (tile_capacity < (int64_t)max_tokens * head_dim / 64) return MSTF_EINVAL;
+    if (q_stride % 8 != 0 || k_stride % 8 != 0 || v_stride % 8 != 0 || rope_stride % 8 != 0) return MSTF_EALIGN;
+    if (!aligned_to(q_in, 16) || !aligned_to(k_in, 16) || !aligned_to(v_in, 16) || !aligned_to(cos, 16) ||
+        !aligned_to(sin, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)) ||
+        !aligned_to(tokens_dev, 4) || !aligned_to(overflow, 4))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    int rc = decode_check(k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q_in, max_tokens, head_dim, Bq, groups,
+                          workspace, workspace_bytes);
+    if (rc != MSTF_OK) return rc;
+    const int ns = fused_nsplit_capacity(max_tokens, Bq / groups), nst = ns + window_blocks(win_len);
+    StepArgs sa = {};
+    sa.q_in = reinterpret_cast<const _Float16*>(q_in);
+    sa.k_in = reinterpret_cast<const _Float16*>(k_in);
+    sa.v_in = reinterpret_cast<const _Float16*>(v_in);
+    sa.q_stride = q_stride;
+    sa.k_stride = k_stride;
+    sa.v_stride = v_stride;
+    sa.cos = reinterpret_cast<const _Float16*>(cos);
+    sa.sin = reinterpret_cast<const _Float16*>(sin);
+    sa.rope_stride = rope_stride;
+    sa.k_win = reinterpret_cast<_Float16*>(k_win);
+    sa.v_win = reinterpret_cast<_Float16*>(v_win);
+    sa.win_len_dev = win_len_dev;
+    sa.overflow = overflow;
+    sa.win_len = win_len;
+    sa.win_stride = win_stride;
+    sa.n_kv = n_kv;
+    rc = decode_launch(as_stream(stream), k_bmp, k_nz, k_idx, k_nz_off, v_bmp, v_nz, v_idx, v_nz_off, q_in, nullptr, max_tokens,
+                       head_dim, Bq, groups, workspace, 0, nst, (size_t)tile_capacity, tokens_dev, &sa);
+    if (rc != MSTF_OK) return rc;
     return merge_splits(as_stream(stream), workspace, out, lse_out, nst, head_dim, Bq);
 }

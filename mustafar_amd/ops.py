@@ -300,6 +300,45 @@ def decode_attention_window_pool(k_pool, v_pool, q, k_win, v_win, win_len, group
     return o
 
 
+def decode_step_pool(k_pool, v_pool, q_in, k_in, v_in, k_win, v_win, win_len, cos=None, sin=None, win_len_dev=None,
+                     overflow=None, out=None, lse=None, ws=None):
+    """The cache side of a decode step in two launches (mstf_decode_step_pool_f16): window_append followed by
+    decode_attention_window_pool, bit for bit, with rotation, append and the attention over the window inside the
+    launch of the compressed tokens.  q_in [bs, n_q * D], k_in / v_in [bs, n_kv * D]: the projection outputs of the
+    new token (views with a batch stride are fine); cos, sin [D] or [bs, D] or None; k_win, v_win
+    [bs * n_kv, win_stride, D]; win_len bounds the count of valid rows after the step, win_len_dev holds it."""
+    D = k_win.shape[-1]
+    bs = k_in.shape[0]
+    n_kv, n_q = k_in.shape[-1] // D, q_in.shape[-1] // D
+    for t in (q_in, k_in, v_in):
+        assert t.dtype == torch.float16 and t.dim() == 2 and t.stride(1) == 1 and t.shape[0] == bs
+    assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
+    assert k_win.shape[0] == bs * n_kv and v_in.shape[-1] == n_kv * D and n_q % n_kv == 0
+    assert k_pool.max_tokens == v_pool.max_tokens
+    rope_stride = 0
+    if cos is not None:
+        assert cos.dtype == torch.float16 and sin.dtype == torch.float16 and cos.shape == sin.shape
+        assert cos.shape[-1] == D and cos.stride(-1) == 1 and sin.stride(-1) == 1
+        if cos.dim() == 2 and cos.shape[0] > 1:
+            assert cos.shape[0] == bs and cos.stride(0) == sin.stride(0)
+            rope_stride = cos.stride(0)
+    L = lib()
+    Bq = bs * n_q
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q_in.device) if out is None else out
+    ws = workspace(q_in.device, L.mstf_decode_attention_window_workspace_bytes(k_pool.max_tokens, int(win_len), D, Bq,
+                                                                              n_q // n_kv), ws)
+    cp = [t.data_ptr() for t in (k_pool.bmp_store, k_pool.nz, k_pool.idx_store, k_pool.nz_off, v_pool.bmp_store, v_pool.nz,
+                                 v_pool.idx_store, v_pool.nz_off)]
+    check(L.mstf_decode_step_pool_f16(
+        _stream(), *cp, q_in.data_ptr(), q_in.stride(0), k_in.data_ptr(), k_in.stride(0), v_in.data_ptr(), v_in.stride(0),
+        bs, n_q, n_kv, cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None,
+        rope_stride, k_win.data_ptr(), v_win.data_ptr(), k_win.shape[1], int(win_len),
+        win_len_dev.data_ptr() if win_len_dev is not None else None, overflow.data_ptr() if overflow is not None else None,
+        o.data_ptr(), lse.data_ptr() if lse is not None else None, k_pool.max_tokens, k_pool.tokens_dev.data_ptr(),
+        k_pool.tile_capacity, D, ws.data_ptr(), ws.numel()), "mstf_decode_step_pool_f16")
+    return o
+
+
 def window_append(k_in, v_in, k_win, v_win, win_len, q_in=None, cos=None, sin=None, q_out=None, win_len_dev=None,
                   overflow=None):
     """The per-token work in front of the attention call in one launch (models/llama_mustafar_kernel.py:363-374, 391,

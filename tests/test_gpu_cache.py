@@ -375,3 +375,65 @@ def test_caches_sharing_a_window_counter_advance_together():
         for c in shared:
             c.advance()
     assert shared[0].compressed_length == lone[0].compressed_length == 512
+
+
+@pytest.mark.parametrize("bs,n_kv,g,L0,steps,per_entry", [(2, 2, 4, 600, 200, False), (1, 1, 8, 300, 70, True),
+                                                           (3, 2, 2, 1100, 40, False)])
+def test_two_launch_step_equals_the_append_and_attention_calls(bs, n_kv, g, L0, steps, per_entry):
+    """mstf_decode_step_pool_f16 (rotation, append and window attention inside the launch of the compressed tokens,
+    then the merge) against mstf_window_append_f16 + mstf_decode_attention_window_pool_f16 on a twin cache: the
+    attention output of every step and the window buffers are identical bit for bit, across a chunk append, with an
+    empty compressed part at the start (second case), partial and full window blocks, and the count overrunning the
+    window buffer flagged the same way."""
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    D, res = 128, 256
+    n_q = n_kv * g
+    H = n_q + 2 * n_kv
+    K, V = orc.make_kv(40 + L0, bs * n_kv, L0, D)
+    Kt = torch.from_numpy(K).to(dev).view(bs, n_kv, L0, D)
+    Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, L0, D)
+    caches = []
+    for step_launch in (True, False):
+        c = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, window_kernel=True, max_tokens=1536)
+        c.step_launch = step_launch
+        c.prefill(Kt, Vt)
+        caches.append(c)
+    a, b = caches
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(L0)
+    for t in range(steps):
+        proj = torch.randn((bs, H * D), generator=gen, device=dev, dtype=torch.float32).half()
+        pos = np.arange(bs) * 7 + L0 + t if per_entry else np.full(bs, L0 + t)
+        cos, sin = orc.rope_tables(pos)
+        ct = torch.from_numpy(cos if per_entry else cos[0]).to(dev)
+        st = torch.from_numpy(sin if per_entry else sin[0]).to(dev)
+        outs = [c.decode_device_proj(proj[:, : n_q * D], proj[:, n_q * D: (n_q + n_kv) * D], proj[:, (n_q + n_kv) * D:], ct, st)
+                for c in (a, b)]
+        assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)), t
+        w = a._wlen + 1
+        assert torch.equal(a._kbuf[:, :w].view(torch.int16), b._kbuf[:, :w].view(torch.int16)), t
+        assert torch.equal(a._vbuf[:, :w].view(torch.int16), b._vbuf[:, :w].view(torch.int16)), t
+        for c in (a, b):
+            c.advance()
+    assert a.compressed_length == b.compressed_length and int(a._wovf) == 0 and int(b._wovf) == 0
+
+
+def test_two_launch_step_flags_a_count_past_the_window_buffer():
+    from mustafar_amd import ops
+    from mustafar_amd.cache import SparseKVCache
+    dev = torch.device("cuda:0")
+    bs, n_kv, g, D = 1, 2, 4, 128
+    n_q = n_kv * g
+    K, V = orc.make_kv(3, bs * n_kv, 600, D)
+    c = SparseKVCache(g, D, 0.7, 0.7, 256, fused=True, window_kernel=True, max_tokens=1024)
+    c.prefill(torch.from_numpy(K).to(dev).view(bs, n_kv, 600, D), torch.from_numpy(V).to(dev).view(bs, n_kv, 600, D))
+    kb, vb = c._kbuf.clone(), c._vbuf.clone()
+    proj = torch.randn((bs, (n_q + 2 * n_kv) * D), device=dev).half()
+    big = torch.full((1,), c._kbuf.shape[1] + 1, dtype=torch.int32, device=dev)
+    ovf = torch.zeros((1,), dtype=torch.int32, device=dev)
+    out = ops.decode_step_pool(c.k_pool, c.v_pool, proj[:, : n_q * D], proj[:, n_q * D: (n_q + n_kv) * D],
+                               proj[:, (n_q + n_kv) * D:], c._kbuf, c._vbuf, c._kbuf.shape[1], win_len_dev=big, overflow=ovf)
+    torch.cuda.synchronize()
+    assert int(ovf) == 1 and torch.isfinite(out).all()
+    assert torch.equal(c._kbuf.view(torch.int16), kb.view(torch.int16)) and torch.equal(c._vbuf.view(torch.int16), vb.view(torch.int16))
