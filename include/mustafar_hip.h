@@ -261,8 +261,8 @@ int mstf_decode_attention_window_pool_f16(void* stream, const uint64_t* k_bmp, c
  * windows; :391-441: key SpMV | q.K_win^T, / sqrt(d), softmax, value SpMV + P_win.V_win): what
  * mstf_window_append_f16 followed by mstf_decode_attention_window_pool_f16 compute, bit for bit, with the rotation of
  * the query heads, the rotation and append of the new key / value row and the attention over the dense window inside
- * the launch of the compressed tokens (extra workgroups behind the token splits; the wavefront whose window block
- * holds the new row rotates and stores it), then the merge.  A launch costs about 5 us on this GPU whatever it does,
+ * the launch of the compressed tokens (wavefronts take a 64-token block of the window behind their compressed blocks;
+ * the one whose block holds the new row rotates and stores it), then the merge.  A launch costs about 5 us on this GPU whatever it does,
  * so a step of 32 layers is 0.3 ms shorter than with the four launches of the two calls.
  * Arguments as for those two calls: q_in / k_in / v_in [bs][n_q * 128] / [bs][n_kv * 128] fp16 with their batch
  * strides (not rotated), cos / sin [bs][128] (rope_stride; both NULL: no rotation), the window buffers

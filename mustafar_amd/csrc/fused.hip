@@ -23,9 +23,9 @@ namespace mstf {
 // The new token of a decode step for the launch that does everything the caller has to do per layer and step on the
 // cache side (models/llama_mustafar_kernel.py:363-374, 391-441): rotary embedding of the new query and key heads, the
 // append of the new key / value row to the dense window, attention over the compressed tokens and over the window.
-// Workgroups 0 .. ns-1 of a KV head are the splits of the compressed tokens (the kernel below as it is, with the query
-// rows rotated on their way into LDS); the workgroups behind them take the window, one 64-token block per wavefront,
-// and the wavefront whose block holds the new row rotates / appends it.
+// The workgroups of a KV head are the splits of the compressed tokens (the kernel below as it is, with the query rows
+// rotated on their way into LDS); behind their compressed blocks, some of their wavefronts take one 64-token block of
+// the window each, and the wavefront whose block holds the new row rotates / appends it.
 struct StepArgs {
     const _Float16* q_in;  // projection outputs of the new token: [bs][n_q * 128], [bs][n_kv * 128] x 2, not rotated
     const _Float16* k_in;
@@ -240,15 +240,16 @@ __device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, c
 // (max, sum, output) into running ones before the workgroup combine.
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
-// STEP: the launch is a whole decode step (StepArgs above): grid = (st.ns splits + workgroups for the window, KV heads),
-// the query rows come rotated out of the projection output instead of q.
+// STEP: the launch is a whole decode step (StepArgs above, the first argument so that it sits at the start of the
+// kernel-argument segment): the query rows come rotated out of the projection output instead of q, and the wavefronts
+// also take the blocks of the dense window.
 template <int NM, bool MULTI, bool STEP = false>
 __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(MSTF_FUSED_OCCUPANCY))) void decode_attention_kernel(
-    const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
+    StepArgs st, const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
     const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
     const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
     _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, size_t tstride, int groups,
-    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev, StepArgs st)
+    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev)
 {
     // tstride: tiles between the bitmap rows of two heads (offsets: one more), which is the tile count of the cached
     // tokens unless the cache is pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read
@@ -293,15 +294,6 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     char* my = lds[wave];
     char* ql = my + kNzLds;
     char* pl = ql + kQLds;
-    if constexpr (STEP) {
-        if (split >= st.ns) {  // the workgroups of the dense window: one 64-token block per wavefront
-            stage_query_rotated(ql, st, kv, groups, lane);
-            const int wblk = (split - st.ns) * kFusedWaves + wave;
-            if (wblk < (st.win_len + 63) / 64)
-                step_window_wave<NM>(my, ql, pl, st, part_o, part_ml, kv, groups, nsplit, wblk, sqrt_d, lane);
-            return;
-        }
-    }
     const uint32_t lbase = lds_addr(my);
     const uint32_t zaddr = lbase + 2 * kSubBytes;
 
@@ -492,6 +484,28 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
         wait_lgkm0();
     }
 
+    if constexpr (STEP) {
+        // The dense window: its 64-token blocks are dealt out over the wavefronts of the head's workgroups - block i to
+        // wavefront i / ns of split i % ns - which take them behind their compressed blocks, so the window costs no
+        // workgroup of its own (a ninth workgroup per head would find no free slot on a full chip and run behind the
+        // others).  The query rows are still in LDS; the value buffers and the weight rows are free again.
+        // (the step's arguments are fetched again here, through a pointer the compiler cannot see through: kept in
+        // scalar registers across the walk above they would push other values out)
+        const StepArgs __attribute__((address_space(4)))* sp =
+            (const StepArgs __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(sp));
+        StepArgs sw;
+        sw.q_in = sp->q_in, sw.k_in = sp->k_in, sw.v_in = sp->v_in;
+        sw.q_stride = sp->q_stride, sw.k_stride = sp->k_stride, sw.v_stride = sp->v_stride;
+        sw.cos = sp->cos, sw.sin = sp->sin, sw.rope_stride = sp->rope_stride;
+        sw.k_win = sp->k_win, sw.v_win = sp->v_win, sw.win_len_dev = sp->win_len_dev, sw.overflow = sp->overflow;
+        sw.win_len = sp->win_len, sw.win_stride = sp->win_stride, sw.n_kv = sp->n_kv, sw.ns = sp->ns;
+        const int wblk = wave * sw.ns + split;
+        if (wblk < (sw.win_len + 63) / 64) {
+            if (!active) stage_query_rotated(ql, sw, kv, groups, lane);
+            step_window_wave<NM>(my, ql, pl, sw, part_o, part_ml, kv, groups, nsplit, wblk, sqrt_d, lane);
+        }
+    }
     workgroup_combine<NM>(&lds[0][0], kWaveLds, wave, lane, acc_v, m_run, l_run, kv, groups, split, nsplit, write_final,
                           out, part_o, part_ml);
 }
@@ -791,31 +805,31 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     float* part_o = reinterpret_cast<float*>(workspace);
     float* part_ml = part_o + (size_t)Bq * nst * head_dim;
     StepArgs sa = {};
-    unsigned extra = 0;  // workgroups per KV head behind the splits: the dense window of a whole-step launch
     if (step) {
         sa = *step;
         sa.ns = ns;
-        extra = (unsigned)((window_blocks(sa.win_len) + kFusedWaves - 1) / kFusedWaves);
+        // the window's blocks are dealt out over the ns * kFusedWaves wavefronts of a head
+        if (window_blocks(sa.win_len) > ns * kFusedWaves) return MSTF_EUNSUPPORTED;
     }
-    const dim3 grid((unsigned)ns + extra, (unsigned)Bkv);
+    const dim3 grid((unsigned)ns, (unsigned)Bkv);
     const char* knz = reinterpret_cast<const char*>(k_nz);
     const char* vnz = reinterpret_cast<const char*>(v_nz);
     const _Float16* qh = reinterpret_cast<const _Float16*>(q);
     _Float16* oh = reinterpret_cast<_Float16*>(out);
     const float sq = sqrtf((float)head_dim);
 #define MSTF_FD(NMV, MULTIV)                                                                                         \
-    hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx, \
+    hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx, \
                        k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,    \
-                       write_final, sq, bpw, tokens_dev, sa)
+                       write_final, sq, bpw, tokens_dev)
     if (step) {  // (token count in device memory: the MULTI form)
         if (groups <= 4)
-            hipLaunchKernelGGL((decode_attention_kernel<1, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx,
+            hipLaunchKernelGGL((decode_attention_kernel<1, true, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx,
                                k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
-                               write_final, sq, bpw, tokens_dev, sa);
+                               write_final, sq, bpw, tokens_dev);
         else
-            hipLaunchKernelGGL((decode_attention_kernel<2, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp, knz, k_idx,
+            hipLaunchKernelGGL((decode_attention_kernel<2, true, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx,
                                k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
-                               write_final, sq, bpw, tokens_dev, sa);
+                               write_final, sq, bpw, tokens_dev);
     } else if (groups <= 4) {
         if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
     } else {

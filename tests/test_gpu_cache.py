@@ -428,6 +428,9 @@ def test_two_launch_step_flags_a_count_past_the_window_buffer():
     K, V = orc.make_kv(3, bs * n_kv, 600, D)
     c = SparseKVCache(g, D, 0.7, 0.7, 256, fused=True, window_kernel=True, max_tokens=1024)
     c.prefill(torch.from_numpy(K).to(dev).view(bs, n_kv, 600, D), torch.from_numpy(V).to(dev).view(bs, n_kv, 600, D))
+    # (the attention of such a step covers the whole buffer, rows never written included: give them values)
+    torch.nan_to_num_(c._kbuf, nan=0.0, posinf=0.0, neginf=0.0).clamp_(-4, 4)
+    torch.nan_to_num_(c._vbuf, nan=0.0, posinf=0.0, neginf=0.0).clamp_(-4, 4)
     kb, vb = c._kbuf.clone(), c._vbuf.clone()
     proj = torch.randn((bs, (n_q + 2 * n_kv) * D), device=dev).half()
     big = torch.full((1,), c._kbuf.shape[1] + 1, dtype=torch.int32, device=dev)
