@@ -387,6 +387,23 @@ int mstf_decode_attention_window_quant_pool(void* stream, const uint64_t* k_bmp,
                                             int groups, int bit, int capacity, int dequant_mode, void* workspace,
                                             size_t workspace_bytes);
 
+/* mstf_decode_step_pool_f16 for the quantised pooled cache: the cache side of a decode step of one layer in two
+ * launches (models/llama_mustafar_quant_kernel.py:445-567: rotation of the new query / key heads, torch.cat of the new
+ * key / value row onto the local windows, key formulation | q.K_win^T, / sqrt(d), softmax, value formulation +
+ * P_win.V_win) - what mstf_window_append_f16 followed by mstf_decode_attention_window_quant_pool compute, bit for bit.
+ * Step arguments as for mstf_decode_step_pool_f16, cache arguments as for mstf_decode_attention_window_quant_pool
+ * (one scale / zero pair per tile). */
+int mstf_decode_step_quant_pool(void* stream, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off,
+                                const mstf_half* k_scales, const mstf_half* k_zeros, const uint64_t* v_bmp,
+                                const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
+                                const mstf_half* v_zeros, const mstf_half* q_in, int64_t q_stride, const mstf_half* k_in,
+                                int64_t k_stride, const mstf_half* v_in, int64_t v_stride, int bs, int n_q, int n_kv,
+                                const mstf_half* cos, const mstf_half* sin, int64_t rope_stride, mstf_half* k_win,
+                                mstf_half* v_win, int win_stride, int win_len, const int32_t* win_len_dev,
+                                uint32_t* overflow, mstf_half* out, float* lse_out, int max_tokens,
+                                const int32_t* tokens_dev, int64_t tile_capacity, int head_dim, int bit, int capacity,
+                                int dequant_mode, void* workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ group-32 scale / zero option
  * No counterpart in the reference's kernels: its harness carries GROUP_SIZE = 32 (benchmark/mem_spd_test_quant.py:33,
  * 104) but the producer quantises per 64-element tile (kernel_quant/compression_quant.py:47-57, 209-210).  With

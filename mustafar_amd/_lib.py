@@ -62,6 +62,8 @@ SIGNATURES = {
                                                    _sz]),
     "mstf_decode_step_pool_f16": (_i, [_vp] * 9 + [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _i,
                                        _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp, _sz]),
+    "mstf_decode_step_quant_pool": (_i, [_vp] * 11 + [_vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp, _vp, _i64, _vp, _vp, _i,
+                                         _i, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _vp, _sz]),
     "mstf_window_append_f16": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _vp, _vp, _i64, _vp, _vp, _vp, _i,
                                _i, _vp, _vp]),
     "mstf_compress_quant_workspace_bytes": (_sz, [_i, _i, _i]),

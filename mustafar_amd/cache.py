@@ -508,12 +508,16 @@ class SparseKVCache:
             self._wlen_dev += 1
         if self.step_launch and self.k_pool is not None:
             # rotation, append and the attention over the window inside the launch of the compressed tokens
-            return ops.decode_step_pool(self.k_pool, self.v_pool, q_in, k_in, v_in, self._kbuf, self._vbuf,
-                                        self._kbuf.shape[1], cos, sin, win_len_dev=self._wlen_dev, overflow=self._wovf,
-                                        ws=self._workspace(q_in.device)).view(bs, n_q, 1, D)
+            return self._step_device(q_in, k_in, v_in, cos, sin).view(bs, n_q, 1, D)
         q2 = ops.window_append(k_in, v_in, self._kbuf, self._vbuf, self._wlen + 1, q_in=q_in, cos=cos, sin=sin,
                                win_len_dev=self._wlen_dev, overflow=self._wovf)
         return self._attend_device(q2).view(bs, n_q, 1, D)
+
+    def _step_device(self, q_in, k_in, v_in, cos, sin):
+        """The cache side of a step from the projection outputs in two launches; returns [Bq, D]."""
+        return ops.decode_step_pool(self.k_pool, self.v_pool, q_in, k_in, v_in, self._kbuf, self._vbuf,
+                                    self._kbuf.shape[1], cos, sin, win_len_dev=self._wlen_dev, overflow=self._wovf,
+                                    ws=self._workspace(q_in.device))
 
     def _attend_device(self, q2):
         """Attention of the query rows q2 [Bq, D] over [compressed | window buffer] (three launches)."""
@@ -626,8 +630,13 @@ class QuantSparseKVCache(SparseKVCache):
         super().__init__(groups, head_dim, k_sparsity, v_sparsity, residual_length, fused=fused,
                          window_kernel=window_kernel, max_tokens=max_tokens, pool_fraction=pool_fraction)
         self.bit, self.dequant_mode = bit, dequant_mode
-        self.step_launch = False    # (the one-launch step exists for the fp16 format only)
         # self.k / self.v: 7-element lists [bitmaps, tile_offsets, packed, counts, units, scales, zeros]
+
+    def _step_device(self, q_in, k_in, v_in, cos, sin):
+        from . import mustafar_package_quant as mpq
+        return mpq.decode_step_quant_pool(self.k_pool, self.v_pool, q_in, k_in, v_in, self._kbuf, self._vbuf,
+                                          self._kbuf.shape[1], cos, sin, self.dequant_mode, win_len_dev=self._wlen_dev,
+                                          overflow=self._wovf, ws=self._workspace(q_in.device))
 
     def _attend_device(self, q2):
         from . import mustafar_package_quant as mpq

@@ -6,6 +6,7 @@
 // tiles.  A stage's packed words and metadata arrive by LDS-direct loads one stage ahead (double buffers); the
 // stage is dequantised into the wavefront's fp16 tile image and expanded from there.
 #include "fused_common.hpp"
+#include "step_device.hpp"
 
 #ifndef MSTF_QPAD
 #define MSTF_QPAD 16
@@ -27,10 +28,11 @@ struct QSide {
     const uint16_t* zeros;
 };
 
-// grid = (token splits, KV heads), kFusedWaves wavefronts; see decode_attention_kernel.
-template <int NM, int BIT, bool G32>
+// grid = (token splits, KV heads), kFusedWaves wavefronts; see decode_attention_kernel.  STEP: the launch is a whole
+// decode step (st, the first argument so that it sits at the start of the kernel-argument segment; step_device.hpp).
+template <int NM, int BIT, bool G32, bool STEP = false>
 __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kernel(
-    const uint64_t* __restrict__ k_bmp, const uint32_t* k_packed, const uint32_t* __restrict__ k_off,
+    StepArgs st, const uint64_t* __restrict__ k_bmp, const uint32_t* k_packed, const uint32_t* __restrict__ k_off,
     const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros, const uint64_t* __restrict__ v_bmp,
     const uint32_t* v_packed, const uint32_t* __restrict__ v_off, const uint32_t* v_off_dma, const uint16_t* v_scales,
     const uint16_t* v_zeros, const _Float16* q, _Float16* __restrict__ out, float* __restrict__ part_o,
@@ -134,8 +136,10 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             return *reinterpret_cast<const uint2*>(reinterpret_cast<const char*>(S.bmp + t) + touch8);
         };
 
-        // the query rows of this KV head: groups x D fp16, contiguous
-        {
+        // the query rows of this KV head: groups x D fp16, contiguous (STEP: rotated out of the projection output)
+        if constexpr (STEP) {
+            stage_query_rotated<kQRow>(ql, st, kv, groups, lane);
+        } else {
             const char* qsrc = reinterpret_cast<const char*>(q + (size_t)kv * groups * D);
             // a row per load: sixteen lanes fetch the 256 bytes of query row `row`, four rows per pass
             const int row_in_pass = lane >> 4;
@@ -201,6 +205,27 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
             wait_lgkm0();  // every read of the image and of the staged buffers is done before they are rewritten
         }
     }
+    if constexpr (STEP) {
+        // The dense window: block i goes to wavefront i / ns of split i % ns, behind its compressed block (see
+        // decode_attention_kernel); the value rows pass through the room of the tile image, eight at a time.  The
+        // step's arguments are fetched again here, through a pointer the compiler cannot see through, so that they
+        // hold no scalar registers above.
+        static_assert(2 * 8 * D * 2 <= kImgBytes, "two buffers of eight value rows in the room of the image");
+        const StepArgs __attribute__((address_space(4)))* sp =
+            (const StepArgs __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(sp));
+        StepArgs sw;
+        sw.q_in = sp->q_in, sw.k_in = sp->k_in, sw.v_in = sp->v_in;
+        sw.q_stride = sp->q_stride, sw.k_stride = sp->k_stride, sw.v_stride = sp->v_stride;
+        sw.cos = sp->cos, sw.sin = sp->sin, sw.rope_stride = sp->rope_stride;
+        sw.k_win = sp->k_win, sw.v_win = sp->v_win, sw.win_len_dev = sp->win_len_dev, sw.overflow = sp->overflow;
+        sw.win_len = sp->win_len, sw.win_stride = sp->win_stride, sw.n_kv = sp->n_kv, sw.ns = sp->ns;
+        const int wblk = wave * sw.ns + split;
+        if (wblk < (sw.win_len + 63) / 64) {
+            if (!active) stage_query_rotated<kQRow>(ql, sw, kv, groups, lane);
+            step_window_wave<NM, kQRow, kPRow, 8>(my, ql, pl, sw, part_o, part_ml, kv, groups, nsplit, wblk, sqrt_d, lane);
+        }
+    }
     workgroup_combine<NM>(lds_all, kWaveLds, wave, lane, acc_v, m_run, l_run, kv, groups, split, nsplit, write_final, out,
                           part_o, part_ml);
 }
@@ -211,15 +236,22 @@ static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp
                                 const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_off,
                                 const uint16_t* v_scales, const uint16_t* v_zeros, const _Float16* q, _Float16* out,
                                 float* part_o, float* part_ml, int tokens, int groups, int ns, int write_final, float sq,
-                                int mode, int group_size, size_t tstride, const int32_t* tokens_dev, int heads_fastest)
+                                int mode, int group_size, size_t tstride, const int32_t* tokens_dev, int heads_fastest,
+                                const StepArgs* step)
 {
-    if (group_size == 32)
-        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
+    const StepArgs sa = step ? *step : StepArgs{};
+    if (step)  // (group_size is 64 there: quant_launch has checked it)
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false, true>), grid, dim3(kFusedWaves * 64), 0, st, sa,
+                           k_bmp, k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales,
+                           v_zeros, q, out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode,
+                           tokens_dev, heads_fastest);
+    else if (group_size == 32)
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp,
                            k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
                            out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
                            heads_fastest);
     else
-        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, k_bmp,
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp,
                            k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
                            out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
                            heads_fastest);
@@ -257,8 +289,12 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
                         const uint32_t* v_packed, const uint32_t* v_tile_off, const mstf_half* v_scales,
                         const mstf_half* v_zeros, const mstf_half* q, mstf_half* out, int tokens, int head_dim, int Bq,
                         int groups, int bit, int dequant_mode, void* workspace, int nst, int write_final,
-                        int group_size = 64, size_t tile_stride = 0, const int32_t* tokens_dev = nullptr)
+                        int group_size = 64, size_t tile_stride = 0, const int32_t* tokens_dev = nullptr,
+                        const StepArgs* step = nullptr)
 {
+    // step: the launch is a whole decode step; its window blocks are dealt out over the wavefronts of a head
+    if (step && (group_size != 64 || window_blocks(step->win_len) > fused_nsplit(tokens) * kFusedWaves))
+        return MSTF_EUNSUPPORTED;
     // tile_stride / tokens_dev: a cache pre-allocated for `tokens` tokens that holds *tokens_dev of them (see the kernel)
     const int Bkv = Bq / groups, ns = fused_nsplit(tokens);
     float* part_o = reinterpret_cast<float*>(workspace);
@@ -276,7 +312,7 @@ static int quant_launch(hipStream_t st, const uint64_t* k_bmp, const uint32_t* k
 #define MSTF_FQ(NMV, BITV)                                                                                             \
     launch_decode_quant<NMV, BITV>(st, grid, k_bmp, k_packed, k_tile_off, ks, kz, v_bmp, v_packed, v_tile_off, vs, vz, \
                                    qh, oh, part_o, part_ml, tokens, groups, nst, write_final, sq, dequant_mode, group_size, \
-                                   tstride, tokens_dev, heads_fastest)
+                                   tstride, tokens_dev, heads_fastest, step)
     if (groups <= 4) {
         if (bit == 2) MSTF_FQ(1, 2); else if (bit == 4) MSTF_FQ(1, 4); else MSTF_FQ(1, 8);
     } else {
@@ -409,5 +445,65 @@ extern "C" int mstf_decode_attention_window_quant_pool(
     if ((rc = window_launch(st, k_win, v_win, q, workspace, win_len, win_len_dev, win_stride, head_dim, Bq, groups, nst,
                             ns)) != MSTF_OK)
         return rc;
+    return merge_splits(st, workspace, out, lse_out, nst, head_dim, Bq);
+}
+
+extern "C" int mstf_decode_step_quant_pool(
+    void* stream, const uint64_t* k_bmp, const uint32_t* k_packed, const uint32_t* k_tile_off, const mstf_half* k_scales,
+    const mstf_half* k_zeros, const uint64_t* v_bmp, const uint32_t* v_packed, const uint32_t* v_tile_off,
+    const mstf_half* v_scales, const mstf_half* v_zeros, const mstf_half* q_in, int64_t q_stride, const mstf_half* k_in,
+    int64_t k_stride, const mstf_half* v_in, int64_t v_stride, int bs, int n_q, int n_kv, const mstf_half* cos,
+    const mstf_half* sin, int64_t rope_stride, mstf_half* k_win, mstf_half* v_win, int win_stride, int win_len,
+    const int32_t* win_len_dev, uint32_t* overflow, mstf_half* out, float* lse_out, int max_tokens,
+    const int32_t* tokens_dev, int64_t tile_capacity, int head_dim, int bit, int capacity, int dequant_mode,
+    void* workspace, size_t workspace_bytes)
+{
+    if (!q_in || !k_in || !v_in || !k_win || !v_win || !out || !tokens_dev) return MSTF_EINVAL;
+    if ((cos == nullptr) != (sin == nullptr)) return MSTF_EINVAL;
+    if (bs <= 0 || n_q <= 0 || n_kv <= 0 || n_q % n_kv != 0) return MSTF_EINVAL;
+    if (max_tokens <= 0 || win_len <= 0 || win_stride < win_len) return MSTF_EINVAL;
+    const int groups = n_q / n_kv;
+    const int64_t Bq64 = (int64_t)bs * n_q;
+    if (Bq64 > 0x7FFFFFF0) return MSTF_EUNSUPPORTED;
+    const int Bq = (int)Bq64;
+    if (head_dim != kFusedD || max_tokens % 64 != 0 || groups > 8) return MSTF_EUNSUPPORTED;
+    if (tile_capacity < (int64_t)max_tokens * head_dim / 64) return MSTF_EINVAL;
+    if (tile_capacity % 2 != 0) return MSTF_EALIGN;  // (rows of the two-byte per-tile arrays stay four-byte aligned)
+    if (q_stride % 8 != 0 || k_stride % 8 != 0 || v_stride % 8 != 0 || rope_stride % 8 != 0) return MSTF_EALIGN;
+    if (!aligned_to(q_in, 16) || !aligned_to(k_in, 16) || !aligned_to(v_in, 16) || !aligned_to(cos, 16) ||
+        !aligned_to(sin, 16) || !aligned_to(k_win, 16) || !aligned_to(v_win, 16) || !aligned_to(out, 2) ||
+        (lse_out && !aligned_to(lse_out, 4)) || (win_len_dev && !aligned_to(win_len_dev, 4)) ||
+        !aligned_to(tokens_dev, 4) || !aligned_to(overflow, 4))
+        return MSTF_EALIGN;
+    const size_t need = mstf_decode_attention_window_workspace_bytes(max_tokens, win_len, head_dim, Bq, groups);
+    if (!workspace || workspace_bytes < need) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 16)) return MSTF_EALIGN;
+    int rc = quant_check(k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros,
+                         q_in, max_tokens, head_dim, Bq, groups, bit, capacity, dequant_mode);
+    if (rc != MSTF_OK) return rc;
+    hipStream_t st = as_stream(stream);
+    const int ns = fused_nsplit(max_tokens), nst = ns + window_blocks(win_len);
+    StepArgs sa = {};
+    sa.q_in = reinterpret_cast<const _Float16*>(q_in);
+    sa.k_in = reinterpret_cast<const _Float16*>(k_in);
+    sa.v_in = reinterpret_cast<const _Float16*>(v_in);
+    sa.q_stride = q_stride;
+    sa.k_stride = k_stride;
+    sa.v_stride = v_stride;
+    sa.cos = reinterpret_cast<const _Float16*>(cos);
+    sa.sin = reinterpret_cast<const _Float16*>(sin);
+    sa.rope_stride = rope_stride;
+    sa.k_win = reinterpret_cast<_Float16*>(k_win);
+    sa.v_win = reinterpret_cast<_Float16*>(v_win);
+    sa.win_len_dev = win_len_dev;
+    sa.overflow = overflow;
+    sa.win_len = win_len;
+    sa.win_stride = win_stride;
+    sa.n_kv = n_kv;
+    sa.ns = ns;
+    rc = quant_launch(st, k_bmp, k_packed, k_tile_off, k_scales, k_zeros, v_bmp, v_packed, v_tile_off, v_scales, v_zeros,
+                      q_in, nullptr, max_tokens, head_dim, Bq, groups, bit, dequant_mode, workspace, nst, 0, 64,
+                      (size_t)tile_capacity, tokens_dev, &sa);
+    if (rc != MSTF_OK) return rc;
     return merge_splits(st, workspace, out, lse_out, nst, head_dim, Bq);
 }

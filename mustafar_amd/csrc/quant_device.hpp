@@ -290,12 +290,10 @@ __device__ __forceinline__ MetaLanes meta_lanes(const uint32_t* off_dma, const u
     return m;
 }
 
-#ifndef MSTF_Q_FORM
-#define MSTF_Q_FORM 1
-#endif
 // batch_step_img_exec (below) for one accumulator group in the form without packing (batch_step_dual in
 // spmv_device.hpp: even tiles into the low halves, odd ones into the high halves of their registers, two sets of sums,
-// the gather registers cleared by vector moves, the weights in MSTF_GB0_3).
+// the weights in MSTF_GB0_3); the gather registers are cleared by two 16-byte reads of the zero slot here - this kernel's
+// vector unit is the busier one, vector moves measured slower.
 template <bool PREFETCH, int BOFF, int IMG, int WOFF>
 __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t& nxt, const uint64_t* bm, uint32_t img,
                                                     uint32_t zaddr, uint32_t wbase, f4_t& acc, f4_t& acc2)
@@ -308,11 +306,7 @@ __device__ __forceinline__ void batch_step_img_dual(const u32x16_t& mv, u32x16_t
     LD " " H ", " A " offset:%[i" #I "]\n\t"
 #define MSTF_LO "ds_read_u16"
 #define MSTF_HI "ds_read_u16_d16_hi"
-#if MSTF_Q_FORM == 1
 #define MSTF_QCLEAR "ds_read_b128 " MSTF_GV0_3 ", %[z]\n\tds_read_b128 " MSTF_GV4_7 ", %[z]\n\t"
-#else
-#define MSTF_QCLEAR "v_mov_b64 " MSTF_GV0_1 ", 0\n\tv_mov_b64 " MSTF_GV2_3 ", 0\n\tv_mov_b64 " MSTF_GV4_5 ", 0\n\tv_mov_b64 " MSTF_GV6_7 ", 0\n\t"
-#endif
 #define MSTF_GATHER                                                                                                  \
     "ds_read_b128 " MSTF_GB0_3 ", %[wa] offset:%[woff]\n\t"                                                          \
     MSTF_QCLEAR \
@@ -364,7 +358,7 @@ __device__ __forceinline__ void batch_step_img_exec(const u32x16_t& mv, u32x16_t
                                                     uint32_t zaddr, uint32_t wbase, uint32_t wgroup, f4_t (&acc)[NM],
                                                     f4_t (&acc2)[NM])
 {
-    if constexpr (NM == 1 && MSTF_DUAL_ACC && MSTF_Q_FORM != 2) {
+    if constexpr (NM == 1 && MSTF_DUAL_ACC) {
         batch_step_img_dual<PREFETCH, BOFF, IMG, WOFF>(mv, nxt, bm, img, zaddr, wbase, acc[0], acc2[0]);
         return;
     }

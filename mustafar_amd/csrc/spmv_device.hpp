@@ -126,22 +126,6 @@ struct Batch {
 #ifndef MSTF_DUAL_ACC
 #define MSTF_DUAL_ACC 1
 #endif
-#ifndef MSTF_TAIL_KIND
-#define MSTF_TAIL_KIND 0
-#endif
-#if MSTF_TAIL_KIND == 1
-#define MSTF_DUAL_TAIL "s_nop 7"
-#elif MSTF_TAIL_KIND == 2
-#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 1"
-#elif MSTF_TAIL_KIND == 3
-#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 7"
-#elif MSTF_TAIL_KIND == 4
-#define MSTF_DUAL_TAIL "s_nop 4\n\ts_sleep 1"
-#elif MSTF_TAIL_KIND == 5
-#define MSTF_DUAL_TAIL "s_nop 7\n\ts_nop 7\n\ts_nop 7"
-#else
-#define MSTF_DUAL_TAIL "s_nop 4"
-#endif
 
 // batch_step_exec (below) for one accumulator group (at most four query heads per KV head), without the packing of
 // two tiles into one register: the tiles with an even index are gathered into the low half of their register, the odd
@@ -155,9 +139,11 @@ struct Batch {
 // (LDS reads return in order, and the scalar loads of the coming batch, on the same counter, can only make that
 // first wait longer).  The statement ends with the wait states the matrix pipeline's results need before an ordinary
 // vector instruction may read them: the compiler cannot see the products in here, and under register pressure it does
-// put such reads - copies of the sums - right behind the statement.  The gather registers are cleared by four 64-bit vector moves instead of two 16-byte LDS reads
-// of a zero slot (the LDS pipe moves 16 bytes per lane for each of those); the weights arrive in four more fixed
-// registers (MSTF_GB0_3).  Same-run comparisons at batch 8: 18.6 -> 18.1 us for the fused kernel.
+// put such reads - copies of the sums - right behind the statement (results then differ from run to run).  The
+// gather registers are cleared by four 64-bit vector moves instead of two 16-byte LDS reads of a zero slot (the LDS
+// pipe moves 16 bytes per lane for each of those); the weights arrive in four more fixed registers (MSTF_GB0_3).
+// Same-run comparisons at batch 8 for the fused kernel: 18.6 us with the packed form, 18.1 us with this one, 17.3 us
+// with the wait states at its end (the copies the compiler placed there stalled on the matrix pipeline before).
 template <bool PREFETCH, int BOFF, int IOFF, int WOFF>
 __device__ __forceinline__ void batch_step_dual(const Batch& b, Batch& nxt, const uint64_t* nbm, const uint32_t* nix,
                                                 uint32_t rel, uint32_t wbase, f4_t& acc, f4_t& acc2)
@@ -187,7 +173,7 @@ __device__ __forceinline__ void batch_step_dual(const Batch& b, Batch& nxt, cons
     "s_waitcnt lgkmcnt(0)\n\t"                                                                                       \
     "v_mfma_f32_4x4x4_16b_f16 %[aa], " MSTF_GV4_5 ", " MSTF_GB2_3 ", %[aa]\n\t"                                      \
     "v_mfma_f32_4x4x4_16b_f16 %[ab], " MSTF_GV6_7 ", " MSTF_GB2_3 ", %[ab]\n\t"                                      \
-    MSTF_DUAL_TAIL
+    "s_nop 4"
 #define MSTF_GATHER_IN                                                                                               \
     [m0] "s"(u64_of(b.mv[0], b.mv[1])), [m1] "s"(u64_of(b.mv[2], b.mv[3])), [m2] "s"(u64_of(b.mv[4], b.mv[5])),      \
         [m3] "s"(u64_of(b.mv[6], b.mv[7])), [m4] "s"(u64_of(b.mv[8], b.mv[9])), [m5] "s"(u64_of(b.mv[10], b.mv[11])), \

@@ -211,6 +211,48 @@ def decode_attention_window_quant_pool(k_pool, v_pool, q, k_win, v_win, win_len,
     return o
 
 
+def decode_step_quant_pool(k_pool, v_pool, q_in, k_in, v_in, k_win, v_win, win_len, cos=None, sin=None, dequant_mode=0,
+                           win_len_dev=None, overflow=None, out=None, lse=None, ws=None):
+    """ops.decode_step_pool over two cache.QuantPool sides (mstf_decode_step_quant_pool): ops.window_append followed
+    by decode_attention_window_quant_pool, bit for bit, in two launches - rotation of the new query / key heads,
+    append of the new rows to the window and the attention over the window run inside the launch of the compressed
+    tokens.  Arguments as for ops.decode_step_pool."""
+    D = k_win.shape[-1]
+    bs = k_in.shape[0]
+    n_kv, n_q = k_in.shape[-1] // D, q_in.shape[-1] // D
+    for t in (q_in, k_in, v_in):
+        assert t.dtype == torch.float16 and t.dim() == 2 and t.stride(1) == 1 and t.shape[0] == bs
+    assert k_win.dtype == torch.float16 and k_win.is_contiguous() and v_win.is_contiguous() and k_win.shape == v_win.shape
+    assert k_win.shape[0] == bs * n_kv and v_in.shape[-1] == n_kv * D and n_q % n_kv == 0
+    assert k_pool.max_tokens == v_pool.max_tokens and k_pool.bit == v_pool.bit
+    rope_stride = 0
+    if cos is not None:
+        assert cos.dtype == torch.float16 and sin.dtype == torch.float16 and cos.shape == sin.shape
+        assert cos.shape[-1] == D and cos.stride(-1) == 1 and sin.stride(-1) == 1
+        if cos.dim() == 2 and cos.shape[0] > 1:
+            assert cos.shape[0] == bs and cos.stride(0) == sin.stride(0)
+            rope_stride = cos.stride(0)
+    L = lib()
+    Bq = bs * n_q
+    o = torch.empty((Bq, D), dtype=torch.float16, device=q_in.device) if out is None else out
+    ws = ops.workspace(q_in.device, L.mstf_decode_attention_window_workspace_bytes(k_pool.max_tokens, int(win_len), D, Bq,
+                                                                                   n_q // n_kv), ws)
+    ptrs = []
+    for p in (k_pool, v_pool):
+        ptrs += [p.bmp_store.data_ptr(), p.packed.data_ptr(), p.off_store.data_ptr(), p.scales_store.data_ptr(),
+                 p.zeros_store.data_ptr()]
+    bit = int(k_pool.bit)
+    check(L.mstf_decode_step_quant_pool(
+        torch.cuda.current_stream().cuda_stream, *ptrs, q_in.data_ptr(), q_in.stride(0), k_in.data_ptr(), k_in.stride(0),
+        v_in.data_ptr(), v_in.stride(0), bs, n_q, n_kv, cos.data_ptr() if cos is not None else None,
+        sin.data_ptr() if sin is not None else None, rope_stride, k_win.data_ptr(), v_win.data_ptr(), k_win.shape[1],
+        int(win_len), win_len_dev.data_ptr() if win_len_dev is not None else None,
+        overflow.data_ptr() if overflow is not None else None, o.data_ptr(), lse.data_ptr() if lse is not None else None,
+        k_pool.max_tokens, k_pool.tokens_dev.data_ptr(), k_pool.tile_capacity, D, bit, 32 // bit, int(dequant_mode),
+        ws.data_ptr(), ws.numel()), "mstf_decode_step_quant_pool")
+    return o
+
+
 # aliases the reference exports for its model code (pybind_quant.cpp:96-176)
 mustafar_quant_sparse_forward = mustafar_key_formulation_quant
 mustafar_quant_sparse_forward_meta = mustafar_key_formulation_quant_meta

@@ -379,13 +379,15 @@ def test_caches_sharing_a_window_counter_advance_together():
 
 @pytest.mark.parametrize("bs,n_kv,g,L0,steps,per_entry", [(2, 2, 4, 600, 200, False), (1, 1, 8, 300, 70, True),
                                                            (3, 2, 2, 1100, 40, False)])
-def test_two_launch_step_equals_the_append_and_attention_calls(bs, n_kv, g, L0, steps, per_entry):
-    """mstf_decode_step_pool_f16 (rotation, append and window attention inside the launch of the compressed tokens,
-    then the merge) against mstf_window_append_f16 + mstf_decode_attention_window_pool_f16 on a twin cache: the
+@pytest.mark.parametrize("bit", [0, 2, 4])
+def test_two_launch_step_equals_the_append_and_attention_calls(bs, n_kv, g, L0, steps, per_entry, bit):
+    """mstf_decode_step_pool_f16 / mstf_decode_step_quant_pool (bit > 0) (rotation, append and window attention inside
+    the launch of the compressed tokens, then the merge) against mstf_window_append_f16 +
+    mstf_decode_attention_window_pool_f16 / mstf_decode_attention_window_quant_pool on a twin cache: the
     attention output of every step and the window buffers are identical bit for bit, across a chunk append, with an
     empty compressed part at the start (second case), partial and full window blocks, and the count overrunning the
     window buffer flagged the same way."""
-    from mustafar_amd.cache import SparseKVCache
+    from mustafar_amd.cache import QuantSparseKVCache, SparseKVCache
     dev = torch.device("cuda:0")
     D, res = 128, 256
     n_q = n_kv * g
@@ -395,7 +397,10 @@ def test_two_launch_step_equals_the_append_and_attention_calls(bs, n_kv, g, L0, 
     Vt = torch.from_numpy(V).to(dev).view(bs, n_kv, L0, D)
     caches = []
     for step_launch in (True, False):
-        c = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, window_kernel=True, max_tokens=1536)
+        if bit:
+            c = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=bit, fused=True, window_kernel=True, max_tokens=1536)
+        else:
+            c = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, window_kernel=True, max_tokens=1536)
         c.step_launch = step_launch
         c.prefill(Kt, Vt)
         caches.append(c)
