@@ -382,8 +382,11 @@ struct ProjArgs {
     RowsView rot;
     int rows;
 };
+#ifndef MSTF_COMPRESS_PARK
+#define MSTF_COMPRESS_PARK 1
+#endif
 template <bool IS_VALUE, int W, int SRC>
-__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void compress_onepass_kernel(
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu((MSTF_COMPRESS_PARK && SRC != kSrcRope) ? 4 : 2))) void compress_onepass_kernel(
     const _Float16* __restrict__ x, ProjArgs proj, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
     uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
     const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
@@ -413,13 +416,25 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
             unit_fetch(proj.view.head(b), (int64_t)tb * 64, lane, raw, proj.view.st);
         else
             unit_fetch_rotated(proj.view, proj.rope, proj.rot, b, tb, proj.rows, lane, raw);
-        unit_rows_from(raw, buf, lane, r);
+        if (MSTF_COMPRESS_PARK)
+            unit_rows_parked(raw, buf, lane, r);  // r[32 .. 64) stays in the staging buffer during the search
+        else
+            unit_rows_from(raw, buf, lane, r);
     }
     uint32_t kept[4];
-    if (kth > 0)
+    if (MSTF_COMPRESS_PARK) {
+        if (kth > 0) {
+            select_kth_planes_parked<true>(r, buf, lane, kth, kept);
+        } else {
+            parked_rows_take(buf, lane, r);
+            kept_nonzero(r, kept);
+        }
+        __builtin_amdgcn_wave_barrier();  // the buffer becomes the image of the output next
+    } else if (kth > 0) {
         select_kth_planes<true>(r, kth, kept);  // the sign bits become planes the search never looks at
-    else
+    } else {
         kept_nonzero(r, kept);
+    }
     uint64_t bmA, bmB;  // tiles tb*128 + lane and tb*128 + 64 + lane
     if (IS_VALUE) {
         bmA = spread_bitmap(kept[0], kept[1]);

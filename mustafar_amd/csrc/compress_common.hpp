@@ -192,14 +192,10 @@ __device__ __forceinline__ void bit_transpose32(uint32_t (&r)[N], int first)
 // four 32-bit candidate masks: with c0 = #candidates whose bit is 0, the bit of the answer is 1 iff k > c0.  About
 // 830 vector instructions against 1900 for a count per candidate value over the packed row.
 // kept[w] (if wanted) = elements >= max(answer, 1): channel c sits in word 2*(c/64) + (c&1), bit (c%64)/2.
+// The search of select_kth_planes on the bit planes p (see there).
 template <bool WANT_KEPT>
-__device__ __forceinline__ uint32_t select_kth_planes(const uint32_t (&mag)[64], int kth, uint32_t (&kept)[4])
+__device__ __forceinline__ uint32_t search_planes(const uint32_t (&p)[64], int kth, uint32_t (&kept)[4])
 {
-    uint32_t p[64];
-#pragma unroll
-    for (int j = 0; j < 64; j++) p[j] = mag[j];
-    bit_transpose32(p, 0);
-    bit_transpose32(p, 32);
     uint32_t alive[4] = {~0u, ~0u, ~0u, ~0u}, greater[4] = {0u, 0u, 0u, 0u};
     uint32_t k = (uint32_t)kth, thr = 0u;
 #pragma unroll
@@ -225,6 +221,63 @@ __device__ __forceinline__ uint32_t select_kth_planes(const uint32_t (&mag)[64],
 #pragma unroll
         for (int w = 0; w < 4; w++) kept[w] = greater[w] | (thr ? alive[w] : 0u);
     }
+    return thr;
+}
+template <bool WANT_KEPT>
+__device__ __forceinline__ uint32_t select_kth_planes(const uint32_t (&mag)[64], int kth, uint32_t (&kept)[4])
+{
+    uint32_t p[64];
+#pragma unroll
+    for (int j = 0; j < 64; j++) p[j] = mag[j];
+    bit_transpose32(p, 0);
+    bit_transpose32(p, 32);
+    return search_planes<WANT_KEPT>(p, kth, kept);
+}
+
+// The same for a wavefront that keeps only the first half of its rows in registers while it searches: after
+// unit_rows_parked the second half of every row is still in the slab; it is read once for its bit planes and once
+// more, into r[32 .. 64), when the search is over and the planes are dead - 32 registers fewer at the peak, which is
+// what lets a kernel that holds a whole unit in registers run four wavefronts per SIMD instead of three.
+__device__ __forceinline__ void unit_rows_parked(const UnitRaw& raw, uint32_t* slab, int lane, uint32_t (&r)[64])
+{
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = j * 64 + lane;
+            uint32_t* d = slab + (e >> 3) * kHalfRowDw + (e & 7) * 4;
+            d[0] = raw.v[h][j].x;
+            d[1] = raw.v[h][j].y;
+            d[2] = raw.v[h][j].z;
+            d[3] = raw.v[h][j].w;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (h == 0) {
+            row_of_lane(slab, lane, r, 0);
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+}
+__device__ __forceinline__ void parked_rows_take(const uint32_t* slab, int lane, uint32_t (&r)[64])
+{
+    // (the compiler must neither reuse the values of an earlier read of the slab nor move this one up)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    row_of_lane(slab, lane, r, 32);
+}
+template <bool WANT_KEPT>
+__device__ __forceinline__ uint32_t select_kth_planes_parked(uint32_t (&r)[64], const uint32_t* slab, int lane, int kth,
+                                                             uint32_t (&kept)[4])
+{
+    uint32_t p[64];
+#pragma unroll
+    for (int j = 0; j < 32; j++) p[j] = r[j];
+    bit_transpose32(p, 0);
+    row_of_lane(slab, lane, p, 32);
+    bit_transpose32(p, 32);
+    const uint32_t thr = search_planes<WANT_KEPT>(p, kth, kept);
+    asm volatile("" : "+v"(kept[0]), "+v"(kept[1]), "+v"(kept[2]), "+v"(kept[3]));  // the search ends here
+    parked_rows_take(slab, lane, r);
     return thr;
 }
 __device__ __forceinline__ uint32_t select_kth(const uint32_t (&mag)[64], int kth)
