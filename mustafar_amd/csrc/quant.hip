@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void quant_finalize_kernel(uint32_t* __restric
 // final global word offsets.  grid = units / W workgroups of W wavefronts, W divides M / 64.
 // total_words reads as all ones when a wait ran out of its polls.
 template <bool IS_VALUE, bool G32, int W>
-__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) void quant_onepass_kernel(
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(4))) void quant_onepass_kernel(
     const _Float16* __restrict__ x, int M, int kth, int bit, uint64_t* __restrict__ bmp, uint32_t* __restrict__ counts,
     uint32_t* __restrict__ units, uint32_t* __restrict__ tile_off, _Float16* __restrict__ scales,
     _Float16* __restrict__ zeros, uint32_t* __restrict__ packed, uint64_t capacity_words,
@@ -185,18 +185,20 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
     {
         UnitRaw raw;
         unit_fetch(x + (size_t)b * M * kD, (int64_t)tb * 64, lane, raw);
-        unit_rows_from(raw, slab, lane, r);
+        unit_rows_parked(raw, slab, lane, r);  // r[32 .. 64) stays in the slab during the search
     }
     uint64_t bm[2];
     uint32_t thr = 1u;
     {
         uint32_t kept[4];
         if (kth > 0) {
-            thr = select_kth_planes<true>(r, kth, kept);  // the sign bits become planes the search never looks at
+            thr = select_kth_planes_parked<true>(r, slab, lane, kth, kept);  // the sign bits become planes the search never looks at
             if (thr == 0u) thr = 1u;
         } else {
+            parked_rows_take(slab, lane, r);
             kept_nonzero(r, kept);
         }
+        __builtin_amdgcn_wave_barrier();
         if (IS_VALUE) {
             bm[0] = spread_bitmap(kept[0], kept[1]);
             bm[1] = spread_bitmap(kept[2], kept[3]);
