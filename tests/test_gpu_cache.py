@@ -445,3 +445,62 @@ def test_two_launch_step_flags_a_count_past_the_window_buffer():
     torch.cuda.synchronize()
     assert int(ovf) == 1 and torch.isfinite(out).all()
     assert torch.equal(c._kbuf.view(torch.int16), kb.view(torch.int16)) and torch.equal(c._vbuf.view(torch.int16), vb.view(torch.int16))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_two_launch_step_against_the_oracle_on_random_shapes(seed):
+    """The two-launch decode step on drawn shapes (batch, KV heads, query heads per KV head, prompt length, 2-bit or
+    fp16 cache, per-entry or shared positions) against the CPU oracle: rotation of the new query / key heads by
+    oracle.rope_rows, dense masked attention over [pruned compressed tokens | dense window with the new row], 2e-3
+    (1e-2 for the quantised cache: the oracle attends over the dequantised codes there)."""
+    from mustafar_amd.cache import QuantSparseKVCache, SparseKVCache
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(7700 + seed)
+    D, res = 128, 256
+    bs = int(rng.integers(1, 4))
+    n_kv = int(rng.integers(1, 3))
+    g = int(rng.choice([1, 2, 4, 5, 8]))
+    L0 = int(rng.integers(260, 900))
+    quant = seed % 3 == 2
+    per_entry = bool(seed % 2)
+    n_q, Bkv = n_kv * g, bs * n_kv
+    K, V = orc.make_kv(500 + seed, Bkv, L0, D)
+    if quant:
+        c = QuantSparseKVCache(g, D, 0.7, 0.7, res, bit=2, fused=True, window_kernel=True, max_tokens=1280)
+    else:
+        c = SparseKVCache(g, D, 0.7, 0.7, res, fused=True, window_kernel=True, max_tokens=1280)
+    assert c.step_launch
+    c.prefill(torch.from_numpy(K).to(dev).view(bs, n_kv, L0, D), torch.from_numpy(V).to(dev).view(bs, n_kv, L0, D))
+    K_all, V_all = K.copy(), V.copy()                      # [Bkv, tokens, D]; the prompt's keys count as rotated
+    steps = 3 if L0 % 256 < 250 else 8
+    for t in range(steps):
+        proj = rng.standard_normal((bs, (n_q + 2 * n_kv) * D)).astype(np.float16)
+        pos = np.arange(bs) * 5 + L0 + t if per_entry else np.full(bs, L0 + t)
+        cos, sin = orc.rope_tables(pos)                    # [bs, D]
+        pt = torch.from_numpy(proj).to(dev)
+        ct = torch.from_numpy(cos if per_entry else cos[0]).to(dev)
+        st = torch.from_numpy(sin if per_entry else sin[0]).to(dev)
+        out = c.decode_device_proj(pt[:, : n_q * D], pt[:, n_q * D: (n_q + n_kv) * D], pt[:, (n_q + n_kv) * D:], ct, st)
+        q = proj[:, : n_q * D].reshape(bs, n_q, D)
+        k = proj[:, n_q * D: (n_q + n_kv) * D].reshape(bs, n_kv, D)
+        v = proj[:, (n_q + n_kv) * D:].reshape(bs, n_kv, D)
+        qr = orc.rope_rows(q, cos[:, None, :], sin[:, None, :]).reshape(bs * n_q, D)
+        kr = orc.rope_rows(k, cos[:, None, :], sin[:, None, :]).reshape(Bkv, 1, D)
+        K_all = np.concatenate([K_all, kr], 1)
+        V_all = np.concatenate([V_all, v.reshape(Bkv, 1, D)], 1)
+        Lc = c.compressed_length
+        Kp, Vp = K_all.copy(), V_all.copy()
+        if Lc:
+            Kp[:, :Lc] = orc.prune_rows(K_all[:, :Lc], c.kth_k)
+            Vp[:, :Lc] = orc.prune_rows(V_all[:, :Lc], c.kth_v)
+            if quant:
+                for x, is_value in ((Kp, 0), (Vp, 1)):
+                    r = orc.compress_quant(np.ascontiguousarray(x[:, :Lc]), is_value, 2)
+                    x[:, :Lc] = np.stack([orc.decode_quant(r[0], r[2], r[1], r[5], r[6], b, Lc, D, is_value, 2, 0)
+                                          for b in range(Bkv)])
+        _, _, o_ref = orc.dense_masked_attention(qr, Kp, Vp, g)
+        got = out.reshape(bs * n_q, D).float().cpu().numpy().astype(np.float64)
+        scale = max(np.abs(o_ref.astype(np.float64)).max(), 1e-30)
+        assert np.abs(got - o_ref).max() < (1e-2 if quant else 2e-3) * scale, (seed, t)
+        c.advance()
+    assert int(c._wovf) == 0
