@@ -105,18 +105,24 @@ def cpu_baseline(args, bs, nkv, groups, L, D, kth):
     }
 
 
+RING_ROUNDS = 4   # passes over the rotating caches captured into one graph
+
+
 def ring_time_us(torch, fn, n_slots, reps):
-    """GPU time of one fn(i): fn(0) .. fn(n_slots - 1) are captured back to back into one HIP graph (slot i works on
-    rotating cache i, so its reads are cold), the graph is replayed `reps` times between two HIP events."""
+    """GPU time of one fn(i): RING_ROUNDS passes of fn(0) .. fn(n_slots - 1) are captured back to back into one HIP
+    graph (slot i works on rotating cache i, so its reads are cold), the graph is replayed `reps` times between two HIP
+    events.  A replay starts with a bubble of a few microseconds on the GPU; with a few dozen launches per graph - as
+    a decode iteration of a model holds the launches of all its layers - it no longer weighs on the per-launch figure."""
     for i in range(n_slots):
         fn(i)   # warm-up outside the capture (module load, workspace growth)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
-        for i in range(n_slots):
-            fn(i)
+        for _ in range(RING_ROUNDS):
+            for i in range(n_slots):
+                fn(i)
     g.replay()
-    return event_time_us(torch, g.replay, max(1, reps)) / n_slots
+    return event_time_us(torch, g.replay, max(1, -(-reps // RING_ROUNDS))) / (n_slots * RING_ROUNDS)
 
 
 def read_calibration(torch):
@@ -416,9 +422,9 @@ def main():
             ops.decode_attention(ck, cv, q2, groups, out=o2, ws=ws)
 
     # The launches are captured once and replayed, so that the timed region measures the GPU work of a step
-    # rather than the Python call overhead of its launches: one graph holds one step on each of the rotating
-    # caches back to back (as a decode iteration holds the attention of consecutive layers in one graph), and
-    # one single-step graph per cache serves the remainder when K is not a multiple of the cache count.
+    # rather than the Python call overhead of its launches: one graph holds RING_ROUNDS passes of one step on each
+    # of the rotating caches back to back (as a decode iteration holds the attention of consecutive layers in one
+    # graph), and one single-step graph per cache serves the remainder when K is not a multiple of its length.
     graphs = ring = None
     if not args.no_graph:
         try:
@@ -433,8 +439,9 @@ def main():
                 graphs.append(g)
             ring = torch.cuda.CUDAGraph()
             with torch.cuda.graph(ring):
-                for i in range(args.caches):
-                    launch(i)
+                for _ in range(RING_ROUNDS):
+                    for i in range(args.caches):
+                        launch(i)
         except Exception as e:  # pragma: no cover - reported in the JSON line
             print("graph capture failed (%s); launching from Python" % e, file=sys.stderr)
             graphs = ring = None
@@ -448,10 +455,10 @@ def main():
             return
         while k > 0:
             i = it[0] % args.caches
-            if i == 0 and k >= args.caches:
+            if i == 0 and k >= args.caches * RING_ROUNDS:
                 ring.replay()
-                it[0] += args.caches
-                k -= args.caches
+                it[0] += args.caches * RING_ROUNDS
+                k -= args.caches * RING_ROUNDS
             else:
                 graphs[i].replay()
                 it[0] += 1
@@ -587,7 +594,7 @@ def main():
                         "head_dim 128, %d cached tokens, per-token magnitude pruning %.0f%% on K and V, one new token; "
                         "%s; %d caches rotated (cold HBM reads); %s"
                         % (bs, L, args.sparsity * 100, step_desc, args.caches,
-                           "steps replayed from HIP graphs (%d consecutive steps per graph)" % args.caches if graphs is not None else "steps launched from Python"),
+                           "steps replayed from HIP graphs (%d consecutive steps per graph)" % (args.caches * RING_ROUNDS) if graphs is not None else "steps launched from Python"),
             "compressed_bytes_per_token_per_kv_head": {"key": round(kbytes / Bkv / L, 2),
                                                        "value": round(vbytes / Bkv / L, 2)},
         },
