@@ -97,11 +97,10 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     if (active) {
         const uint64_t* bmK = k_bmp + (size_t)kv * T + (size_t)tb * D;
         const uint32_t* ixK = k_idx + (size_t)kv * (T + 1) + (size_t)tb * D;
-        const char* nzK = k_nz + (size_t)k_nz_off[kv] * 16u;
         const uint64_t* bmV = v_bmp + (size_t)kv * T + (size_t)tb * D;
         const uint32_t* ixV = v_idx + (size_t)kv * (T + 1) + (size_t)tb * D;
-        const char* nzV = v_nz + (size_t)v_nz_off[kv] * 16u;
         if (lane < 4) reinterpret_cast<uint32_t*>(my + 2 * kSubBytes)[lane] = 0u;
+        const char *nzK = nullptr, *nzV = nullptr;  // the head's value streams (set below, from the boundary load)
 
         // sub-chunk n of a block's walk: n < kKeySubs -> key tiles n*32.., else value tiles (n-kKeySubs)*32..
         auto bm_of = [&](int n) { return n < kKeySubs ? bmK + n * kSubTiles : bmV + (n - kKeySubs) * kSubTiles; };
@@ -115,7 +114,15 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
         // scalar batch is live)
         const bool bnd_v = lane >= 16 && lane <= 16 + kValSubs;
         const int bnd_i = bnd_v ? (lane - 16) * kSubTiles : (lane <= kKeySubs ? lane * kSubTiles : 0);
-        auto boundaries = [&](const uint32_t* ik, const uint32_t* iv) { return (bnd_v ? iv : ik)[bnd_i]; };
+        // Lanes 62 and 63 fetch the head's entries of v_nz_off and k_nz_off in the same load: fetched on their own
+        // they are a round trip of their own in front of this one (the compiler waits for them where the value
+        // streams' addresses are formed, which is before it issues this load).
+        const uint32_t* const off_p = lane == 63 ? k_nz_off + kv : v_nz_off + kv;
+        auto boundaries = [&](const uint32_t* ik, const uint32_t* iv) {
+            const uint32_t* p = (bnd_v ? iv : ik) + bnd_i;
+            p = lane >= 62 ? off_p : p;
+            return *p;
+        };
         uint32_t bnd = boundaries(ixK, ixV);
         uint32_t bnd_next = bnd;  // MULTI: boundaries of the coming block
         const uint32_t lane16 = (uint32_t)lane * 16u;
@@ -148,6 +155,8 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
                 if (o < qbytes) dma16(qsrc + o, ql + i * 1024);
             }
         }
+        nzK = k_nz + (size_t)(uint32_t)__builtin_amdgcn_readlane(bnd, 63) * 16u;
+        nzV = v_nz + (size_t)(uint32_t)__builtin_amdgcn_readlane(bnd, 62) * 16u;
         Touch touch = issue(0);
 
         const uint32_t qrow = lds_addr(ql) + (uint32_t)j * D * 2u;
