@@ -60,18 +60,55 @@ int window_launch(hipStream_t st, const mstf_half* k_win, const mstf_half* v_win
                   int split0);
 static inline int window_blocks(int win_len) { return (win_len + 63) / 64; }
 
+// Reductions over the sixteen lanes 4b+j (b = 0..15) that hold column j, without LDS round trips: inside a row of
+// sixteen lanes by two rotations (DPP row_ror 4 and 8, folded into the combining instruction), across the four rows by
+// v_permlane16_swap / v_permlane32_swap (a and b copies of v: afterwards a holds the even rows / the lower half twice,
+// b the odd rows / the upper half twice).  Every lane ends up with the maximum; of the sum, lanes 4b+j of one column may
+// differ in the last bit (the rotations add in a different order per lane), and lanes 0..3 are the ones that are used.
+typedef uint32_t u32x2v_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dpp_row_ror(float v, int n4)
+{
+    const int x = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, n4 == 4 ? __builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false)
+                                               : __builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false));
+}
+__device__ __forceinline__ void rows_swapped(float v, bool halves, float& a, float& b)
+{
+    const uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const u32x2v_t r = halves ? __builtin_amdgcn_permlane32_swap(x, x, false, false)
+                              : __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];  // (a bit cast applied to a vector element directly reads element 0)
+    a = __builtin_bit_cast(float, r0);
+    b = __builtin_bit_cast(float, r1);
+}
 __device__ __forceinline__ float wave_max_same_column(float v)
 {
-    // lanes 4b+j for b = 0..15 hold column j: combine over b with xor shuffles of 4, 8, 16, 32
-#pragma unroll
-    for (int o = 4; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    float a, b;
+    v = fmaxf(v, dpp_row_ror(v, 4));
+    v = fmaxf(v, dpp_row_ror(v, 8));
+    rows_swapped(v, false, a, b);
+    v = fmaxf(a, b);
+    rows_swapped(v, true, a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float wave_sum_same_column(float v)
 {
-#pragma unroll
-    for (int o = 4; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    float a, b;
+    v += dpp_row_ror(v, 4);
+    v += dpp_row_ror(v, 8);
+    rows_swapped(v, false, a, b);
+    v = a + b;
+    rows_swapped(v, true, a, b);
+    return a + b;
+}
+
+// x / c for |x| up to the fp16 range and c = sqrt(head_dim), r = 1 / c rounded: the quotient estimate and one
+// correction by the exact remainder - the correctly rounded quotient, as the full division sequence gives it, without
+// that sequence's scaling and special cases (a dozen instructions per value), which these operands never need.
+__device__ __forceinline__ float div_small(float x, float c, float r)
+{
+    const float q = x * r;
+    return __builtin_fmaf(__builtin_fmaf(-c, q, x), r, q);
 }
 
 // Softmax statistics of one 64-token block from its scores; lane 4b+j holds tokens 4b..4b+3 of head 4m+j in acc_k[m].
@@ -83,6 +120,7 @@ __device__ __forceinline__ void block_softmax(const f4_t (&acc_k)[NM], float sqr
                                               float (&m_run)[NM], float (&l_run)[NM])
 {
     const int j = lane & 3;
+    const float rcp_d = 1.0f / sqrt_d;
 #pragma unroll
     for (int m = 0; m < NM; m++) {
         float w[4];
@@ -90,7 +128,7 @@ __device__ __forceinline__ void block_softmax(const f4_t (&acc_k)[NM], float sqr
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const _Float16 s16 = (_Float16)acc_k[m][r];
-            w[r] = ((lane & ~3) + r < nt) ? (float)(_Float16)((float)s16 / sqrt_d) : -INFINITY;
+            w[r] = ((lane & ~3) + r < nt) ? (float)(_Float16)div_small((float)s16, sqrt_d, rcp_d) : -INFINITY;
             mx = fmaxf(mx, w[r]);
         }
         mx = wave_max_same_column(mx);

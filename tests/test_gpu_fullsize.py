@@ -286,7 +286,7 @@ def test_decode_attention_many_blocks(bkv, blocks, groups):
     Vp = torch_prune(V, KTH)
     o_exact = torch.einsum("bgl,bld->bgd", torch.softmax(w, -1).view(bkv, groups, length), Vp.float()).half().view(-1, D)
     assert rel_err(o, o_exact) < 2e-3
-    tol_ref = 2e-3 if length <= 32768 else 4e-3
+    tol_ref = 2e-3 if length <= 32768 else 5e-3   # (the reference formula's own loss at 131072 tokens: 3.9e-3 - 4.2e-3 here)
     assert rel_err(o, o_ref) < tol_ref
     m_ref = w.amax(-1)
     assert float((lse[:, 0] - m_ref).abs().max()) <= 2e-2 * max(float(m_ref.abs().max()), 1.0)

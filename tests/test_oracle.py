@@ -371,3 +371,20 @@ def test_group32_reduces_to_the_per_tile_quantiser_on_half_tiles(bit, is_value):
     e32 = np.abs(d32.astype(np.float32) - x.astype(np.float32))
     e64 = np.abs(d64.astype(np.float32) - x.astype(np.float32))
     assert e32.mean() <= e64.mean()
+
+
+def test_quotient_by_one_correction_step_equals_the_division_for_every_half_score():
+    """The fused kernels scale a score by x / sqrt(d) as q = x * r, q + r * (x - c * q) with r = 1 / c (div_small in
+    csrc/fused_common.hpp; the remainder by a fused multiply-add, emulated here in double precision, which holds the
+    24 x 24-bit product exactly).  For every finite fp16 score and the head dimensions in use the result is the
+    correctly rounded fp32 quotient, so the fp16 value the softmax sees is the one the reference's division gives
+    (-0.0 comes out as +0.0: the same score)."""
+    x = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    x = x[np.isfinite(x)]
+    for d in (64, 128, 256):
+        c = np.float32(np.sqrt(np.float32(d)))
+        r = np.float32(1) / c
+        q = (x * r).astype(np.float32)
+        e = (np.float64(x) - np.float64(c) * np.float64(q)).astype(np.float32)
+        q2 = (np.float64(q) + np.float64(e) * np.float64(r)).astype(np.float32)
+        assert np.array_equal(q2, (x / c).astype(np.float32))
