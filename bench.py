@@ -212,6 +212,15 @@ def compress_record(torch, ops, dev, gen, bs, L, sparsity, reps):
         out[name] = {"us": round(us, 1), "read_bytes": int(read), "written_bytes": int(written),
                      "gbs": round((read + written) / us / 1e3, 1),
                      "frac_of_peak": round((read + written) / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # keys and values of the context in one call (one clearing launch, one kernel over both sides)
+    keep = [None] * slots
+
+    def run_kv(i):
+        keep[i] = ops.compress_kv(Ks[i % copies], Vs[i % copies], kth, kth, capacity_halfs=Ks[0].numel(), ws=ws)
+    us = ring_time_us(torch, run_kv, slots, reps)
+    moved = out["key"]["read_bytes"] + out["key"]["written_bytes"] + out["value"]["read_bytes"] + out["value"]["written_bytes"]
+    out["key_and_value_one_call"] = {"us": round(us, 1), "us_per_side": round(us / 2, 1), "gbs": round(moved / us / 1e3, 1),
+                                     "frac_of_peak": round(moved / us / 1e3 / HBM_PEAK_GBS, 4)}
     return out
 
 
@@ -603,9 +612,11 @@ def main():
         # GPU time of each kernel, replayed from HIP graphs on the rotating caches (no Python launch gaps inside)
         "stages_us": {"fused_decode_attention": round(fused_us, 2), "fused_merge": round(merge_us, 2),
                       "key_spmv": round(key_us, 2), "scale_softmax": round(sm_us, 2), "value_spmv": round(val_us, 2),
-                      "prune_compress_key_ctx": comp["key"]["us"], "prune_compress_value_ctx": comp["value"]["us"]},
+                      "prune_compress_key_ctx": comp["key"]["us"], "prune_compress_value_ctx": comp["value"]["us"],
+                      "prune_compress_key_and_value_ctx_one_call": comp["key_and_value_one_call"]["us"]},
         # BASELINE configs[1] asks for the compression of the cached context timed with the step: their sum
-        "configs1_total_us": round(comp["key"]["us"] + comp["value"]["us"] + wall_us, 2),
+        "configs1_total_us": round(comp["key_and_value_one_call"]["us"] + wall_us, 2),
+        "configs1_total_us_separate_calls": round(comp["key"]["us"] + comp["value"]["us"] + wall_us, 2),
         "compress": comp,
         "quant_stages_us": quant_here,
         "dense_fp16_attention_us": dense_us,

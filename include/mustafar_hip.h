@@ -113,6 +113,26 @@ int mstf_append_value_f16(void* stream, const mstf_half* x, int B, int M, int N,
                           const uint32_t* dst_off, const uint32_t* dst_limit, mstf_half* nz, uint32_t* overflow,
                           void* workspace, size_t workspace_bytes);
 
+/* Keys and values of the same tokens in one launch instead of two (the reference converts K and V of a context or of a
+ * chunk back to back, models/llama_mustafar_kernel.py:540-557 and :461-511): exactly what mstf_compress_key_f16 followed
+ * by mstf_compress_value_f16 (both with a value buffer), or mstf_append_key_f16 followed by mstf_append_value_f16,
+ * write - the outputs are identical bit for bit - behind one clearing launch, with the workgroups of the two sides in
+ * one grid.  A launch with twice the workgroups runs less in lockstep (the loads of the values overlap the arithmetic
+ * of the keys): 49 us against 28 + 26 us at 64 heads x 4096 tokens, 91 against 54 + 52 us at 128 heads.  Both value
+ * buffers are required (no sizing-only form); the append form shares one sticky flag word between the sides.
+ * Workspace: mstf_compress_kv_workspace_bytes(B, M, N), 256-byte aligned. */
+size_t mstf_compress_kv_workspace_bytes(int B, int M, int N);
+int mstf_compress_kv_f16(void* stream, const mstf_half* k, const mstf_half* v, int B, int M, int N, int kth_k, int kth_v,
+                         uint64_t* k_bmp, uint32_t* k_idx, uint32_t* k_nz_off, uint64_t* k_total_halfs, mstf_half* k_nz,
+                         uint64_t k_capacity_halfs, uint64_t* v_bmp, uint32_t* v_idx, uint32_t* v_nz_off,
+                         uint64_t* v_total_halfs, mstf_half* v_nz, uint64_t v_capacity_halfs, void* workspace,
+                         size_t workspace_bytes);
+int mstf_append_kv_f16(void* stream, const mstf_half* k, const mstf_half* v, int B, int M, int N, int kth_k, int kth_v,
+                       uint64_t* k_bmp, uint32_t* k_idx, const uint32_t* k_dst_off, const uint32_t* k_dst_limit,
+                       mstf_half* k_nz, uint64_t* v_bmp, uint32_t* v_idx, const uint32_t* v_dst_off,
+                       const uint32_t* v_dst_limit, mstf_half* v_nz, uint32_t* overflow, void* workspace,
+                       size_t workspace_bytes);
+
 /* ------------------------------------------------------------------ compression from the projection output
  * The prefill of the reference turns the projection outputs [batch, tokens, heads * 128] into [batch, heads,
  * tokens, 128] views, rotates the keys (apply_rotary_pos_emb of transformers 4.43.1, called at

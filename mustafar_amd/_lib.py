@@ -44,6 +44,11 @@ SIGNATURES = {
     "mstf_scatter_value_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _u64]),
     "mstf_append_key_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "mstf_append_value_f16": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "mstf_compress_kv_workspace_bytes": (_sz, [_i, _i, _i]),
+    "mstf_compress_kv_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp, _vp, _vp, _vp,
+                                  _u64, _vp, _sz]),
+    "mstf_append_kv_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                _vp, _sz]),
     "mstf_compress_proj_f16": (_i, [_vp, _ps, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _sz]),
     "mstf_append_proj_f16": (_i, [_vp, _ps, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "mstf_key_spmv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),

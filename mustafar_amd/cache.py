@@ -234,6 +234,42 @@ def packed_fraction_for(kth, head_dim, bit):
     return min(1.0, words / (tiles * 64 / cap))
 
 
+def append_pair(k_pool, v_pool, xk, xv, kth_k, kth_v, ws=None):
+    """k_pool.append(xk, kth_k) and v_pool.append(xv, kth_v) of the same tokens as one call (mstf_append_kv_f16: both
+    sides in one launch, identical results).  The sides share one flag word; should a slab overflow, the chunk is
+    taken back and appended again side by side, where each pool grows its own slabs."""
+    B, M, N = xk.shape
+    assert xv.shape == xk.shape and not k_pool.is_value and v_pool.is_value
+    for p in (k_pool, v_pool):
+        assert B == p.heads and N == p.head_dim and M % 64 == 0 and p.tokens + M <= p.max_tokens
+    xk, xv = xk.contiguous(), xv.contiguous()
+    L = lib()
+    Tc = M * N // 64
+    dev = xk.device
+    chunk = [(torch.empty((B, Tc), dtype=torch.int64, device=dev), torch.empty((B, Tc + 1), dtype=torch.int32, device=dev),
+              p.nz_off + p.idx_store[:, p.tiles] // 4) for p in (k_pool, v_pool)]
+    w = ops.workspace(dev, L.mstf_compress_kv_workspace_bytes(B, M, N), ws)
+    (kb, ki, kd), (vb, vi, vd) = chunk
+    check(L.mstf_append_kv_f16(torch.cuda.current_stream().cuda_stream, xk.data_ptr(), xv.data_ptr(), B, M, N, int(kth_k),
+                               int(kth_v), kb.data_ptr(), ki.data_ptr(), kd.data_ptr(), k_pool.limit.data_ptr(),
+                               k_pool.nz.data_ptr(), vb.data_ptr(), vi.data_ptr(), vd.data_ptr(), v_pool.limit.data_ptr(),
+                               v_pool.nz.data_ptr(), k_pool.overflow.data_ptr(), w.data_ptr(), w.numel()),
+          "mstf_append_kv_f16")
+    k_pool._publish(kb, ki, M)
+    v_pool._publish(vb, vi, M)
+    flag = int(k_pool.overflow.item())
+    if flag & 2:
+        raise RuntimeError("the compressor gave up waiting for an earlier workgroup; the appended chunk is incomplete "
+                           "and the pools are no longer usable")
+    if flag & 1:
+        k_pool.overflow.zero_()
+        for p in (k_pool, v_pool):
+            p.tokens -= M
+            p.tokens_dev -= M
+        k_pool.append(xk, kth_k, ws)
+        v_pool.append(xv, kth_v, ws)
+
+
 class QuantPool:
     """One side (keys or values) of a quantised cache that grows in place.
 
@@ -392,8 +428,8 @@ class SparseKVCache:
             if self.k_pool is None:
                 self._make_pools(bs * n_kv, D, K.device)
             ws = self._workspace(K.device)
-            self.k_pool.append(K.reshape(bs * n_kv, M, D), self.kth_k, ws)
-            self.v_pool.append(V.reshape(bs * n_kv, M, D), self.kth_v, ws)
+            append_pair(self.k_pool, self.v_pool, K.reshape(bs * n_kv, M, D), V.reshape(bs * n_kv, M, D), self.kth_k,
+                        self.kth_v, ws)
             self._pool_views()
             return
         ck, cv = self._compress(K, V)

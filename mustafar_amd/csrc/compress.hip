@@ -385,25 +385,34 @@ struct ProjArgs {
 #ifndef MSTF_COMPRESS_PARK
 #define MSTF_COMPRESS_PARK 1
 #endif
-template <bool IS_VALUE, int W, int SRC>
-__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu((MSTF_COMPRESS_PARK && SRC != kSrcRope) ? 4 : 2))) void compress_onepass_kernel(
-    const _Float16* __restrict__ x, ProjArgs proj, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
-    uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
-    const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
-    uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total, uint32_t spin_limit)
-{
+// The LDS of a workgroup of the one-pass kernels.
+template <int W>
+struct OnepassLds {
     // per wavefront: staging buffer of a half-slab, then image of half a unit's output (at most 64 tiles x 128 bytes)
-    __shared__ __attribute__((aligned(16))) uint32_t bufs[W][kHalfSlabDw];
-    __shared__ uint32_t wave_total[W];
-    __shared__ uint64_t bases[W][3];  // per wavefront: its part of the sum over the earlier heads, of the sum over
-                                      // the head's earlier workgroups, and whether its waits ended
-    static_assert(kHalfSlabDw * 4 >= 64 * 128, "the image fits the staging buffer");
+    uint32_t bufs[W][kHalfSlabDw] __attribute__((aligned(16)));
+    uint32_t wave_total[W];
+    uint64_t bases[W][3];  // per wavefront: its part of the sum over the earlier heads, of the sum over the head's
+                           // earlier workgroups, and whether its waits ended
+};
+static_assert(kHalfSlabDw * 4 >= 64 * 128, "the image fits the staging buffer");
+
+// The work of workgroup g of a one-pass launch over one side (keys or values).
+template <bool IS_VALUE, int W, int SRC>
+__device__ __forceinline__ void onepass_workgroup(
+    OnepassLds<W>& lds, int g, const _Float16* __restrict__ x, const ProjArgs& proj, int M, int kth,
+    uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx, uint32_t* __restrict__ nz_off,
+    uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off, const uint32_t* __restrict__ dst_limit,
+    uint32_t* __restrict__ overflow, char* __restrict__ nz, uint64_t nz_capacity_halfs, uint64_t* state, int units,
+    int groups_total, uint32_t spin_limit)
+{
+    auto& bufs = lds.bufs;
+    auto& wave_total = lds.wave_total;
+    auto& bases = lds.bases;
     const int lane = lane_id();
     const int wave = wave_id();
     const int nblk = M / 64;
     const size_t T = (size_t)M * kD / 64;
     uint64_t* gave_up = state + groups_total;
-    const int g = (int)blockIdx.x;
     const int u = g * W + wave;  // all W units are of one head and exist: W divides nblk
     const int b = u / nblk, tb = u - b * nblk;
     uint32_t* buf = bufs[wave];
@@ -509,6 +518,51 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu((MSTF_CO
     stream_image(img, totB * 4u, dst + (size_t)totA * 4u, lane);
 }
 
+template <bool IS_VALUE, int W, int SRC>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu((MSTF_COMPRESS_PARK && SRC != kSrcRope) ? 4 : 2))) void compress_onepass_kernel(
+    const _Float16* __restrict__ x, ProjArgs proj, int M, int kth, uint64_t* __restrict__ bmp, uint32_t* __restrict__ idx,
+    uint32_t* __restrict__ nz_off, uint64_t* __restrict__ total_halfs, const uint32_t* __restrict__ dst_off,
+    const uint32_t* __restrict__ dst_limit, uint32_t* __restrict__ overflow, char* __restrict__ nz,
+    uint64_t nz_capacity_halfs, uint64_t* state, int units, int groups_total, uint32_t spin_limit)
+{
+    __shared__ OnepassLds<W> lds;
+    onepass_workgroup<IS_VALUE, W, SRC>(lds, (int)blockIdx.x, x, proj, M, kth, bmp, idx, nz_off, total_halfs, dst_off,
+                                        dst_limit, overflow, nz, nz_capacity_halfs, state, units, groups_total, spin_limit);
+}
+
+// Keys and values of the same tokens in one launch: workgroups 0 .. groups_total-1 compress the keys, the next
+// groups_total the values, each side with its own status words and outputs.  One launch has twice the generations of
+// workgroups of a launch per side, which run less in lockstep (the loads of one generation overlap the arithmetic of
+// the one before), and one clearing launch in front instead of two.
+struct OnepassSide {
+    const _Float16* x;
+    int kth;
+    uint64_t* bmp;
+    uint32_t* idx;
+    uint32_t* nz_off;
+    uint64_t* total_halfs;
+    const uint32_t* dst_off;
+    const uint32_t* dst_limit;
+    char* nz;
+    uint64_t nz_capacity_halfs;
+    uint64_t* state;
+};
+template <int W>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(4))) void compress_onepass_kv_kernel(
+    OnepassSide k, OnepassSide v, int M, uint32_t* __restrict__ overflow, int units, int groups_total, uint32_t spin_limit)
+{
+    __shared__ OnepassLds<W> lds;
+    const int g = (int)blockIdx.x;
+    if (g < groups_total)
+        onepass_workgroup<false, W, kSrcMatrix>(lds, g, k.x, ProjArgs{}, M, k.kth, k.bmp, k.idx, k.nz_off, k.total_halfs,
+                                                k.dst_off, k.dst_limit, overflow, k.nz, k.nz_capacity_halfs, k.state, units,
+                                                groups_total, spin_limit);
+    else
+        onepass_workgroup<true, W, kSrcMatrix>(lds, g - groups_total, v.x, ProjArgs{}, M, v.kth, v.bmp, v.idx, v.nz_off,
+                                               v.total_halfs, v.dst_off, v.dst_limit, overflow, v.nz, v.nz_capacity_halfs,
+                                               v.state, units, groups_total, spin_limit);
+}
+
 // ------------------------------------------------------------------------------- dense prune
 // y = x * (|x| >= kth-th smallest |x| of the row); 64 rows per wavefront.
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void prune_rows_kernel(const _Float16* __restrict__ x, _Float16* y, int64_t rows,
@@ -570,7 +624,7 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, const ProjArgs& pr
     const int words = groups + 1;
     const uint32_t spin_limit = onepass_spin_limit();
     hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
-                       dim3(256), 0, st, state, words, total_halfs);
+                       dim3(256), 0, st, state, words, total_halfs, static_cast<uint64_t*>(nullptr));
     int rc = check_launch();
     if (rc != MSTF_OK) return rc;
 #define MSTF_OP(WV)                                                                                                   \
@@ -584,6 +638,33 @@ static int launch_onepass(hipStream_t st, const _Float16* xh, const ProjArgs& pr
     else
         MSTF_OP(1);
 #undef MSTF_OP
+    return check_launch();
+}
+
+// Keys and values of the same tokens behind one clearing launch (status words of the keys, then of the values).
+static int launch_onepass_kv(hipStream_t st, OnepassSide k, OnepassSide v, int B, int M, uint32_t* overflow, void* ws)
+{
+    const int nblk = M / 64, units = B * nblk;
+    const int W = nblk % MSTF_ONEPASS_W == 0 ? MSTF_ONEPASS_W : (nblk % 2 == 0 ? 2 : 1);
+    const int groups = units / W;
+    const int words = groups + 1;
+    k.state = reinterpret_cast<uint64_t*>(ws);
+    v.state = k.state + words;
+    const uint32_t spin_limit = onepass_spin_limit();
+    hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((2 * words + 255) / 256 < 256 ? (2 * words + 255) / 256 : 256)),
+                       dim3(256), 0, st, k.state, 2 * words, k.total_halfs, v.total_halfs);
+    int rc = check_launch();
+    if (rc != MSTF_OK) return rc;
+#define MSTF_OPKV(WV)                                                                                            \
+    hipLaunchKernelGGL((compress_onepass_kv_kernel<WV>), dim3(2u * (unsigned)groups), dim3(64 * WV), 0, st, k, v, M, \
+                       overflow, units, groups, spin_limit)
+    if (W == MSTF_ONEPASS_W)
+        MSTF_OPKV(MSTF_ONEPASS_W);
+    else if (W == 2)
+        MSTF_OPKV(2);
+    else
+        MSTF_OPKV(1);
+#undef MSTF_OPKV
     return check_launch();
 }
 
@@ -826,4 +907,62 @@ extern "C" int mstf_append_proj_f16(void* stream, const mstf_proj_source* src, i
     if (!dst_off) return MSTF_EINVAL;
     return proj_impl(stream, src, is_value, M, N, kth, bmp, idx, nullptr, nullptr, dst_off, dst_limit, nz, 0, overflow,
                      workspace, workspace_bytes);
+}
+
+extern "C" size_t mstf_compress_kv_workspace_bytes(int B, int M, int N)
+{
+    if (B <= 0 || M <= 0 || N <= 0 || M % 64 != 0) return 0;
+    return 2 * compress_ws_bytes(B, M);
+}
+
+static int kv_side_check(const void* x, int B, int M, int N, int kth, const void* bmp, const void* idx, const void* nz)
+{
+    int rc = check_compress_args(x, B, M, N, kth);
+    if (rc != MSTF_OK) return rc;
+    if (!bmp || !idx || !nz) return MSTF_EINVAL;
+    if (!aligned_to(bmp, 8) || !aligned_to(idx, 4) || !aligned_to(nz, 16)) return MSTF_EALIGN;
+    return MSTF_OK;
+}
+
+extern "C" int mstf_compress_kv_f16(void* stream, const mstf_half* k, const mstf_half* v, int B, int M, int N, int kth_k,
+                                    int kth_v, uint64_t* k_bmp, uint32_t* k_idx, uint32_t* k_nz_off,
+                                    uint64_t* k_total_halfs, mstf_half* k_nz, uint64_t k_capacity_halfs, uint64_t* v_bmp,
+                                    uint32_t* v_idx, uint32_t* v_nz_off, uint64_t* v_total_halfs, mstf_half* v_nz,
+                                    uint64_t v_capacity_halfs, void* workspace, size_t workspace_bytes)
+{
+    int rc = kv_side_check(k, B, M, N, kth_k, k_bmp, k_idx, k_nz);
+    if (rc == MSTF_OK) rc = kv_side_check(v, B, M, N, kth_v, v_bmp, v_idx, v_nz);
+    if (rc != MSTF_OK) return rc;
+    if (!k_nz_off || !k_total_halfs || !v_nz_off || !v_total_halfs) return MSTF_EINVAL;
+    if (!aligned_to(k_nz_off, 4) || !aligned_to(v_nz_off, 4) || !aligned_to(k_total_halfs, 8) || !aligned_to(v_total_halfs, 8))
+        return MSTF_EALIGN;
+    if (!workspace || workspace_bytes < mstf_compress_kv_workspace_bytes(B, M, N)) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 256)) return MSTF_EALIGN;
+    OnepassSide ks = {reinterpret_cast<const _Float16*>(k), kth_k, k_bmp, k_idx, k_nz_off, k_total_halfs, nullptr, nullptr,
+                      reinterpret_cast<char*>(k_nz), k_capacity_halfs, nullptr};
+    OnepassSide vs = {reinterpret_cast<const _Float16*>(v), kth_v, v_bmp, v_idx, v_nz_off, v_total_halfs, nullptr, nullptr,
+                      reinterpret_cast<char*>(v_nz), v_capacity_halfs, nullptr};
+    return launch_onepass_kv(as_stream(stream), ks, vs, B, M, nullptr, workspace);
+}
+
+extern "C" int mstf_append_kv_f16(void* stream, const mstf_half* k, const mstf_half* v, int B, int M, int N, int kth_k,
+                                  int kth_v, uint64_t* k_bmp, uint32_t* k_idx, const uint32_t* k_dst_off,
+                                  const uint32_t* k_dst_limit, mstf_half* k_nz, uint64_t* v_bmp, uint32_t* v_idx,
+                                  const uint32_t* v_dst_off, const uint32_t* v_dst_limit, mstf_half* v_nz,
+                                  uint32_t* overflow, void* workspace, size_t workspace_bytes)
+{
+    int rc = kv_side_check(k, B, M, N, kth_k, k_bmp, k_idx, k_nz);
+    if (rc == MSTF_OK) rc = kv_side_check(v, B, M, N, kth_v, v_bmp, v_idx, v_nz);
+    if (rc != MSTF_OK) return rc;
+    if (!k_dst_off || !k_dst_limit || !v_dst_off || !v_dst_limit || !overflow) return MSTF_EINVAL;
+    if (!aligned_to(k_dst_off, 4) || !aligned_to(k_dst_limit, 4) || !aligned_to(v_dst_off, 4) || !aligned_to(v_dst_limit, 4) ||
+        !aligned_to(overflow, 4))
+        return MSTF_EALIGN;
+    if (!workspace || workspace_bytes < mstf_compress_kv_workspace_bytes(B, M, N)) return MSTF_EWORKSPACE;
+    if (!aligned_to(workspace, 256)) return MSTF_EALIGN;
+    OnepassSide ks = {reinterpret_cast<const _Float16*>(k), kth_k, k_bmp, k_idx, nullptr, nullptr, k_dst_off, k_dst_limit,
+                      reinterpret_cast<char*>(k_nz), ~0ull, nullptr};
+    OnepassSide vs = {reinterpret_cast<const _Float16*>(v), kth_v, v_bmp, v_idx, nullptr, nullptr, v_dst_off, v_dst_limit,
+                      reinterpret_cast<char*>(v_nz), ~0ull, nullptr};
+    return launch_onepass_kv(as_stream(stream), ks, vs, B, M, overflow, workspace);
 }

@@ -536,10 +536,14 @@ uint32_t onepass_spin_limit();
 // Clears the status words and the caller's total (nullable): the kernel raises the total with atomic maxima - the
 // last workgroup to the sum, a workgroup that gave up to all ones - so whichever comes last, a give-up stays visible.
 static __global__ __launch_bounds__(256) void onepass_init_kernel(uint64_t* __restrict__ state, int n,
-                                                                  uint64_t* __restrict__ total)
+                                                                  uint64_t* __restrict__ total,
+                                                                  uint64_t* __restrict__ total2 = nullptr)
 {
     for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < n; i += (int)(gridDim.x * 256)) state[i] = 0ull;
-    if (total && blockIdx.x == 0 && threadIdx.x == 0) *total = 0ull;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (total) *total = 0ull;
+        if (total2) *total2 = 0ull;
+    }
 }
 // The marker of a workgroup whose wait ran out, from one thread: the flag word behind the status words, all ones in
 // the caller's total (compress contract) or bit 1 of the caller's sticky flag (append contract).

@@ -446,7 +446,7 @@ static int compress_quant_impl(void* stream, const mstf_half* x, int B, int M, i
         const int words = groups + 1;
         const uint32_t spin_limit = onepass_spin_limit();
         hipLaunchKernelGGL(onepass_init_kernel, dim3((unsigned)((words + 255) / 256 < 256 ? (words + 255) / 256 : 256)),
-                           dim3(256), 0, st, state, words, total_words);
+                           dim3(256), 0, st, state, words, total_words, static_cast<uint64_t*>(nullptr));
         if ((rc = check_launch()) != MSTF_OK) return rc;
 #define MSTF_QOP(WV)                                                                                                  \
     hipLaunchKernelGGL((quant_onepass_kernel<IS_VALUE, G32, WV>), dim3((unsigned)groups), dim3(64 * WV), 0, st, xh, M, kth, \

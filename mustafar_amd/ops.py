@@ -144,6 +144,32 @@ def compress(x, is_value, kth=0, capacity_halfs=None, ws=None):
     return CompressedKV(bmp, idx, nz, nz_off, M, N, is_value, total)
 
 
+def compress_kv(k, v, kth_k=0, kth_v=0, capacity_halfs=None, ws=None):
+    """compress(k, False, kth_k) and compress(v, True, kth_v) of the same tokens in one launch (mstf_compress_kv_f16):
+    identical outputs, less time - a launch of both sides runs less in lockstep than two launches of one side each.
+    k, v: [B, M, N]; capacity_halfs (default: room for the dense rows) sizes both value buffers, the totals stay on
+    the device.  Returns (CompressedKV of the keys, CompressedKV of the values)."""
+    assert k.is_cuda and v.is_cuda and k.dtype == v.dtype == torch.float16 and k.dim() == 3 and k.shape == v.shape
+    k, v = k.contiguous(), v.contiguous()
+    B, M, N = k.shape
+    T = M * N // 64
+    dev = k.device
+    L = lib()
+    cap = B * M * N if capacity_halfs is None else int(capacity_halfs)
+    out = []
+    for _ in range(2):
+        out.append((torch.empty((B, T), dtype=torch.int64, device=dev), torch.empty((B, T + 1), dtype=torch.int32, device=dev),
+                    torch.empty((B,), dtype=torch.int32, device=dev), torch.empty((1,), dtype=torch.int64, device=dev),
+                    torch.empty((cap,), dtype=torch.float16, device=dev)))
+    ws = workspace(dev, L.mstf_compress_kv_workspace_bytes(B, M, N), ws)
+    (kb, ki, ko, kt, kn), (vb, vi, vo, vt, vn) = out
+    check(L.mstf_compress_kv_f16(_stream(), k.data_ptr(), v.data_ptr(), B, M, N, int(kth_k), int(kth_v), kb.data_ptr(),
+                                 ki.data_ptr(), ko.data_ptr(), kt.data_ptr(), kn.data_ptr(), cap, vb.data_ptr(),
+                                 vi.data_ptr(), vo.data_ptr(), vt.data_ptr(), vn.data_ptr(), cap, ws.data_ptr(),
+                                 ws.numel()), "mstf_compress_kv_f16")
+    return CompressedKV(kb, ki, kn, ko, M, N, False, kt), CompressedKV(vb, vi, vn, vo, M, N, True, vt)
+
+
 def proj_source(x, cos=None, sin=None, rot=None):
     """The mstf_proj_source of x [batch, rows, heads, 128] fp16 (any strides with contiguous channels, e.g. a view of
     a projection output [batch, rows, heads * 128]).  cos, sin: [rows, 128] or [batch, rows, 128] fp16 (keys only);

@@ -348,3 +348,24 @@ def test_quantised_producer_flags_a_wait_that_ran_out(no_polls):
             elif gs == 64:
                 n = cq.words_written(total)
                 assert np.array_equal(out[2][:n].cpu().numpy().view(np.uint32), ref[2].view(np.uint32))
+
+
+@pytest.mark.parametrize("B,M,kth_k,kth_v", [(3, 256, 89, 89), (2, 128, 38, 115), (5, 64, 0, 64), (1, 1024, 128, 1),
+                                              (16, 512, 89, 89)])
+def test_keys_and_values_in_one_launch_equal_the_two_calls(B, M, kth_k, kth_v):
+    """mstf_compress_kv_f16 against mstf_compress_key_f16 + mstf_compress_value_f16 (one-pass form): bitmaps, offsets,
+    nz_off, totals and packed values bit for bit, for 4, 2 and 1 units per workgroup, kth = 0 (input already pruned),
+    1 and 128."""
+    from mustafar_amd import ops
+    D = 128
+    K, V = orc.make_kv(77 + B * M, B, M, D)
+    if kth_k == 0:
+        K = orc.prune_rows(K, 89)
+    Kt, Vt = torch.from_numpy(K).to("cuda:0"), torch.from_numpy(V).to("cuda:0")
+    ck, cv = ops.compress_kv(Kt, Vt, kth_k, kth_v)
+    for got, x, is_value, kth in ((ck, Kt, False, kth_k), (cv, Vt, True, kth_v)):
+        ref = ops.compress(x, is_value, kth=kth, capacity_halfs=x.numel())
+        n = int(ref.total_halfs)
+        assert int(got.total_halfs) == n
+        assert torch.equal(got.bmp, ref.bmp) and torch.equal(got.idx, ref.idx) and torch.equal(got.nz_off, ref.nz_off)
+        assert torch.equal(got.nz[:n].view(torch.int16), ref.nz[:n].view(torch.int16))
