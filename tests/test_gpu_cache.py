@@ -106,6 +106,34 @@ def test_pool_that_overflows_grows_and_ends_up_like_one_that_never_did():
         assert np.array_equal(pool.head_values(b).cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+def test_pair_append_equals_two_appends_and_survives_an_overflow():
+    """cache.append_pair (keys and values of a chunk in one launch, one shared flag word) against one append per side:
+    same bitmaps, offsets and values; with slabs too small for the second chunk - of one side only, and of both - the
+    chunk is taken back, appended side by side and each pool grows its own slabs."""
+    from mustafar_amd.cache import CompressedPool, append_pair
+    dev = torch.device("cuda:0")
+    heads, D = 3, 128
+    K, V = orc.make_kv(19, heads, 256, D)
+    Kt, Vt = torch.from_numpy(K).to(dev), torch.from_numpy(V).to(dev)
+    refs = []
+    for x, is_value in ((Kt, False), (Vt, True)):
+        r = CompressedPool(heads, D, 256, is_value, dev, slab_fraction=1.0)
+        r.append(x[:, :64], 89)
+        r.append(x[:, 64:256], 89)
+        refs.append(r)
+    for fk, fv, grown in ((1.0, 1.0, (0, 0)), (0.2, 1.0, (1, 0)), (0.2, 0.2, (1, 1))):
+        kp = CompressedPool(heads, D, 256, False, dev, slab_fraction=fk)
+        vp = CompressedPool(heads, D, 256, True, dev, slab_fraction=fv)
+        append_pair(kp, vp, Kt[:, :64], Vt[:, :64], 89, 89)
+        append_pair(kp, vp, Kt[:, 64:256], Vt[:, 64:256], 89, 89)
+        assert (kp.generation, vp.generation) == grown and int(kp.overflow) == 0 and int(vp.overflow) == 0
+        for p, r in ((kp, refs[0]), (vp, refs[1])):
+            assert p.tokens == 256 and int(p.tokens_dev) == 256
+            assert torch.equal(p.bmp, r.bmp) and torch.equal(p.idx, r.idx)
+            for b in range(heads):
+                assert torch.equal(p.head_values(b).view(torch.int16), r.head_values(b).view(torch.int16))
+
+
 def test_quantised_pool_that_overflows_grows_and_ends_up_like_one_that_never_did():
     from mustafar_amd.cache import QuantPool
     dev = torch.device("cuda:0")
