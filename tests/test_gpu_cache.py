@@ -526,9 +526,16 @@ def test_two_launch_step_against_the_oracle_on_random_shapes(seed):
                     r = orc.compress_quant(np.ascontiguousarray(x[:, :Lc]), is_value, 2)
                     x[:, :Lc] = np.stack([orc.decode_quant(r[0], r[2], r[1], r[5], r[6], b, Lc, D, is_value, 2, 0)
                                           for b in range(Bkv)])
-        _, _, o_ref = orc.dense_masked_attention(qr, Kp, Vp, g)
+        s_ref, _, o_ref = orc.dense_masked_attention(qr, Kp, Vp, g)
         got = out.reshape(bs * n_q, D).float().cpu().numpy().astype(np.float64)
         scale = max(np.abs(o_ref.astype(np.float64)).max(), 1e-30)
-        assert np.abs(got - o_ref).max() < (1e-2 if quant else 2e-3) * scale, (seed, t)
+        # per row: the stated tolerance plus one fp16 ulp of the row's largest score / sqrt(d) - with the outlier
+        # channels of these keys the scores reach +-100, where two correct summation orders round a score to
+        # neighbouring fp16 values and a token's probability moves by that much (tests/test_gpu_config4.py)
+        smax = np.abs(s_ref.astype(np.float64)).reshape(bs * n_q, -1).max(axis=1)
+        ulp = np.exp2(np.floor(np.log2(np.maximum(smax, 2.0 ** -14))) - 10)
+        tol = (1e-2 if quant else 2e-3) + ulp / np.sqrt(D)
+        err = np.abs(got - o_ref).max(axis=1) / scale
+        assert (err < tol).all() and np.median(err) < (1e-2 if quant else 2e-3), (seed, t, float(err.max()))
         c.advance()
     assert int(c._wovf) == 0
