@@ -288,6 +288,9 @@ __global__ __launch_bounds__(64) void compress_scatter_kernel(const _Float16* __
 // owns the unit of its workgroup index, selects, builds bitmaps and padded counts, publishes the unit's total,
 // compacts the first half of the unit into an LDS image while the units in front of it publish theirs, learns where
 // its values start from a decoupled look-back, and streams the two halves out of the rows it still holds in registers.
+// While the threshold is searched only the first half of the lane's row is in registers - the second half waits in
+// the staging buffer (unit_rows_parked, select_kth_planes_parked) - which keeps the kernel at four wavefronts per
+// SIMD; compress_onepass_kv_kernel runs the keys and the values of the same tokens as one grid over this same body.
 //
 // A workgroup of W wavefronts owns W consecutive units (W divides the units of a head), adds up their totals in LDS
 // and publishes one 64-bit word state[g] = bit 63 | total of workgroup g (4-byte units) with an agent-scope store.
@@ -382,6 +385,7 @@ struct ProjArgs {
     RowsView rot;
     int rows;
 };
+// (0: the whole row in registers during the search - three wavefronts per SIMD; kept for A/B builds)
 #ifndef MSTF_COMPRESS_PARK
 #define MSTF_COMPRESS_PARK 1
 #endif
