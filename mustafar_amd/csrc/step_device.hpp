@@ -101,6 +101,19 @@ __device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, c
     const bool has_new = new_row >= row0 && new_row < row0 + 64;  // wave-uniform
     const bool is_new = row0 + lane == new_row;
 
+    // ---- the first two pieces of the value rows are requested up front: they do not depend on the scores, both
+    // buffers are free, and they land while the keys are multiplied
+    const char* vsrc = reinterpret_cast<const char*>(sa.v_win + ((size_t)kv * sa.win_stride + row0) * D);
+    auto issue_rows = [&](int qd) {
+#pragma unroll
+        for (int i = 0; i < VROWS / 4; i++) {
+            const int row = qd * VROWS + i * 4 + (lane >> 4);
+            if (row < nt) dma16(vsrc + (size_t)row * (D * 2) + (lane & 15) * 16, my + (qd & 1) * kVBuf + i * 1024);
+        }
+    };
+    issue_rows(0);
+    if (VROWS < nt) issue_rows(1);
+
     // ---- key rows into registers
     uint4 kr[16];
     {
@@ -164,23 +177,14 @@ __device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, c
         vnew = *reinterpret_cast<const uint4*>(sa.v_in + b * sa.v_stride + (int64_t)hk * D + (lane & 15) * 8);
         if (lane < 16) *reinterpret_cast<uint4*>(sa.v_win + ((size_t)kv * sa.win_stride + new_row) * D + lane * 8) = vnew;
     }
-    const char* vsrc = reinterpret_cast<const char*>(sa.v_win + ((size_t)kv * sa.win_stride + row0) * D);
-    auto issue_rows = [&](int qd) {
-#pragma unroll
-        for (int i = 0; i < VROWS / 4; i++) {
-            const int row = qd * VROWS + i * 4 + (lane >> 4);
-            if (row < nt) dma16(vsrc + (size_t)row * (D * 2) + (lane & 15) * 16, my + (qd & 1) * kVBuf + i * 1024);
-        }
-    };
     const uint32_t prow = lds_addr(pl) + (uint32_t)j * kPRow;
-    issue_rows(0);
 #pragma unroll
     for (int qd = 0; qd < 64 / VROWS; qd++) {
         if (qd * VROWS >= nt) break;  // wave-uniform
         wait_vm0();
         wait_lgkm0();  // the reads of the other buffer (two pieces back) are done before it is filled again
         __builtin_amdgcn_sched_barrier(0);
-        if (qd + 1 < 64 / VROWS) issue_rows(qd + 1);
+        if (qd >= 1 && qd + 1 < 64 / VROWS) issue_rows(qd + 1);  // (piece 1 is on its way since the start)
         char* buf = my + (qd & 1) * kVBuf;
         // the new row is not in the window buffer yet as far as this wavefront's loads can tell: from registers
         if (has_new && new_row - row0 >= qd * VROWS && new_row - row0 < qd * VROWS + VROWS && lane < 16)
