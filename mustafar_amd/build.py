@@ -11,6 +11,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the leading kernel arguments (up to fourteen 32-bit words) arrive in scalar registers with the wavefront
+    # instead of through a load from the argument segment: the first memory round trip of every kernel less
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function",
 ]
 

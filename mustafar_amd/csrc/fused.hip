@@ -27,27 +27,37 @@ namespace mstf {
 // (max, sum, output) into running ones before the workgroup combine.
 //   write_final (only with one split) : out[(kv*groups + h)*D + d] fp16 final
 //   otherwise   : part_o[((kv*groups + h)*nsplit + split)*D + d], part_ml[..][2] = (max, sum)
-// STEP: the launch is a whole decode step (StepArgs above, the first argument so that it sits at the start of the
-// kernel-argument segment): the query rows come rotated out of the projection output instead of q, and the wavefronts
-// also take the blocks of the dense window.
+// STEP: the launch is a whole decode step (StepArgs above, the last argument; DecodeKernargs mirrors the argument list
+// and tells where it sits in the kernel-argument segment): the query rows come rotated out of the projection output
+// instead of q, and the wavefronts also take the blocks of the dense window.
+struct DecodeKernargs {
+    const void* first_ptrs[4];
+    size_t tstride;
+    const void* tokens_dev;
+    int nblk, bpw;
+    const void* ptrs[8];
+    int groups, nsplit, write_final;
+    float sqrt_d;
+    StepArgs st;
+};
+constexpr size_t kStepArgsAt = offsetof(DecodeKernargs, st);
 template <int NM, bool MULTI, bool STEP = false>
 __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_eu(MSTF_FUSED_OCCUPANCY))) void decode_attention_kernel(
-    StepArgs st, const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint32_t* __restrict__ k_idx,
-    const uint32_t* __restrict__ k_nz_off, const uint64_t* __restrict__ v_bmp, const char* __restrict__ v_nz,
-    const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ v_nz_off, const _Float16* __restrict__ q,
-    _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, size_t tstride, int groups,
-    int nblk, int nsplit, int write_final, float sqrt_d, int bpw, const int* __restrict__ tokens_dev)
+    const uint32_t* __restrict__ k_idx, const uint32_t* __restrict__ v_idx, const uint32_t* __restrict__ k_nz_off,
+    const uint32_t* __restrict__ v_nz_off, size_t tstride, const int* __restrict__ tokens_dev, int nblk, int bpw,
+    const uint64_t* __restrict__ k_bmp, const char* __restrict__ k_nz, const uint64_t* __restrict__ v_bmp,
+    const char* __restrict__ v_nz, const _Float16* __restrict__ q, _Float16* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int groups, int nsplit, int write_final, float sqrt_d,
+    StepArgs st)
 {
+    // Argument order: the first fourteen 32-bit words - what the first load of a wavefront, the stage boundaries,
+    // needs - are in scalar registers when the wavefront starts (kernel-argument preload, a compile option of this
+    // library); the others are fetched from the argument segment while that load is on its way.
     // tstride: tiles between the bitmap rows of two heads (offsets: one more), which is the tile count of the cached
     // tokens unless the cache is pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read
     // from device memory, at most nblk blocks of it; the launch is then sized for the capacity and the wavefronts
     // beyond the valid blocks leave neutral partials, so a recorded launch stays valid while the cache grows.
     constexpr int D = kFusedD;
-    // every argument in registers before anything else: left alone, the compiler fetches them where they are first
-    // used, three dependent round trips in front of the first load of data
-    asm volatile("" ::"s"(k_bmp), "s"(k_nz), "s"(k_idx), "s"(k_nz_off), "s"(v_bmp), "s"(v_nz), "s"(v_idx), "s"(v_nz_off),
-                 "s"(q), "s"(out), "s"(part_o), "s"(part_ml), "s"(tstride), "s"(groups), "s"(nblk), "s"(nsplit),
-                 "s"(write_final), "s"(sqrt_d), "s"(bpw), "s"(tokens_dev));
     if (tokens_dev) {
         const int valid = *tokens_dev / 64;
         nblk = valid < nblk ? valid : nblk;
@@ -124,6 +134,11 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
             return *p;
         };
         uint32_t bnd = boundaries(ixK, ixV);
+        __builtin_amdgcn_sched_barrier(0);  // (the load goes out before anything waits for the other arguments)
+        // every other argument in registers now: left alone, the compiler fetches them where they are first used,
+        // dependent round trips in front of the first load of data
+        asm volatile("" ::"s"(k_bmp), "s"(k_nz), "s"(v_bmp), "s"(v_nz), "s"(q), "s"(out), "s"(part_o), "s"(part_ml),
+                     "s"(groups), "s"(nsplit), "s"(write_final), "s"(sqrt_d));
         uint32_t bnd_next = bnd;  // MULTI: boundaries of the coming block
         const uint32_t lane16 = (uint32_t)lane * 16u;
         const uint32_t off8 = (uint32_t)(lane < kSubTiles ? lane : kSubTiles - 1) * 8u;
@@ -287,8 +302,8 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
         // others).  The query rows are still in LDS; the value buffers and the weight rows are free again.
         // (the step's arguments are fetched again here, through a pointer the compiler cannot see through: kept in
         // scalar registers across the walk above they would push other values out)
-        const StepArgs __attribute__((address_space(4)))* sp =
-            (const StepArgs __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+        const StepArgs __attribute__((address_space(4)))* sp = (const StepArgs __attribute__((address_space(4)))*)(
+            (const char __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr() + kStepArgsAt);
         asm volatile("" : "+s"(sp));
         StepArgs sw;
         sw.q_in = sp->q_in, sw.k_in = sp->k_in, sw.v_in = sp->v_in;
@@ -614,18 +629,18 @@ static int decode_launch(hipStream_t st, const uint64_t* k_bmp, const mstf_half*
     _Float16* oh = reinterpret_cast<_Float16*>(out);
     const float sq = sqrtf((float)head_dim);
 #define MSTF_FD(NMV, MULTIV)                                                                                         \
-    hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx, \
-                       k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,    \
-                       write_final, sq, bpw, tokens_dev)
+    hipLaunchKernelGGL((decode_attention_kernel<NMV, MULTIV>), grid, dim3(kFusedWaves * 64), 0, st, k_idx, v_idx,   \
+                       k_nz_off, v_nz_off, tstride, tokens_dev, nblk, bpw, k_bmp, knz, v_bmp, vnz, qh, oh, part_o,  \
+                       part_ml, groups, nst, write_final, sq, sa)
     if (step) {  // (token count in device memory: the MULTI form)
         if (groups <= 4)
-            hipLaunchKernelGGL((decode_attention_kernel<1, true, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx,
-                               k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
-                               write_final, sq, bpw, tokens_dev);
+            hipLaunchKernelGGL((decode_attention_kernel<1, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_idx,
+                               v_idx, k_nz_off, v_nz_off, tstride, tokens_dev, nblk, bpw, k_bmp, knz, v_bmp, vnz, qh, oh,
+                               part_o, part_ml, groups, nst, write_final, sq, sa);
         else
-            hipLaunchKernelGGL((decode_attention_kernel<2, true, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp, knz, k_idx,
-                               k_nz_off, v_bmp, vnz, v_idx, v_nz_off, qh, oh, part_o, part_ml, tstride, groups, nblk, nst,
-                               write_final, sq, bpw, tokens_dev);
+            hipLaunchKernelGGL((decode_attention_kernel<2, true, true>), grid, dim3(kFusedWaves * 64), 0, st, k_idx,
+                               v_idx, k_nz_off, v_nz_off, tstride, tokens_dev, nblk, bpw, k_bmp, knz, v_bmp, vnz, qh, oh,
+                               part_o, part_ml, groups, nst, write_final, sq, sa);
     } else if (groups <= 4) {
         if (bpw == 1) MSTF_FD(1, false); else MSTF_FD(1, true);
     } else {

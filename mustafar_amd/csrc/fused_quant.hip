@@ -29,16 +29,31 @@ struct QSide {
 };
 
 // grid = (token splits, KV heads), kFusedWaves wavefronts; see decode_attention_kernel.  STEP: the launch is a whole
-// decode step (st, the first argument so that it sits at the start of the kernel-argument segment; step_device.hpp).
+// decode step (st, the last argument; QuantKernargs mirrors the argument list and tells where it sits in the
+// kernel-argument segment; step_device.hpp).
+struct QuantKernargs {
+    const void* first_ptrs[4];
+    size_t tstride;
+    const void* tokens_dev;
+    int nblk, heads_fastest;
+    const void* ptrs[12];
+    int groups, nsplit, write_final;
+    float sqrt_d;
+    int mode;
+    StepArgs st;
+};
+constexpr size_t kQuantStepArgsAt = offsetof(QuantKernargs, st);
 template <int NM, int BIT, bool G32, bool STEP = false>
 __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kernel(
-    StepArgs st, const uint64_t* __restrict__ k_bmp, const uint32_t* k_packed, const uint32_t* __restrict__ k_off,
-    const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros, const uint64_t* __restrict__ v_bmp,
-    const uint32_t* v_packed, const uint32_t* __restrict__ v_off, const uint32_t* v_off_dma, const uint16_t* v_scales,
-    const uint16_t* v_zeros, const _Float16* q, _Float16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, size_t tstride, int groups, int nblk, int nsplit, int write_final, float sqrt_d, int mode,
-    const int* __restrict__ tokens_dev, int heads_fastest)
+    const uint32_t* __restrict__ k_off, const uint32_t* __restrict__ v_off, const uint64_t* __restrict__ k_bmp,
+    const uint64_t* __restrict__ v_bmp, size_t tstride, const int* __restrict__ tokens_dev, int nblk, int heads_fastest,
+    const uint32_t* k_packed, const uint32_t* k_off_dma, const uint16_t* k_scales, const uint16_t* k_zeros,
+    const uint32_t* v_packed, const uint32_t* v_off_dma, const uint16_t* v_scales, const uint16_t* v_zeros,
+    const _Float16* q, _Float16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int groups,
+    int nsplit, int write_final, float sqrt_d, int mode, StepArgs st)
 {
+    // Argument order: the first fourteen 32-bit words - what a wavefront's first loads need - are in scalar registers
+    // when it starts (kernel-argument preload, a compile option of this library).
     // tstride: tiles between the per-tile rows of two heads - the tile count of the cached tokens unless the arrays are
     // pre-allocated for more.  tokens_dev (nullable): the number of cached tokens is read from device memory, at most
     // nblk blocks of it; the launch is then sized for the capacity and the wavefronts beyond the valid blocks leave
@@ -211,8 +226,8 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
         // step's arguments are fetched again here, through a pointer the compiler cannot see through, so that they
         // hold no scalar registers above.
         static_assert(2 * 8 * D * 2 <= kImgBytes, "two buffers of eight value rows in the room of the image");
-        const StepArgs __attribute__((address_space(4)))* sp =
-            (const StepArgs __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr();
+        const StepArgs __attribute__((address_space(4)))* sp = (const StepArgs __attribute__((address_space(4)))*)(
+            (const char __attribute__((address_space(4)))*)__builtin_amdgcn_kernarg_segment_ptr() + kQuantStepArgsAt);
         asm volatile("" : "+s"(sp));
         StepArgs sw;
         sw.q_in = sp->q_in, sw.k_in = sp->k_in, sw.v_in = sp->v_in;
@@ -241,20 +256,20 @@ static void launch_decode_quant(hipStream_t st, dim3 grid, const uint64_t* k_bmp
 {
     const StepArgs sa = step ? *step : StepArgs{};
     if (step)  // (group_size is 64 there: quant_launch has checked it)
-        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false, true>), grid, dim3(kFusedWaves * 64), 0, st, sa,
-                           k_bmp, k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales,
-                           v_zeros, q, out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode,
-                           tokens_dev, heads_fastest);
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false, true>), grid, dim3(kFusedWaves * 64), 0, st, k_off,
+                           v_off, k_bmp, v_bmp, tstride, tokens_dev, tokens / 64, heads_fastest, k_packed, k_off, k_scales,
+                           k_zeros, v_packed, v_off, v_scales, v_zeros, q, out, part_o, part_ml, groups, ns, write_final,
+                           sq, mode, sa);
     else if (group_size == 32)
-        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp,
-                           k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
-                           out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
-                           heads_fastest);
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, true>), grid, dim3(kFusedWaves * 64), 0, st, k_off,
+                           v_off, k_bmp, v_bmp, tstride, tokens_dev, tokens / 64, heads_fastest, k_packed, k_off, k_scales,
+                           k_zeros, v_packed, v_off, v_scales, v_zeros, q, out, part_o, part_ml, groups, ns, write_final,
+                           sq, mode, sa);
     else
-        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, sa, k_bmp,
-                           k_packed, k_off, k_off, k_scales, k_zeros, v_bmp, v_packed, v_off, v_off, v_scales, v_zeros, q,
-                           out, part_o, part_ml, tstride, groups, tokens / 64, ns, write_final, sq, mode, tokens_dev,
-                           heads_fastest);
+        hipLaunchKernelGGL((decode_attention_quant_kernel<NM, BIT, false>), grid, dim3(kFusedWaves * 64), 0, st, k_off,
+                           v_off, k_bmp, v_bmp, tstride, tokens_dev, tokens / 64, heads_fastest, k_packed, k_off, k_scales,
+                           k_zeros, v_packed, v_off, v_scales, v_zeros, q, out, part_o, part_ml, groups, ns, write_final,
+                           sq, mode, sa);
 }
 
 }  // namespace mstf
