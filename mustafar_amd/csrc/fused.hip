@@ -86,6 +86,10 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
     int nb = nblk - tb;                                                // its blocks (wave-uniform)
     if (MULTI) nb = nb > bpw ? bpw : nb;
     const bool active = nb > 0;
+    // STEP: a wavefront that also has a block of the dense window to do keeps the highest issue priority through its
+    // walk (it has the longest way to go; see set_wave_priority)
+    uint32_t prio_boost = 0u;
+    if constexpr (STEP) prio_boost = step_window_boost(st, wave, split);
     const int j = lane & 3;
     const size_t T = tstride;
     char* my = lds[wave];
@@ -223,6 +227,9 @@ __global__ __launch_bounds__(kFusedWaves * 64) __attribute__((amdgpu_waves_per_e
             }
             static_for<kStages>([&](auto nc) {
                 constexpr int n = decltype(nc)::value;
+                // 3, 2, 1, 0 over the key stages and again over the value stages
+                if constexpr (STEP) set_wave_priority_uniform(prio_boost | (uint32_t)(3 - n % 4));
+                else set_wave_priority(3 - n % 4);
                 wait_vm0_keep(touch);  // sub-chunk n has landed (with the query rows for the first one)
                 // The buffer of sub-chunk n-1 is refilled now: every LDS read of that sub-chunk fed an MFMA that was
                 // issued before this point, so the reads have returned.

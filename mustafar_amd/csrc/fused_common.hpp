@@ -160,8 +160,8 @@ __device__ __forceinline__ void workgroup_combine(char* lds_base, int wave_strid
 {
     constexpr int D = kFusedD;
     const int j = lane & 3;
-    __syncthreads();
     {
+        // (the wavefront parks its triple in its own LDS region, which only it has used so far: no barrier in front)
         float* po = reinterpret_cast<float*>(lds_base + wave * wave_stride);
 #pragma unroll
         for (int m = 0; m < NM; m++) {

@@ -188,6 +188,9 @@ __global__ __launch_bounds__(kFusedWaves * 64) void decode_attention_quant_kerne
 
 #pragma unroll
         for (int n = 0; n < kKeySubs + kValSubs; n++) {
+            // 3, 2, 1, 0 over the key stages and again over the value stages (keeping the wavefronts that also take a
+            // block of the dense window at 3, as the fp16 kernel does, measured slower here: one block per wavefront)
+            set_wave_priority(3 - n % 4);
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
             const uint2 bits = touch;  // lane l < 32: bitmap l of stage n
             if (n + 1 < kKeySubs + kValSubs) touch = issue(n + 1);

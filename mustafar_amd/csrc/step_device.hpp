@@ -29,6 +29,16 @@ struct StepArgs {
     int win_len, win_stride, n_kv, ns;
 };
 
+// 3 for a wavefront that step_window_wave gives a block of the dense window (block wave * ns + split of the rows that
+// are valid after this step), else 0: OR-ed into the issue priority of its walk over the compressed tokens.
+__device__ __forceinline__ uint32_t step_window_boost(const StepArgs& sa, int wave, int split)
+{
+    int wlen = sa.win_len_dev ? *sa.win_len_dev : sa.win_len;
+    wlen = wlen < sa.win_len ? wlen : sa.win_len;
+    const int has = wave * sa.ns + split < (wlen + 63) / 64;
+    return (uint32_t)__builtin_amdgcn_readfirstlane(has ? 3 : 0);
+}
+
 // The query rows of KV head kv into LDS (ql: [4*NM][128] fp16), rotated: eight lanes per query head, a lane holds
 // channels c .. c+7 and their partners 64 channels on.
 template <int QROW = kFusedD * 2>
