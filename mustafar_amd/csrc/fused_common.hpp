@@ -22,24 +22,25 @@ constexpr int kValSubs = kFusedD / kSubTiles;       // sub-chunks of the value p
 constexpr int kFusedResident = 1024 * MSTF_FUSED_OCCUPANCY;  // wavefronts of the fused kernel the 256 CUs hold at once
 constexpr int kFusedMaxBpw = 8;
 
+// (The planning helpers below are constexpr, hence usable from device code as well as from the launchers.)
 // Token blocks one wavefront of the fp16 kernel walks: 1 while every block can have a resident wavefront of its
 // own; beyond that the blocks are spread over one chip-filling set of wavefronts, so that only a wavefront's first
 // block waits for memory.
-static inline int fused_blocks_per_wave(int tokens, int Bkv)
+constexpr int fused_blocks_per_wave(int tokens, int Bkv)
 {
     const long long blocks = (long long)Bkv * (tokens / 64);
     const long long r = (blocks + kFusedResident - 1) / kFusedResident;
     return r < 1 ? 1 : (r > kFusedMaxBpw ? kFusedMaxBpw : (int)r);
 }
 // Split slots (= workgroups) per KV head: kFusedWaves * bpw token blocks each.
-static inline int fused_nsplit(int tokens, int bpw = 1)
+constexpr int fused_nsplit(int tokens, int bpw = 1)
 {
     return (tokens / 64 + kFusedWaves * bpw - 1) / (kFusedWaves * bpw);
 }
 
 // Split slots that any token count up to `tokens` can need when the blocks per wavefront follow the count (a launch
 // sized once for a cache that grows): far fewer than one block per wavefront would take once the chip is full.
-static inline int fused_nsplit_capacity(int tokens, int Bkv)
+constexpr int fused_nsplit_capacity(int tokens, int Bkv)
 {
     int ns = 1;
     for (int n = 64; n <= tokens; n += 64) {
@@ -58,7 +59,7 @@ int merge_splits(hipStream_t st, const void* workspace, mstf_half* out, float* l
 int window_launch(hipStream_t st, const mstf_half* k_win, const mstf_half* v_win, const mstf_half* q, void* workspace,
                   int win_len, const int32_t* win_len_dev, int win_stride, int head_dim, int Bq, int groups, int nst,
                   int split0);
-static inline int window_blocks(int win_len) { return (win_len + 63) / 64; }
+constexpr int window_blocks(int win_len) { return (win_len + 63) / 64; }
 
 // Reductions over the sixteen lanes 4b+j (b = 0..15) that hold column j, without LDS round trips: inside a row of
 // sixteen lanes by two rotations (DPP row_ror 4 and 8, folded into the combining instruction), across the four rows by
