@@ -84,9 +84,7 @@ __device__ __forceinline__ void walk_subs_q(int nsubs, TileOf tile_of, StageW st
     uint32_t s_nxt, e_nxt;
     bounds(t_nxt, s_nxt, e_nxt);
     for (int n = 0; n < nsubs; n++) {
-#if MSTF_WALK_PRIO
-        set_wave_priority_uniform(3u - ((uint32_t)n & 3u));
-#endif
+        set_wave_priority_uniform(3u - ((uint32_t)n & 3u));  // falls from stage to stage (see set_wave_priority)
         asm volatile("s_waitcnt vmcnt(0)" : "+v"(touch.x), "+v"(touch.y)::"memory");  // stage n has landed
         const uint2 bits = touch;  // lane l < 32: bitmap l of stage n
         if (n + 1 < nsubs) touch = issue(n + 1, t_nxt, s_nxt, e_nxt);

@@ -123,9 +123,6 @@ struct Batch {
     u32x8_t ov;   // idx of the 8 tiles (4-byte units from the start of the KV head's values)
 };
 
-#ifndef MSTF_WALK_PRIO
-#define MSTF_WALK_PRIO 1
-#endif
 #ifndef MSTF_DUAL_ACC
 #define MSTF_DUAL_ACC 1
 #endif
@@ -436,9 +433,7 @@ __device__ __forceinline__ void walk_subs(int nsubs, TileOf tile_of, StageW stag
 #pragma unroll
     for (int m = 0; m < NM; m++) acc2[m] = f4_t{0.f, 0.f, 0.f, 0.f};
     for (int n = 0; n < nsubs; n++) {
-#if MSTF_WALK_PRIO
-        set_wave_priority_uniform(3u - ((uint32_t)n & 3u));
-#endif
+        set_wave_priority_uniform(3u - ((uint32_t)n & 3u));  // falls from stage to stage (see set_wave_priority)
         wait_vm0_keep(touch);  // sub-chunk n (values, weights) has landed
         // Buffer (n+1)&1 is refilled now.  Its last reader was sub-chunk n-1, and every LDS read of that sub-chunk
         // fed an MFMA issued before this point, so the reads have returned.
