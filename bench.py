@@ -108,6 +108,16 @@ def cpu_baseline(args, bs, nkv, groups, L, D, kth):
 RING_ROUNDS = 4   # passes over the rotating caches captured into one graph
 
 
+def settle(torch, fn, seconds):
+    """Runs fn() untimed for `seconds`: after an idle period (set-up on the host, a graph capture) the GPU needs some
+    tens of milliseconds of load before its clocks are where a decode loop keeps them - launches timed right after
+    such a pause read 5 - 8 % longer than the same launches a moment later."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        fn()
+        torch.cuda.synchronize()
+
+
 def ring_time_us(torch, fn, n_slots, reps):
     """GPU time of one fn(i): RING_ROUNDS passes of fn(0) .. fn(n_slots - 1) are captured back to back into one HIP
     graph (slot i works on rotating cache i, so its reads are cold), the graph is replayed `reps` times between two HIP
@@ -121,7 +131,7 @@ def ring_time_us(torch, fn, n_slots, reps):
         for _ in range(RING_ROUNDS):
             for i in range(n_slots):
                 fn(i)
-    g.replay()
+    settle(torch, g.replay, 0.02)
     return event_time_us(torch, g.replay, max(1, -(-reps // RING_ROUNDS))) / (n_slots * RING_ROUNDS)
 
 
@@ -473,6 +483,9 @@ def main():
                 it[0] += 1
                 k -= 1
 
+    # steady state first (see settle), then the W warm-up steps and the K timed ones
+    settle(torch, lambda: run_steps(args.caches * RING_ROUNDS if ring is not None else 1), 0.1)
+    it[0] = 0
     run_steps(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
