@@ -118,8 +118,8 @@ int mstf_append_value_f16(void* stream, const mstf_half* x, int B, int M, int N,
  * by mstf_compress_value_f16 (both with a value buffer), or mstf_append_key_f16 followed by mstf_append_value_f16,
  * write - the outputs are identical bit for bit - behind one clearing launch, with the workgroups of the two sides in
  * one grid.  A launch with twice the workgroups runs less in lockstep (the loads of the values overlap the arithmetic
- * of the keys): 94 us against 53 + 51 us at 128 heads x 4096 tokens, 179 against 102 + 93 us at 256 heads (52 against
- * 28 + 25 us at 64 heads, where each side is one generation of workgroups).  Both value
+ * of the keys): 86 us against 51 + 50 us at 128 heads x 4096 tokens, 159 against 88 + 85 us at 256 heads (51 against
+ * 27 + 25 us at 64 heads, where each side is one generation of workgroups).  Both value
  * buffers are required (no sizing-only form); the append form shares one sticky flag word between the sides.
  * Workspace: mstf_compress_kv_workspace_bytes(B, M, N), 256-byte aligned. */
 size_t mstf_compress_kv_workspace_bytes(int B, int M, int N);
