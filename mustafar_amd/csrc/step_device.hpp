@@ -123,6 +123,15 @@ __device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, c
     };
     issue_rows(0);
     if (VROWS < nt) issue_rows(1);
+    // the rows of the later pieces are pulled into the L2 cache meanwhile (one 4-byte load per 128-byte line, result
+    // unused): their LDS-direct loads, which have to wait for a free buffer, then find them there
+    uint32_t warm = 0u, warm2 = 0u;
+    {
+        const int wrow = 2 * VROWS + lane / 2;
+        if (wrow < nt) warm = *reinterpret_cast<const uint32_t*>(vsrc + (size_t)(2 * VROWS) * (D * 2) + (size_t)lane * 128);
+        if (2 * VROWS + 32 < 64 && wrow + 32 < (nt < 64 ? nt : 64))  // (eight rows per piece: rows 48 .. 63 as well)
+            warm2 = *reinterpret_cast<const uint32_t*>(vsrc + (size_t)(2 * VROWS + 32) * (D * 2) + (size_t)lane * 128);
+    }
 
     // ---- key rows into registers
     uint4 kr[16];
@@ -221,6 +230,7 @@ __device__ __forceinline__ void step_window_wave(char* my, char* ql, char* pl, c
         }
     }
     wait_vm0();
+    asm volatile("" ::"v"(warm), "v"(warm2));  // (kept until here: a load must not land in a register given to something else)
     // lane 4b+j holds channels 4b..4b+3 of both halves for head 4m+j
 #pragma unroll
     for (int m = 0; m < NM; m++) {
